@@ -1,0 +1,92 @@
+"""Seeded synthetic inputs for the five benchmark cases of the biased-attention path.
+
+Shapes follow the shapes the reference's harness runs (examples/dot_product_attention.py:47-85:
+`(L,4,L,32)` triangle attention, `(1,16,L,24|48)` diffusion attention); values are drawn in
+fp32 from one torch CPU generator in the order q, k, v, bias and then cast, so a case is
+reproducible from its name and seed alone.  Masks: truthy = attend.
+"""
+from dataclasses import dataclass
+
+import torch
+
+
+@dataclass(frozen=True)
+class Case:
+    name: str
+    B: int
+    H: int
+    L: int
+    D: int
+    io_dtype: str          # "fp32" | "bf16"
+    mma_dtype: str         # "fp32" | "bf16" | "fp8"
+    mask_kind: str         # "tail:<n>" (last n keys dropped), "tail1:<n>" (only in the last batch row), "bernoulli:<keep>"
+    mask_rank: int         # 1 -> [L], 2 -> [B,L]
+    tol: float             # max-abs tolerance against the fp32 formula
+    seed: int = 0
+
+    @property
+    def flops(self) -> float:
+        return 4.0 * self.B * self.H * self.L * self.L * self.D
+
+    @property
+    def bytes(self) -> float:
+        io = 4 if self.io_dtype == "fp32" else 2
+        bias = 4 if self.io_dtype == "fp32" else 2
+        return 4.0 * self.B * self.H * self.L * self.D * io + self.H * self.L * self.L * bias + self.B * self.L
+
+
+CASES = {
+    # CPU-runnable plumbing case
+    "cfg1": Case("cfg1", 2, 4, 128, 32, "fp32", "fp32", "tail1:16", 2, 1e-4),
+    # AF3 triangle attention, N=384
+    "cfg2": Case("cfg2", 384, 4, 384, 32, "bf16", "bf16", "tail:38", 2, 2e-2),
+    # pairformer single attention with pair bias, N=768, 16 heads x 24
+    "cfg3": Case("cfg3", 1, 16, 768, 24, "bf16", "bf16", "tail:38", 1, 2e-2),
+    # large-crop triangle attention, N=768 (headline)
+    "cfg4": Case("cfg4", 768, 4, 768, 32, "bf16", "bf16", "bernoulli:0.92", 2, 2e-2),
+    # diffusion transformer token attention, fp8 MMA with bf16 I/O
+    "cfg5": Case("cfg5", 5, 16, 1536, 24, "bf16", "fp8", "tail:154", 1, 6e-2),
+}
+
+
+def make_mask(case: Case, gen: torch.Generator) -> torch.Tensor:
+    kind, _, arg = case.mask_kind.partition(":")
+    B, L = case.B, case.L
+    if kind == "tail":
+        m = torch.ones(L, dtype=torch.bool)
+        m[L - int(arg):] = False
+        return m if case.mask_rank == 1 else m[None, :].expand(B, L).contiguous()
+    if kind == "tail1":
+        m = torch.ones(B, L, dtype=torch.bool)
+        m[B - 1, L - int(arg):] = False
+        return m
+    if kind == "bernoulli":
+        m = torch.rand(B, L, generator=gen) < float(arg)
+        m[:, 0] |= ~m.any(dim=1)  # at least one live key per row
+        return m
+    raise ValueError(case.mask_kind)
+
+
+def make_inputs(case, device="cpu", batch=None):
+    """Returns q, k, v, mask, bias.  `batch` truncates the batch axis (a bounded sample of the
+    same workload: the bias and per-row work are unchanged)."""
+    if isinstance(case, str):
+        case = CASES[case]
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(case.seed)
+    B = case.B if batch is None else min(batch, case.B)
+    dt = torch.float32 if case.io_dtype == "fp32" else torch.bfloat16
+    shape = (B, case.H, case.L, case.D)
+
+    def draw(s):
+        return torch.randn(s, generator=gen, dtype=torch.float32)
+
+    q, k, v = draw(shape), draw(shape), draw(shape)
+    bias = draw((case.H, case.L, case.L))
+    mgen = torch.Generator(device="cpu")
+    mgen.manual_seed(case.seed + 1)
+    mask = make_mask(case, mgen)
+    if mask.dim() == 2:
+        mask = mask[:B]
+    q, k, v, bias = [t.to(dt).to(device) for t in (q, k, v, bias)]
+    return q, k, v, mask.to(device), bias

@@ -1,0 +1,148 @@
+"""ctypes loader for the CPU oracle (oracle/af3_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: import this from tests/, from the smoke check and from the
+CPU-baseline leg of the benchmark, never from the shipped package.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "_build", "libaf3_oracle.so")
+
+F32, BF16 = 0, 1
+
+
+def build(force: bool = False) -> str:
+    src = os.path.join(_HERE, "af3_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.run(["make", "-C", _HERE] + (["-B"] if force else []), check=True, capture_output=True)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = ctypes.CDLL(_SO)
+        fp = ctypes.POINTER(ctypes.c_float)
+        u8 = ctypes.POINTER(ctypes.c_uint8)
+        u16 = ctypes.POINTER(ctypes.c_uint16)
+        i64 = ctypes.c_int64
+        L.af3o_dpa_reference.argtypes = [fp, fp, fp, fp, u8, fp, i64, i64, i64, i64, ctypes.c_int, ctypes.c_int, i64, i64]
+        L.af3o_dpa_reference.restype = ctypes.c_int
+        L.af3o_dpa_formula.argtypes = [fp, fp, fp, fp, u8, fp, i64, i64, i64, i64]
+        L.af3o_dpa_formula.restype = ctypes.c_int
+        L.af3o_convert_f32_to_bf16.argtypes = [fp, u16, i64]
+        L.af3o_convert_bf16_to_f32.argtypes = [u16, fp, i64]
+        L.af3o_quantize_e4m3.argtypes = [fp, u8, i64]
+        L.af3o_quantize_e4m3.restype = ctypes.c_float
+        L.af3o_dequantize_e4m3.argtypes = [u8, fp, i64, ctypes.c_float]
+        L.af3o_f32_to_e4m3_bits.argtypes = [ctypes.c_float]
+        L.af3o_f32_to_e4m3_bits.restype = ctypes.c_uint8
+        L.af3o_e4m3_bits_to_f32.argtypes = [ctypes.c_uint8]
+        L.af3o_e4m3_bits_to_f32.restype = ctypes.c_float
+        L.af3o_vnni_repack.argtypes = [u16, u16, i64, i64, i64]
+        L.af3o_vnni_repack.restype = ctypes.c_int
+        L.af3o_pad_2d.argtypes = [fp, fp, i64, i64, i64, i64, ctypes.c_float]
+        L.af3o_softmax_fwd.argtypes = [fp, fp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        L.af3o_brgemm.argtypes = [fp, fp, fp] + [ctypes.c_int] * 8
+        _lib = L
+    return _lib
+
+
+def _f(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a, a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+
+
+def _keep(mask, B, L):
+    """Lift a user mask (1-D [L] or 2-D [B,L], truthy = attend) to contiguous [B,L] bytes,
+    broadcasting a 1-D mask over the batch like examples/dot_product_attention.py:33-37."""
+    m = np.asarray(mask).astype(bool)
+    if m.ndim == 1:
+        m = np.broadcast_to(m[None, :], (B, L))
+    m = np.ascontiguousarray(m.reshape(B, L).astype(np.uint8))
+    return m, m.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8))
+
+
+def dpa_reference(q, k, v, mask, bias, dtype=F32, use_flash=False, BLK_SZ=128, FLASH_SZ=1024):
+    """Restatement of dot_product_attention_impl<T> (dot_product_attention.cpp:25-198).
+    Inputs are float32 numpy arrays whose values are already representable in T."""
+    B, H, L, D = q.shape
+    q, qp = _f(q); k, kp = _f(k); v, vp = _f(v); bias, bp = _f(bias)
+    m, mp = _keep(mask, B, L)
+    out = np.empty((B, H, L, D), np.float32)
+    rc = lib().af3o_dpa_reference(qp, kp, vp, bp, mp, out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                                  B, H, L, D, dtype, int(bool(use_flash)), BLK_SZ, FLASH_SZ)
+    if rc != 0:
+        raise MemoryError("af3o_dpa_reference failed")
+    return out
+
+
+def dpa_formula(q, k, v, mask, bias):
+    """examples/dot_product_attention.py:20-43 evaluated in double precision."""
+    B, H, L, D = q.shape
+    q, qp = _f(q); k, kp = _f(k); v, vp = _f(v); bias, bp = _f(bias)
+    m, mp = _keep(mask, B, L)
+    out = np.empty((B, H, L, D), np.float32)
+    rc = lib().af3o_dpa_formula(qp, kp, vp, bp, mp, out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), B, H, L, D)
+    if rc != 0:
+        raise MemoryError("af3o_dpa_formula failed")
+    return out
+
+
+def f32_to_bf16_bits(x):
+    x, xp = _f(x)
+    out = np.empty(x.shape, np.uint16)
+    lib().af3o_convert_f32_to_bf16(xp, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint16)), x.size)
+    return out
+
+
+def bf16_bits_to_f32(h):
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib().af3o_convert_bf16_to_f32(h.ctypes.data_as(ctypes.POINTER(ctypes.c_uint16)), out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), h.size)
+    return out
+
+
+def round_bf16(x):
+    return bf16_bits_to_f32(f32_to_bf16_bits(x))
+
+
+def quantize_e4m3(x):
+    """Returns (bits uint8, scale) with scale = 448/amax."""
+    x, xp = _f(x)
+    out = np.empty(x.shape, np.uint8)
+    scale = lib().af3o_quantize_e4m3(xp, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), x.size)
+    return out, float(scale)
+
+
+def dequantize_e4m3(bits, inv_scale=1.0):
+    bits = np.ascontiguousarray(bits, dtype=np.uint8)
+    out = np.empty(bits.shape, np.float32)
+    lib().af3o_dequantize_e4m3(bits.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), bits.size, inv_scale)
+    return out
+
+
+def vnni_repack(bits, blk=0):
+    bits = np.ascontiguousarray(bits, dtype=np.uint16)
+    M, N = bits.shape
+    out = np.empty((M, N), np.uint16)
+    rc = lib().af3o_vnni_repack(bits.ctypes.data_as(ctypes.POINTER(ctypes.c_uint16)), out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint16)), M, N, blk)
+    if rc != 0:
+        raise ValueError("N must be divisible by BLK_SZ and M even")
+    return out
+
+
+def pad_2d(x, prows, pcols, init=0.0):
+    x, xp = _f(x)
+    out = np.empty((prows, pcols), np.float32)
+    lib().af3o_pad_2d(xp, out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), x.shape[0], x.shape[1], prows, pcols, init)
+    return out

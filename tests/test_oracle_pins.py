@@ -1,0 +1,223 @@
+"""Pins for the CPU oracle (oracle/af3_oracle.c) -- everything here runs without a GPU.
+
+The reference ships no tests, fixtures or golden vectors for this path, and its compiled code
+cannot be built (libxsmm is absent), so the oracle is pinned by what the mathematics fixes:
+a library routine (torch SDPA), an independent float64 closed form, a scalar brute force,
+invariants of softmax attention, and torch's own dtype casts.  Each check is chosen so that a
+plausible slip (dropped scale, wrong mask polarity, transposed K, bias indexed by batch,
+un-normalised softmax, flash recurrence error) fails at least one of them.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dpa_numpy
+
+
+def rand_case(rng, B, H, L, D, mask_p=0.8, mask_rank=2):
+    q, k, v = [rng.standard_normal((B, H, L, D)).astype(np.float32) for _ in range(3)]
+    bias = rng.standard_normal((H, L, L)).astype(np.float32)
+    shape = (L,) if mask_rank == 1 else (B, L)
+    mask = rng.random(shape) < mask_p
+    mask[..., 0] = True
+    return q, k, v, mask, bias
+
+
+def test_formula_matches_brute_force_tiny(oracle):
+    rng = np.random.default_rng(1)
+    for (B, H, L, D) in [(1, 1, 5, 3), (2, 2, 8, 4), (1, 3, 7, 2)]:
+        q, k, v, mask, bias = rand_case(rng, B, H, L, D, 0.6)
+        want = dpa_numpy.dpa_brute_force(q, k, v, mask, bias)
+        assert np.abs(oracle.dpa_formula(q, k, v, mask, bias) - want).max() < 1e-6
+        assert np.abs(dpa_numpy.dpa_closed_form(q, k, v, mask, bias) - want).max() < 1e-12
+        assert np.abs(oracle.dpa_reference(q, k, v, mask, bias, BLK_SZ=4) - want).max() < 1e-5
+
+
+@pytest.mark.parametrize("B,H,L,D,rank", [(2, 4, 128, 32, 2), (3, 2, 37, 24, 2), (1, 16, 100, 48, 1), (4, 1, 65, 16, 1)])
+def test_formula_matches_numpy_closed_form(oracle, B, H, L, D, rank):
+    rng = np.random.default_rng(2)
+    q, k, v, mask, bias = rand_case(rng, B, H, L, D, 0.85, rank)
+    want = dpa_numpy.dpa_closed_form(q, k, v, mask, bias)
+    assert np.abs(oracle.dpa_formula(q, k, v, mask, bias) - want).max() < 1e-6
+
+
+def test_reduces_to_torch_sdpa_without_bias_and_mask(oracle):
+    rng = np.random.default_rng(3)
+    B, H, L, D = 2, 3, 96, 32
+    q, k, v, _, _ = rand_case(rng, B, H, L, D)
+    bias = np.zeros((H, L, L), np.float32)
+    mask = np.ones((B, L), bool)
+    want = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(q).double(), torch.from_numpy(k).double(), torch.from_numpy(v).double()).numpy()
+    assert np.abs(oracle.dpa_formula(q, k, v, mask, bias) - want).max() < 1e-6
+    assert np.abs(oracle.dpa_reference(q, k, v, mask, bias, BLK_SZ=32) - want).max() < 2e-6
+
+
+def test_torch_sdpa_with_additive_mask(oracle):
+    # SDPA's float attn_mask is exactly "bias + (-inf on dropped keys)".
+    rng = np.random.default_rng(4)
+    B, H, L, D = 2, 4, 64, 16
+    q, k, v, mask, bias = rand_case(rng, B, H, L, D, 0.7)
+    add = torch.from_numpy(bias).double()[None].repeat(B, 1, 1, 1)
+    add = add.masked_fill(~torch.from_numpy(mask)[:, None, None, :], float("-inf"))
+    want = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(q).double(), torch.from_numpy(k).double(), torch.from_numpy(v).double(), attn_mask=add).numpy()
+    assert np.abs(oracle.dpa_formula(q, k, v, mask, bias) - want).max() < 1e-6
+
+
+@pytest.mark.parametrize("L,BLK,FLASH", [(128, 32, 64), (100, 32, 64), (37, 16, 16), (200, 64, 128)])
+def test_reference_restatement_fp32_flash_equals_nonflash_equals_formula(oracle, L, BLK, FLASH):
+    rng = np.random.default_rng(5)
+    q, k, v, mask, bias = rand_case(rng, 2, 2, L, 24, 0.8)
+    want = oracle.dpa_formula(q, k, v, mask, bias)
+    a = oracle.dpa_reference(q, k, v, mask, bias, use_flash=False, BLK_SZ=BLK, FLASH_SZ=FLASH)
+    b = oracle.dpa_reference(q, k, v, mask, bias, use_flash=True, BLK_SZ=BLK, FLASH_SZ=FLASH)
+    assert np.abs(a - want).max() < 1e-5
+    assert np.abs(b - want).max() < 1e-5
+    assert np.abs(a - b).max() < 1e-5
+
+
+def test_reference_restatement_bf16_within_tolerance(oracle):
+    rng = np.random.default_rng(6)
+    q, k, v, mask, bias = [oracle.round_bf16(t) if t.dtype == np.float32 else t for t in rand_case(rng, 2, 4, 256, 32, 0.9)]
+    want = oracle.dpa_formula(q, k, v, mask, bias)
+    for flash in (False, True):
+        got = oracle.dpa_reference(q, k, v, mask, bias, dtype=oracle.BF16, use_flash=flash, BLK_SZ=64, FLASH_SZ=128)
+        # The reference stores the logits as bf16 (dot_product_attention.cpp:94-110), so its own bf16 result sits
+        # ~2e-2 from the fp32 formula on N(0,1) data; a kernel that keeps logits in fp32 is closer than this.
+        assert np.abs(got - want).max() < 5e-2
+        assert np.abs(got - want).mean() < 3e-3
+        assert np.array_equal(got, oracle.round_bf16(got))  # stored as bf16
+
+
+# ---- invariants of the formula: each would expose a class of indexing / sign mistakes ----
+
+def test_invariants(oracle):
+    rng = np.random.default_rng(7)
+    B, H, L, D = 2, 3, 40, 16
+    q, k, v, mask, bias = rand_case(rng, B, H, L, D, 0.7)
+    base = oracle.dpa_formula(q, k, v, mask, bias)
+    # rows of the weights sum to 1: with v == 1 the output is 1
+    ones = oracle.dpa_formula(q, k, np.ones_like(v), mask, bias)
+    assert np.abs(ones - 1).max() < 1e-6
+    # convex combination of live V rows
+    for b in range(B):
+        live = v[b][:, mask[b], :]
+        assert (base[b] <= live.max(1, keepdims=True) + 1e-5).all() and (base[b] >= live.min(1, keepdims=True) - 1e-5).all()
+    # adding a per-(head,query) constant to the bias changes nothing
+    shift = rng.standard_normal((H, L, 1)).astype(np.float32) * 3
+    assert np.abs(oracle.dpa_formula(q, k, v, mask, bias + shift) - base).max() < 1e-5
+    # permuting keys together with bias columns and mask leaves the output unchanged
+    p = rng.permutation(L)
+    perm = oracle.dpa_formula(q, k[:, :, p], v[:, :, p], mask[:, p], bias[:, :, p])
+    assert np.abs(perm - base).max() < 1e-5
+    # values of K and bias at dropped keys never matter
+    k2, bias2 = k.copy(), bias.copy()
+    for b in range(B):
+        k2[b][:, ~mask[b], :] = 1e4
+    bias2[:, :, ~(mask.all(0))] += 0  # bias is shared over the batch: only perturb where every row drops it
+    dropped_everywhere = ~mask.any(0)
+    bias2[:, :, dropped_everywhere] = 77.0
+    assert np.abs(oracle.dpa_formula(q, k2, v, mask, bias2) - base).max() < 1e-5
+    # the bias is indexed [head, query, key] and broadcast over the batch
+    assert np.abs(oracle.dpa_formula(q[1:], k[1:], v[1:], mask[1:], bias) - base[1:]).max() < 1e-6
+
+
+def test_single_live_key_returns_that_value_row(oracle):
+    rng = np.random.default_rng(8)
+    B, H, L, D = 2, 2, 33, 8
+    q, k, v, mask, bias = rand_case(rng, B, H, L, D)
+    mask[:] = False
+    mask[0, 5] = True
+    mask[1, 32] = True
+    for fn in (oracle.dpa_formula, lambda *a: oracle.dpa_reference(*a, BLK_SZ=16)):
+        out = fn(q, k, v, mask, bias)
+        assert np.abs(out[0] - v[0][:, 5:6, :]).max() < 1e-6
+        assert np.abs(out[1] - v[1][:, 32:33, :]).max() < 1e-6
+
+
+def test_fully_masked_row_is_the_mean_of_v(oracle):
+    # examples/dot_product_attention.py:37: masked_fill(-1e9) on every key -> uniform weights.
+    rng = np.random.default_rng(9)
+    B, H, L, D = 2, 2, 48, 8
+    q, k, v, mask, bias = rand_case(rng, B, H, L, D)
+    mask[1, :] = False
+    out = oracle.dpa_formula(q, k, v, mask, bias)
+    assert np.isfinite(out).all()
+    assert np.abs(out[1] - v[1].mean(1, keepdims=True)).max() < 1e-6
+    # the compiled reference agrees when L is a multiple of the block (padded keys otherwise dilute the mean,
+    # dot_product_attention.cpp:54 pads the mask with 1.0 and tools.cpp pads V with zeros)
+    ref = oracle.dpa_reference(q, k, v, mask, bias, BLK_SZ=16)
+    assert np.abs(ref[1] - v[1].mean(1, keepdims=True)).max() < 1e-5
+
+
+def test_one_d_mask_broadcasts_over_batch(oracle):
+    rng = np.random.default_rng(10)
+    q, k, v, mask, bias = rand_case(rng, 3, 2, 24, 8, 0.7, mask_rank=1)
+    a = oracle.dpa_formula(q, k, v, mask, bias)
+    b = oracle.dpa_formula(q, k, v, np.broadcast_to(mask, (3, 24)).copy(), bias)
+    assert np.array_equal(a, b)
+
+
+# ---- converters ---------------------------------------------------------------------------
+
+def test_bf16_round_trip_matches_torch(oracle):
+    rng = np.random.default_rng(11)
+    x = np.concatenate([rng.standard_normal(20000).astype(np.float32) * 10,
+                        np.array([0.0, -0.0, 1.0, 1.00390625, 1.0 + 2 ** -8, 1.0 + 3 * 2 ** -8, 3.3895e38, 1e-40, np.inf, -np.inf], np.float32)])
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = oracle.f32_to_bf16_bits(x)
+    assert np.array_equal(got, want)
+    back = torch.from_numpy(want.view(np.int16)).view(torch.bfloat16).float().numpy()
+    assert np.array_equal(oracle.bf16_bits_to_f32(got), back)
+    assert np.isnan(oracle.round_bf16(np.array([np.nan], np.float32))[0])
+
+
+def test_e4m3_matches_torch_for_every_code_and_random_values(oracle):
+    codes = np.arange(256, dtype=np.uint8)
+    want = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    got = oracle.dequantize_e4m3(codes)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(got[~np.isnan(got)], want[~np.isnan(want)])
+    rng = np.random.default_rng(12)
+    x = np.concatenate([rng.standard_normal(50000).astype(np.float32) * 100, rng.standard_normal(50000).astype(np.float32) * 0.01,
+                        np.linspace(-448, 448, 7001, dtype=np.float32), np.array([0.0, -0.0, 2 ** -10, 2 ** -9, 1.5 * 2 ** -9, 0.0146484375], np.float32)])
+    x = np.clip(x, -448, 448)
+    want = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    lib = oracle.lib()
+    got = np.array([lib.af3o_f32_to_e4m3_bits(float(t)) for t in x], np.uint8)
+    assert np.array_equal(got, want)
+    assert lib.af3o_f32_to_e4m3_bits(1e6) == 0x7E and lib.af3o_f32_to_e4m3_bits(-1e6) == 0xFE  # saturating
+
+
+def test_quantize_e4m3_uses_per_tensor_amax_scale(oracle):
+    rng = np.random.default_rng(13)
+    x = rng.standard_normal(4096).astype(np.float32) * 3
+    bits, scale = oracle.quantize_e4m3(x)
+    assert scale == pytest.approx(448.0 / np.abs(x).max(), rel=1e-6)
+    want = torch.from_numpy(x * np.float32(scale)).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(bits, want)
+    back = oracle.dequantize_e4m3(bits, 1.0 / scale)
+    assert np.abs(back - x).max() <= np.abs(x).max() / 16 + 1e-6  # 3 mantissa bits: half an ulp at the top binade
+
+
+def test_vnni_repack_is_a_view_permute_per_panel(oracle):
+    rng = np.random.default_rng(14)
+    M, N, blk = 16, 24, 8
+    w = rng.integers(0, 65535, (M, N)).astype(np.uint16)
+    got = oracle.vnni_repack(w, blk)
+    t = torch.from_numpy(w.astype(np.int32))
+    panels = [t[:, p:p + blk].reshape(M // 2, 2, blk).permute(0, 2, 1).reshape(-1) for p in range(0, N, blk)]
+    want = torch.cat(panels).numpy().astype(np.uint16).reshape(M, N)
+    assert np.array_equal(got, want)
+    assert np.array_equal(oracle.vnni_repack(w, 0), torch.from_numpy(w.astype(np.int32)).reshape(M // 2, 2, N).permute(0, 2, 1).reshape(M, N).numpy().astype(np.uint16))
+    with pytest.raises(ValueError):
+        oracle.vnni_repack(w, 7)
+
+
+def test_pad_2d(oracle):
+    x = np.arange(6, dtype=np.float32).reshape(2, 3)
+    got = oracle.pad_2d(x, 4, 5, 1.0)
+    want = np.ones((4, 5), np.float32)
+    want[:2, :3] = x
+    assert np.array_equal(got, want)

@@ -1,0 +1,29 @@
+"""MI355X-native drop-in for the attention hot path of af3_kernels.
+
+Public names, argument order and defaults follow the reference's Python module
+(src/af3_kernels/__init__.py:31-52, :108-135): `dot_product_attention_cpp`,
+`pad_and_align_tensor`, `vnni_repack_tensor`, `reset_debug_timers`, `print_debug_timers`,
+`print_debug_thread_imbalance`.  Behind them a torch custom op hands raw device pointers to
+libaf3_dpa.so (hand-written HIP for gfx950) through the C ABI of include/af3_dpa.h.
+
+Inputs must live on a ROCm device; there is no CPU path and no PyTorch fallback.
+"""
+from . import _lib
+from .ops import (  # noqa: F401
+    convert,
+    dot_product_attention_cpp,
+    dot_product_attention_fp8,
+    pad_and_align_tensor,
+    print_debug_thread_imbalance,
+    print_debug_timers,
+    quantize_fp8_e4m3,
+    reset_debug_timers,
+    selected_kernel,
+    vnni_repack_tensor,
+)
+
+__all__ = [
+    "dot_product_attention_cpp", "dot_product_attention_fp8", "pad_and_align_tensor", "vnni_repack_tensor",
+    "reset_debug_timers", "print_debug_timers", "print_debug_thread_imbalance", "convert", "quantize_fp8_e4m3",
+    "selected_kernel",
+]

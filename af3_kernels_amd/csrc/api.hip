@@ -1,0 +1,87 @@
+// C-ABI entry points for the attention forward pass: validation and kernel selection.
+// Declared in include/af3_dpa.h.  Nothing here allocates, synchronises or exits.
+#include "common.hpp"
+
+using namespace af3;
+
+namespace {
+
+int validate(const af3_dpa_params* p) {
+	if(!p) return AF3_ERR_NULL_POINTER;
+	if(p->B <= 0 || p->H <= 0 || p->L <= 0 || p->D <= 0) return AF3_ERR_BAD_SHAPE;
+	if(p->D > AF3_DPA_MAX_HEAD_DIM) return AF3_ERR_UNSUPPORTED_D;
+	if(p->L > 0x3fffffff || p->B > 0x3fffffff || p->H > 0xffff) return AF3_ERR_BAD_SHAPE;
+	if(!p->q || !p->k || !p->v || !p->out) return AF3_ERR_NULL_POINTER;
+	for(int i = 0; i < 3; i++)
+		if(p->q_stride[i] < 0 || p->k_stride[i] < 0 || p->v_stride[i] < 0 || p->out_stride[i] < 0) return AF3_ERR_BAD_STRIDE;
+	// rows must not overlap: the innermost axis has stride 1 and D (or L for transposed fp8 V) elements
+	if(p->q_stride[2] < p->D || p->k_stride[2] < p->D || p->out_stride[2] < p->D) return AF3_ERR_BAD_STRIDE;
+	if(p->io_dtype == AF3_FP8_E4M3) {
+		if(p->v_stride[2] < p->L) return AF3_ERR_BAD_STRIDE;
+	} else if(p->v_stride[2] < p->D) {
+		return AF3_ERR_BAD_STRIDE;
+	}
+	if(p->bias && (p->bias_stride[0] < 0 || p->bias_stride[1] < p->L)) return AF3_ERR_BAD_STRIDE;
+	if(p->key_mask && p->key_mask_stride_b != 0 && p->key_mask_stride_b < p->L) return AF3_ERR_BAD_STRIDE;
+	if(p->out_dtype != AF3_F32 && p->out_dtype != AF3_BF16) return AF3_ERR_BAD_DTYPE;
+	if(p->bias && p->bias_dtype != AF3_F32 && p->bias_dtype != AF3_BF16) return AF3_ERR_BAD_DTYPE;
+	if(!(p->softmax_scale > 0.f) || !(p->softmax_scale < INFINITY)) return AF3_ERR_BAD_ARGUMENT;
+	switch(p->io_dtype) {
+		case AF3_F32:
+			if(p->mma_dtype != AF3_F32) return AF3_ERR_BAD_DTYPE;
+			break;
+		case AF3_BF16:
+			if(p->mma_dtype != AF3_BF16 && p->mma_dtype != AF3_F32) return AF3_ERR_BAD_DTYPE;
+			break;
+		case AF3_FP8_E4M3:
+			if(p->mma_dtype != AF3_FP8_E4M3) return AF3_ERR_BAD_DTYPE;
+			break;
+		default:
+			return AF3_ERR_BAD_DTYPE;
+	}
+	return AF3_OK;
+}
+
+// 0 generic, 1 bf16 MFMA, 2 fp8 MFMA, or a negative status
+int select_kernel(const af3_dpa_params& p) {
+	if(p.io_dtype == AF3_FP8_E4M3) return mfma_fp8_eligible(p) ? 2 : AF3_ERR_BAD_ARGUMENT;
+	if(p.force_generic || p.mma_dtype == AF3_F32) return 0;
+	return mfma_bf16_eligible(p) ? 1 : 0;
+}
+
+}  // namespace
+
+extern "C" int af3_dpa_select_kernel(const af3_dpa_params* params) {
+	const int rc = validate(params);
+	if(rc != AF3_OK) return rc;
+	return select_kernel(*params);
+}
+
+extern "C" int af3_dpa_forward(const af3_dpa_params* params, void* hip_stream) {
+	const int rc = validate(params);
+	if(rc != AF3_OK) return rc;
+	hipStream_t s = static_cast<hipStream_t>(hip_stream);
+	switch(select_kernel(*params)) {
+		case 0: return launch_dpa_generic(*params, s);
+		case 1: return launch_dpa_mfma_bf16(*params, s);
+		case 2: return launch_dpa_mfma_fp8(*params, s);
+		default: return AF3_ERR_BAD_ARGUMENT;
+	}
+}
+
+extern "C" const char* af3_status_string(int status) {
+	switch(status) {
+		case AF3_OK: return "ok";
+		case AF3_ERR_NULL_POINTER: return "a required pointer is NULL";
+		case AF3_ERR_BAD_DTYPE: return "dtype combination not implemented";
+		case AF3_ERR_BAD_SHAPE: return "a dimension is not positive or exceeds the supported maximum";
+		case AF3_ERR_BAD_STRIDE: return "negative stride, overlapping rows, or innermost stride != 1";
+		case AF3_ERR_UNSUPPORTED_D: return "head_dim exceeds the supported maximum (128)";
+		case AF3_ERR_LAUNCH: return "kernel launch failed";
+		case AF3_ERR_BAD_ARGUMENT: return "invalid argument";
+		case AF3_ERR_NO_DEVICE_CODE: return "this library only carries gfx950 code";
+		default: return "unknown status";
+	}
+}
+
+extern "C" int af3_abi_version(void) { return 1; }

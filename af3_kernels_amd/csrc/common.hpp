@@ -1,0 +1,49 @@
+// Shared declarations for the gfx950 attention library (internal; the public ABI is include/af3_dpa.h).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/af3_dpa.h"
+
+namespace af3 {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+
+// Additive key-mask values, exact in bf16 and powers of two so that multiplying them by any fp32
+// constant is exact.  A dropped key adds MASK_DROPPED to its logit; a key beyond L adds
+// MASK_OUT_OF_RANGE.  |logit| << 2^76, so logit + MASK_DROPPED == MASK_DROPPED in fp32: a row
+// whose keys are all dropped sees equal logits on its L real keys and weight 0 on the padding,
+// i.e. the mean of V, which is what masked_fill(-1e9) + softmax gives in the reference harness.
+constexpr float    MASK_DROPPED            = -0x1p100f;
+constexpr float    MASK_OUT_OF_RANGE       = -0x1p120f;
+constexpr uint16_t MASK_DROPPED_BF16       = 0xF180;
+constexpr uint16_t MASK_OUT_OF_RANGE_BF16  = 0xFB80;
+constexpr float    LOG2E                   = 1.4426950408889634f;
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// fp32 -> bf16 bits, round-to-nearest-even (NaN stays NaN).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+	uint32_t u = __float_as_uint(f);
+	if((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+	return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+	typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+	bf16x2 p = {(__bf16)lo, (__bf16)hi};  // v_cvt_pk_bf16_f32
+	return __builtin_bit_cast(uint32_t, p);
+}
+
+// Launchers implemented in the .hip files; all validated by api.hip before the call.
+int launch_dpa_generic(const af3_dpa_params& p, hipStream_t s);
+int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s);
+int launch_dpa_mfma_fp8(const af3_dpa_params& p, hipStream_t s);
+bool mfma_bf16_eligible(const af3_dpa_params& p);
+bool mfma_fp8_eligible(const af3_dpa_params& p);
+
+}  // namespace af3

@@ -1,0 +1,278 @@
+// Vectorised element-wise kernels: dtype casts, per-tensor fp8 scaling, pad and VNNI repack.
+//
+// Casts replace tpp::ConvertTPP and the AVX-512 converters of the reference
+// (src/csrc/xsmm_functors.h:139-145, :838-885).  The e4m3 path has no reference behaviour to
+// follow (src/csrc/xsmm_functors.h:218-226 asserts "not implemented"); it implements OCP e4m3fn
+// with round-to-nearest-even and saturation, which is what gfx950's v_cvt_pk_fp8_f32 does.
+#include "common.hpp"
+
+namespace af3 {
+
+constexpr int EW_THREADS = 256;
+
+static inline unsigned ew_blocks(int64_t work_items, int64_t cap = 256 * 64) {
+	int64_t b = (work_items + EW_THREADS - 1) / EW_THREADS;
+	if(b < 1) b = 1;
+	return (unsigned)(b > cap ? cap : b);
+}
+
+// ---- f32 <-> bf16 ----------------------------------------------------------------------------
+__global__ void __launch_bounds__(EW_THREADS) cvt_f32_bf16_kernel(const float* __restrict__ src, uint16_t* __restrict__ dst, int64_t n) {
+	const int64_t stride = (int64_t)gridDim.x * EW_THREADS;
+	const int64_t nvec   = n >> 3;
+	const bool    vec    = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0;
+	int64_t       done   = 0;
+	if(vec) {
+		for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < nvec; i += stride) {
+			const float4 a = reinterpret_cast<const float4*>(src)[2 * i], c = reinterpret_cast<const float4*>(src)[2 * i + 1];
+			u32x4        o = {pack_bf16x2(a.x, a.y), pack_bf16x2(a.z, a.w), pack_bf16x2(c.x, c.y), pack_bf16x2(c.z, c.w)};
+			reinterpret_cast<u32x4*>(dst)[i] = o;
+		}
+		done = nvec << 3;
+	}
+	for(int64_t i = done + (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += stride) dst[i] = (uint16_t)f32_to_bf16_bits(src[i]);
+}
+
+__global__ void __launch_bounds__(EW_THREADS) cvt_bf16_f32_kernel(const uint16_t* __restrict__ src, float* __restrict__ dst, int64_t n) {
+	const int64_t stride = (int64_t)gridDim.x * EW_THREADS;
+	const int64_t nvec   = n >> 3;
+	const bool    vec    = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0;
+	int64_t       done   = 0;
+	if(vec) {
+		for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < nvec; i += stride) {
+			const u32x4 a = reinterpret_cast<const u32x4*>(src)[i];
+			float4      lo = {bf16_bits_to_f32(a[0] & 0xffffu), bf16_bits_to_f32(a[0] >> 16), bf16_bits_to_f32(a[1] & 0xffffu), bf16_bits_to_f32(a[1] >> 16)};
+			float4      hi = {bf16_bits_to_f32(a[2] & 0xffffu), bf16_bits_to_f32(a[2] >> 16), bf16_bits_to_f32(a[3] & 0xffffu), bf16_bits_to_f32(a[3] >> 16)};
+			reinterpret_cast<float4*>(dst)[2 * i]     = lo;
+			reinterpret_cast<float4*>(dst)[2 * i + 1] = hi;
+		}
+		done = nvec << 3;
+	}
+	for(int64_t i = done + (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += stride) dst[i] = bf16_bits_to_f32(src[i]);
+}
+
+// ---- e4m3 -> f32 / bf16 ----------------------------------------------------------------------
+template <bool TO_BF16>
+__global__ void __launch_bounds__(EW_THREADS) cvt_e4m3_kernel(const uint8_t* __restrict__ src, void* __restrict__ dst, int64_t n) {
+	const int64_t stride = (int64_t)gridDim.x * EW_THREADS;
+	const int64_t nvec   = n >> 2;
+	const bool    vec    = ((reinterpret_cast<uintptr_t>(src) & 3) | (reinterpret_cast<uintptr_t>(dst) & 15)) == 0;
+	int64_t       done   = 0;
+	if(vec) {
+		for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < nvec; i += stride) {
+			const uint32_t w  = reinterpret_cast<const uint32_t*>(src)[i];
+			const auto     lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+			const auto     hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+			if(TO_BF16) {
+				u32x2 o = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(hi[0], hi[1])};
+				reinterpret_cast<u32x2*>(dst)[i] = o;
+			} else {
+				float4 o = {lo[0], lo[1], hi[0], hi[1]};
+				reinterpret_cast<float4*>(dst)[i] = o;
+			}
+		}
+		done = nvec << 2;
+	}
+	for(int64_t i = done + (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += stride) {
+		const float f = __builtin_amdgcn_cvt_pk_f32_fp8((uint32_t)src[i], false)[0];
+		if(TO_BF16) static_cast<uint16_t*>(dst)[i] = (uint16_t)f32_to_bf16_bits(f);
+		else static_cast<float*>(dst)[i] = f;
+	}
+}
+
+// ---- per-tensor amax -------------------------------------------------------------------------
+template <bool SRC_BF16>
+__global__ void __launch_bounds__(EW_THREADS) amax_kernel(const void* __restrict__ src, int64_t n, float* amax_out) {
+	const int64_t stride = (int64_t)gridDim.x * EW_THREADS;
+	float         a      = 0.f;
+	for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += stride) {
+		const float f = SRC_BF16 ? bf16_bits_to_f32(static_cast<const uint16_t*>(src)[i]) : static_cast<const float*>(src)[i];
+		a = fmaxf(a, fabsf(f));  // fmaxf drops NaN operands: a NaN element does not poison the scale
+	}
+	for(int o = 32; o > 0; o >>= 1) a = fmaxf(a, __shfl_xor(a, o));
+	// non-negative floats order like their bit patterns
+	if((threadIdx.x & 63) == 0) atomicMax(reinterpret_cast<unsigned int*>(amax_out), __float_as_uint(a));
+}
+
+// scale = 2^floor(log2(448 / (amax*pre_scale))); the power of two keeps every descale product exact.
+__device__ __forceinline__ float fp8_pow2_scale(float amax, float pre_scale) {
+	const float a = amax * fabsf(pre_scale);
+	if(!(a > 0.f) || !(a < INFINITY)) return 1.f;
+	int e;
+	frexpf(448.f / a, &e);             // 448/a = m * 2^e with m in [0.5, 1)  ->  floor(log2) = e - 1
+	e = e - 1;
+	e = e > 120 ? 120 : (e < -120 ? -120 : e);
+	return ldexpf(1.f, e);
+}
+
+template <bool SRC_BF16>
+__global__ void __launch_bounds__(EW_THREADS) quantize_e4m3_kernel(const void* __restrict__ src, uint8_t* __restrict__ dst, int64_t rows, int64_t cols,
+																	 int64_t src_row_stride, int transpose, int64_t rows_per_matrix, int64_t dst_row_stride,
+																	 float pre_scale, const float* amax, float* descale_out) {
+	const float scale = fp8_pow2_scale(*amax, pre_scale);
+	if(blockIdx.x == 0 && threadIdx.x == 0 && descale_out) *descale_out = 1.f / scale;
+	const float   mul    = pre_scale * scale;
+	const int64_t stride = (int64_t)gridDim.x * EW_THREADS;
+	auto          ld     = [&](int64_t r, int64_t c) -> float {
+        const int64_t i = r * src_row_stride + c;
+        const float   f = SRC_BF16 ? bf16_bits_to_f32(static_cast<const uint16_t*>(src)[i]) : static_cast<const float*>(src)[i];
+        return fminf(fmaxf(f * mul, -448.f), 448.f);
+	};
+	if(!transpose) {
+		// one thread = 4 consecutive columns of one row (cols % 4 == 0 is checked by the launcher)
+		const int64_t cq = cols >> 2, total = rows * cq;
+		for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += stride) {
+			const int64_t r = i / cq, c = (i % cq) << 2;
+			uint32_t      w = 0;
+			w = __builtin_amdgcn_cvt_pk_fp8_f32(ld(r, c), ld(r, c + 1), w, false);
+			w = __builtin_amdgcn_cvt_pk_fp8_f32(ld(r, c + 2), ld(r, c + 3), w, true);
+			*reinterpret_cast<uint32_t*>(dst + r * dst_row_stride + c) = w;
+		}
+	} else {
+		// one thread = 4 consecutive rows of one column, written as 4 consecutive bytes of dst[matrix][col][row..row+3]
+		const int64_t rq = rows_per_matrix >> 2, n_mat = rows / rows_per_matrix, total = n_mat * rq * cols;
+		for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += stride) {
+			const int64_t c   = i % cols;
+			const int64_t r4  = (i / cols) % rq;
+			const int64_t mat = i / (cols * rq);
+			const int64_t r   = mat * rows_per_matrix + (r4 << 2);
+			uint32_t      w   = 0;
+			w = __builtin_amdgcn_cvt_pk_fp8_f32(ld(r, c), ld(r + 1, c), w, false);
+			w = __builtin_amdgcn_cvt_pk_fp8_f32(ld(r + 2, c), ld(r + 3, c), w, true);
+			*reinterpret_cast<uint32_t*>(dst + (mat * cols + c) * dst_row_stride + (r4 << 2)) = w;
+		}
+	}
+}
+
+// ---- pad / repack ----------------------------------------------------------------------------
+struct PadDims {
+	int     ndim;
+	int64_t src_shape[AF3_PAD_MAX_DIMS], src_stride[AF3_PAD_MAX_DIMS], dst_shape[AF3_PAD_MAX_DIMS];
+};
+
+template <typename T>
+__global__ void __launch_bounds__(EW_THREADS) pad_nd_kernel(const T* __restrict__ src, T* __restrict__ dst, PadDims d, int64_t total, T fill) {
+	const int64_t stride = (int64_t)gridDim.x * EW_THREADS;
+	for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += stride) {
+		int64_t rem = i, soff = 0;
+		bool    in  = true;
+		for(int a = d.ndim - 1; a >= 0; a--) {
+			const int64_t c = rem % d.dst_shape[a];
+			rem /= d.dst_shape[a];
+			in = in && c < d.src_shape[a];
+			soff += c * d.src_stride[a];
+		}
+		dst[i] = in ? src[soff] : fill;
+	}
+}
+
+__global__ void __launch_bounds__(EW_THREADS) vnni_repack_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, int64_t M, int64_t N, int64_t blk) {
+	const int64_t stride = (int64_t)gridDim.x * EW_THREADS, total = M * N;
+	for(int64_t o = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; o < total; o += stride) {
+		// o = panel*M*blk + i*blk*2 + j*2 + k   (src/csrc/xsmm_functors.h:2100-2111 applied per panel, tools.cpp:171-173)
+		const int64_t panel = o / (M * blk), rem = o % (M * blk);
+		const int64_t i = rem / (2 * blk), j = (rem % (2 * blk)) >> 1, k = rem & 1;
+		dst[o] = src[(2 * i + k) * N + panel * blk + j];
+	}
+}
+
+}  // namespace af3
+
+using namespace af3;
+
+extern "C" int af3_convert(const void* src, int32_t sd, void* dst, int32_t dd, int64_t n, void* stream) {
+	if(n < 0) return AF3_ERR_BAD_SHAPE;
+	if(n == 0) return AF3_OK;
+	if(!src || !dst) return AF3_ERR_NULL_POINTER;
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	if(sd == AF3_F32 && dd == AF3_BF16)
+		hipLaunchKernelGGL(cvt_f32_bf16_kernel, dim3(ew_blocks((n + 7) / 8)), dim3(EW_THREADS), 0, s, static_cast<const float*>(src), static_cast<uint16_t*>(dst), n);
+	else if(sd == AF3_BF16 && dd == AF3_F32)
+		hipLaunchKernelGGL(cvt_bf16_f32_kernel, dim3(ew_blocks((n + 7) / 8)), dim3(EW_THREADS), 0, s, static_cast<const uint16_t*>(src), static_cast<float*>(dst), n);
+	else if(sd == AF3_FP8_E4M3 && dd == AF3_F32)
+		hipLaunchKernelGGL(cvt_e4m3_kernel<false>, dim3(ew_blocks((n + 3) / 4)), dim3(EW_THREADS), 0, s, static_cast<const uint8_t*>(src), dst, n);
+	else if(sd == AF3_FP8_E4M3 && dd == AF3_BF16)
+		hipLaunchKernelGGL(cvt_e4m3_kernel<true>, dim3(ew_blocks((n + 3) / 4)), dim3(EW_THREADS), 0, s, static_cast<const uint8_t*>(src), dst, n);
+	else
+		return AF3_ERR_BAD_DTYPE;
+	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+extern "C" int af3_amax(const void* src, int32_t sd, int64_t n, float* amax_out, void* stream) {
+	if(n < 0) return AF3_ERR_BAD_SHAPE;
+	if(!amax_out || (n > 0 && !src)) return AF3_ERR_NULL_POINTER;
+	if(n == 0) return AF3_OK;
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	if(sd == AF3_F32) hipLaunchKernelGGL(amax_kernel<false>, dim3(ew_blocks(n, 2048)), dim3(EW_THREADS), 0, s, src, n, amax_out);
+	else if(sd == AF3_BF16) hipLaunchKernelGGL(amax_kernel<true>, dim3(ew_blocks(n, 2048)), dim3(EW_THREADS), 0, s, src, n, amax_out);
+	else return AF3_ERR_BAD_DTYPE;
+	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+extern "C" int af3_quantize_fp8_e4m3(const void* src, int32_t sd, void* dst, int64_t rows, int64_t cols, int64_t src_row_stride, int32_t transpose_last2,
+									 int64_t rows_per_matrix, int64_t dst_row_stride, float pre_scale, const float* amax, float* descale_out, void* stream) {
+	if(rows < 0 || cols < 0) return AF3_ERR_BAD_SHAPE;
+	if(!amax) return AF3_ERR_NULL_POINTER;
+	if(rows == 0 || cols == 0) return AF3_OK;
+	if(!src || !dst) return AF3_ERR_NULL_POINTER;
+	if(src_row_stride < cols) return AF3_ERR_BAD_STRIDE;
+	if(transpose_last2) {
+		if(rows_per_matrix <= 0 || rows % rows_per_matrix != 0 || rows_per_matrix % 4 != 0) return AF3_ERR_BAD_ARGUMENT;
+		if(dst_row_stride < rows_per_matrix || dst_row_stride % 4 != 0) return AF3_ERR_BAD_STRIDE;
+	} else {
+		if(cols % 4 != 0) return AF3_ERR_BAD_ARGUMENT;
+		if(dst_row_stride < cols || dst_row_stride % 4 != 0) return AF3_ERR_BAD_STRIDE;
+	}
+	if(reinterpret_cast<uintptr_t>(dst) & 3) return AF3_ERR_BAD_ARGUMENT;
+	hipStream_t    s = static_cast<hipStream_t>(stream);
+	const unsigned g = ew_blocks(rows * cols / 4);
+	if(sd == AF3_F32)
+		hipLaunchKernelGGL(quantize_e4m3_kernel<false>, dim3(g), dim3(EW_THREADS), 0, s, src, static_cast<uint8_t*>(dst), rows, cols, src_row_stride, (int)transpose_last2,
+						   rows_per_matrix, dst_row_stride, pre_scale, amax, descale_out);
+	else if(sd == AF3_BF16)
+		hipLaunchKernelGGL(quantize_e4m3_kernel<true>, dim3(g), dim3(EW_THREADS), 0, s, src, static_cast<uint8_t*>(dst), rows, cols, src_row_stride, (int)transpose_last2,
+						   rows_per_matrix, dst_row_stride, pre_scale, amax, descale_out);
+	else
+		return AF3_ERR_BAD_DTYPE;
+	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+extern "C" int af3_pad_nd(const void* src, void* dst, int32_t ndim, const int64_t* src_shape, const int64_t* src_strides, const int64_t* dst_shape,
+						  int32_t elem_size, uint32_t fill_bits, void* stream) {
+	if(ndim < 1 || ndim > AF3_PAD_MAX_DIMS) return AF3_ERR_BAD_SHAPE;
+	if(!src_shape || !src_strides || !dst_shape) return AF3_ERR_NULL_POINTER;
+	PadDims d;
+	d.ndim = ndim;
+	int64_t total = 1, src_total = 1;
+	for(int a = 0; a < ndim; a++) {
+		if(src_shape[a] < 0 || dst_shape[a] < src_shape[a]) return AF3_ERR_BAD_SHAPE;
+		if(src_strides[a] < 0) return AF3_ERR_BAD_STRIDE;
+		d.src_shape[a] = src_shape[a], d.src_stride[a] = src_strides[a], d.dst_shape[a] = dst_shape[a];
+		total *= dst_shape[a];
+		src_total *= src_shape[a];
+	}
+	if(total == 0) return AF3_OK;
+	if(!dst || (src_total > 0 && !src)) return AF3_ERR_NULL_POINTER;
+	hipStream_t    s = static_cast<hipStream_t>(stream);
+	const unsigned g = ew_blocks(total);
+	if(elem_size == 4)
+		hipLaunchKernelGGL(pad_nd_kernel<uint32_t>, dim3(g), dim3(EW_THREADS), 0, s, static_cast<const uint32_t*>(src), static_cast<uint32_t*>(dst), d, total, fill_bits);
+	else if(elem_size == 2)
+		hipLaunchKernelGGL(pad_nd_kernel<uint16_t>, dim3(g), dim3(EW_THREADS), 0, s, static_cast<const uint16_t*>(src), static_cast<uint16_t*>(dst), d, total, (uint16_t)fill_bits);
+	else if(elem_size == 1)
+		hipLaunchKernelGGL(pad_nd_kernel<uint8_t>, dim3(g), dim3(EW_THREADS), 0, s, static_cast<const uint8_t*>(src), static_cast<uint8_t*>(dst), d, total, (uint8_t)fill_bits);
+	else
+		return AF3_ERR_BAD_DTYPE;
+	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+extern "C" int af3_vnni_repack_bf16(const void* src, void* dst, int64_t M, int64_t N, int64_t blk, void* stream) {
+	if(M <= 0 || N <= 0) return AF3_ERR_BAD_SHAPE;
+	if(!src || !dst) return AF3_ERR_NULL_POINTER;
+	if(blk == 0) blk = N;
+	// the reference asserts N % BLK_SZ == 0 and exits (src/csrc/tools.cpp:167); here it is an error code
+	if(blk < 0 || N % blk != 0 || (M & 1)) return AF3_ERR_BAD_ARGUMENT;
+	hipLaunchKernelGGL(vnni_repack_kernel, dim3(ew_blocks(M * N)), dim3(EW_THREADS), 0, static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(src),
+					   static_cast<uint16_t*>(dst), M, N, blk);
+	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}

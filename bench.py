@@ -1,0 +1,129 @@
+"""Benchmark of the biased dot-product-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--case cfg4] [--no-cpu-baseline]
+
+A step is one call of dot_product_attention_cpp (the drop-in for the reference's
+af3_kernels.dot_product_attention_cpp) on synthetic inputs already resident in HBM.  The default
+workload is the headline case: triangle attention, N = 768, 4 heads x 32, batched over 768
+rows, bf16.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "fp32": 157.3}   # MI355X dense matrix peaks
+PEAK_HBM_GBS = 8000.0
+
+
+def cpu_baseline(case, budget_s=12.0):
+    """The CPU restatement of the reference algorithm (oracle/af3_oracle.c, OpenMP over
+    batch x head x 128-row query tiles like src/csrc/dot_product_attention.cpp:88-91), timed on
+    this host with the reference harness's protocol (2 warm-ups, then timed calls, wall clock:
+    examples/dot_product_attention.py:87,130-148) on a bounded sample of the same workload."""
+    import numpy as np
+    from af3_kernels_amd.synthetic import make_inputs
+    from oracle import af3_oracle
+    dtype = af3_oracle.F32 if case.io_dtype == "fp32" else af3_oracle.BF16
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+    batch = min(case.B, 2)
+    per_row = 4.0 * case.H * case.L * case.L * case.D
+
+    def run(nb):
+        q, k, v, mask, bias = [t.float().numpy() if t.dtype != __import__("torch").bool else t.numpy() for t in make_inputs(case, batch=nb)]
+        af3_oracle.dpa_reference(q[:1], k[:1], v[:1], mask[:1] if mask.ndim == 2 else mask, bias, dtype=dtype)   # warm-up
+        t0 = time.time()
+        af3_oracle.dpa_reference(q, k, v, mask, bias, dtype=dtype)
+        return time.time() - t0
+
+    t = run(batch)
+    # grow the sample towards the time budget (whole batch rows; every row is the same amount of work)
+    target = int(min(case.B, max(batch, batch * budget_s / max(t, 1e-3))))
+    if target > batch:
+        batch = target
+        t = run(batch)
+    return {"value": round(per_row * batch / t / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{batch} of {case.B} batch rows of {case.name} (same H, L, D, bias and mask), {t:.2f} s wall, OpenMP restatement of the reference algorithm in {case.io_dtype}",
+            "ms_full_workload_extrapolated": round(t / batch * case.B * 1e3, 1)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--case", default="cfg4")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every (batch, head, query-tile) task is "
+              "independent; see DESIGN.md for how it would shard). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import af3_kernels_amd as af3
+    from af3_kernels_amd.synthetic import CASES, make_inputs
+    af3._lib.load()
+    case = CASES[args.case]
+    dev = torch.device("cuda:0")
+    q, k, v, mask, bias = make_inputs(case, device=dev)
+    fp8 = case.mma_dtype == "fp8"
+    fn = (lambda: af3.dot_product_attention_fp8(q, k, v, mask, bias)) if fp8 else (lambda: af3.dot_product_attention_cpp(q, k, v, mask, bias))
+    kernel = "fp8_mfma" if fp8 else af3.selected_kernel(q, k, v, mask, bias)
+
+    for _ in range(args.warmup):
+        out = fn()
+    torch.cuda.synchronize()
+    # The kernel is enqueued on torch's current stream, so events recorded on that stream bracket it.
+    stream = torch.cuda.current_stream(dev)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for s, e in evs:
+        s.record(stream)
+        out = fn()
+        e.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    per_launch = sorted(s.elapsed_time(e) for s, e in evs)
+    kernel_ms = sum(per_launch) / len(per_launch)          # average launch duration of the timed region
+    ms_per_step = max(wall_ms, kernel_ms) if args.steps < 5 else (evs[0][0].elapsed_time(evs[-1][1]) / args.steps)
+    assert torch.isfinite(out).all()
+
+    tflops = case.flops / (ms_per_step * 1e-3) / 1e12
+    k_tflops = case.flops / (kernel_ms * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[case.mma_dtype]
+    hbm_bound = case.name in ("cfg3", "cfg5")
+    if hbm_bound:
+        ach = case.bytes / (kernel_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+                    "bias_stream_GBps": round(case.H * case.L * case.L * 2 / (kernel_ms * 1e-3) / 1e9, 1)}
+    else:
+        roofline = {"bound": "mfma", "achieved": round(k_tflops, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(k_tflops / peak, 4), "traffic": None}
+    roofline["kernel"] = kernel
+    roofline["kernel_ms_avg"] = round(kernel_ms, 4)
+    roofline["kernel_ms_median"] = round(per_launch[len(per_launch) // 2], 4)
+    roofline["algorithmic_flops_per_launch"] = case.flops
+    roofline["algorithmic_bytes_per_launch"] = case.bytes
+
+    line = {
+        "metric": "biased-attention TFLOP/s + % MFMA peak, triangle attn N=768 bf16 (1 GPU)" if case.name == "cfg4" else f"biased-attention TFLOP/s ({case.name})",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": case.mma_dtype, "data": "synthetic",
+        "config": {"workload": f"{case.name}: B={case.B} H={case.H} L={case.L} D={case.D} io={case.io_dtype} mask={case.mask_kind}",
+                   "flops": case.flops, "pct_of_mfma_peak": round(100 * tflops / peak, 2)},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(case)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,176 @@
+/*
+ * af3_dpa.h -- C ABI of the MI355X (gfx950) biased dot-product-attention library.
+ *
+ * One shared library, libaf3_dpa.so, built from af3_kernels_amd/csrc/ by hipcc.  Every entry
+ * point takes raw device pointers, sizes, element strides and a HIP stream; none of them
+ * allocates, frees, synchronises or terminates the process.  All work is enqueued on the
+ * stream that is passed in (NULL = the default stream).  Return value: AF3_OK (0) or a negative
+ * af3_status; af3_status_string() turns it into text.
+ *
+ * The reference interface each entry point replaces is named beside it (paths are relative to
+ * the reference repository).
+ */
+#ifndef AF3_DPA_H
+#define AF3_DPA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum af3_status {
+	AF3_OK                 = 0,
+	AF3_ERR_NULL_POINTER   = -1, /* a required pointer is NULL */
+	AF3_ERR_BAD_DTYPE      = -2, /* dtype combination not implemented */
+	AF3_ERR_BAD_SHAPE      = -3, /* a dimension is <= 0 or exceeds the supported maximum */
+	AF3_ERR_BAD_STRIDE     = -4, /* negative stride, or innermost stride != 1 */
+	AF3_ERR_UNSUPPORTED_D  = -5, /* head_dim above the supported maximum */
+	AF3_ERR_LAUNCH         = -6, /* hipGetLastError() reported a launch failure */
+	AF3_ERR_BAD_ARGUMENT   = -7, /* any other invalid argument (e.g. N % BLK_SZ != 0) */
+	AF3_ERR_NO_DEVICE_CODE = -8  /* the GPU in use is not gfx950 */
+} af3_status;
+
+typedef enum af3_dtype {
+	AF3_F32      = 0,
+	AF3_BF16     = 1,
+	AF3_FP8_E4M3 = 2 /* OCP e4m3fn: bias 7, max 448, no infinity */
+} af3_dtype;
+
+#define AF3_DPA_MAX_HEAD_DIM 128
+
+/*
+ * Arguments of one attention call: out = softmax(q . k^T * softmax_scale + bias, key_mask) . v
+ *
+ *   q, k, v, out : [B, H, L, D], element strides given for the B, H and L axes, innermost
+ *                  (D) stride is 1.  q_len == k_len == L, as the reference assumes
+ *                  (src/csrc/dot_product_attention.cpp:50-52).
+ *   bias         : [H, L, L] shared by every batch row, element strides for H and the query
+ *                  axis, key axis stride 1.  A bias that is already padded to [H, M, M] is
+ *                  passed with its padded strides (examples/self_attention.py:134-149).
+ *                  NULL means no bias.
+ *   key_mask     : bytes, non-zero = attend (the caller's mask BEFORE the reference wrapper
+ *                  inverts it).  Laid out [B, L] with batch stride key_mask_stride_b; a stride
+ *                  of 0 broadcasts one [L] mask over the batch.  NULL means attend to all.
+ *                  A batch row whose keys are all dropped yields the mean of its V rows, as
+ *                  masked_fill(-1e9) + softmax does in examples/dot_product_attention.py:37-39.
+ *
+ *   io_dtype     : element type of q, k, v.  AF3_F32, AF3_BF16, or AF3_FP8_E4M3 (then q, k
+ *                  are e4m3 bytes [B,H,L,D] and v is e4m3 bytes laid out TRANSPOSED as
+ *                  [B, H, D, L] -- v_stride then holds strides for B, H and D, innermost (L) 1 --
+ *                  as written by af3_quantize_fp8_e4m3 with transpose_last2 = 1).
+ *   bias_dtype   : AF3_F32 or AF3_BF16.          out_dtype : AF3_F32 or AF3_BF16.
+ *   mma_dtype    : arithmetic of the two products: AF3_F32 (fp32 FMA), AF3_BF16 (bf16 MFMA,
+ *                  fp32 accumulate) or AF3_FP8_E4M3 (e4m3 MFMA, fp32 accumulate).
+ *   softmax_scale: D^-1/2 for the reference semantics.  For fp8 inputs the caller may fold it
+ *                  into q before quantisation and pass 1.
+ *   q_descale, k_descale, v_descale : real value = stored value * descale (fp8 only; must be
+ *                  powers of two so that the bias can ride the matrix pipeline exactly).
+ */
+typedef struct af3_dpa_params {
+	const void*    q;
+	const void*    k;
+	const void*    v;
+	const void*    bias;
+	const uint8_t* key_mask;
+	void*          out;
+	int64_t        B, H, L, D;
+	int64_t        q_stride[3];
+	int64_t        k_stride[3];
+	int64_t        v_stride[3];
+	int64_t        out_stride[3];
+	int64_t        bias_stride[2];
+	int64_t        key_mask_stride_b;
+	int32_t        io_dtype;
+	int32_t        bias_dtype;
+	int32_t        out_dtype;
+	int32_t        mma_dtype;
+	float          softmax_scale;
+	float          q_descale;
+	float          k_descale;
+	float          v_descale;
+	int32_t        force_generic; /* non-zero: always take the fp32-FMA kernel (testing aid) */
+	int32_t        reserved;
+	/* Optional: 3 device floats {q_descale, k_descale, v_descale} as written by
+	 * af3_quantize_fp8_e4m3; when non-NULL they override the three host values above, so a
+	 * quantise -> attend sequence needs no device-to-host copy. */
+	const float*   device_descales;
+} af3_dpa_params;
+
+/*
+ * The attention forward pass.
+ * Replaces: at::Tensor dot_product_attention(q, k, v, mask, bias, use_flash_attention, BLK_SZ,
+ * FLASH_SZ) -- src/csrc/dot_product_attention.h:25-32, implemented at
+ * src/csrc/dot_product_attention.cpp:25-198 and :545-559, bound at src/csrc/init.cpp:349-351.
+ * Differences: inputs are const (the reference scales q in place and returns it); the mask is
+ * the un-inverted byte mask instead of a T-typed tensor of 0/1 later multiplied by -1e9; the
+ * CPU blocking hints use_flash_attention / BLK_SZ / FLASH_SZ have no counterpart (the kernel is
+ * always an online-softmax kernel and its tiling is fixed by the hardware).
+ */
+int af3_dpa_forward(const af3_dpa_params* params, void* hip_stream);
+
+/* Which kernel af3_dpa_forward would run for these arguments: 0 = fp32-FMA kernel,
+ * 1 = bf16 MFMA kernel, 2 = fp8 MFMA kernel; negative = af3_status error.  Host only. */
+int af3_dpa_select_kernel(const af3_dpa_params* params);
+
+/*
+ * Element-wise dtype conversion, n contiguous elements, round-to-nearest-even.
+ * Replaces: tpp::ConvertTPP (src/csrc/xsmm_functors.h:838-885) and the AVX-512 helpers
+ * _mm512_convert_bf_ps / _mm256_convert_ps_bf (src/csrc/xsmm_functors.h:139-145).
+ * Supported pairs: f32->bf16, bf16->f32, fp8_e4m3->f32, fp8_e4m3->bf16.
+ */
+int af3_convert(const void* src, int32_t src_dtype, void* dst, int32_t dst_dtype, int64_t n, void* hip_stream);
+
+/*
+ * Per-tensor absolute maximum of n contiguous f32 or bf16 elements, accumulated into
+ * *amax_out (a device float the caller has set to 0, or to a running maximum).
+ * No reference counterpart: the reference's e4m3 converters are "not implemented" asserts
+ * (src/csrc/xsmm_functors.h:218-226); this is the first half of per-tensor fp8 scaling.
+ */
+int af3_amax(const void* src, int32_t src_dtype, int64_t n, float* amax_out, void* hip_stream);
+
+/*
+ * Second half of per-tensor fp8 scaling.  Reads *amax (device), derives
+ *     scale = 2^floor(log2(448 / (amax * pre_scale)))        (1 when amax == 0)
+ * writes dst = e4m3(src * pre_scale * scale), saturating at +-448, and stores the descale
+ * 1/scale to *descale_out (device float).  src is viewed as [rows, cols] row-major with
+ * row stride src_row_stride; with transpose_last2 != 0, every consecutive block of
+ * `rows_per_matrix` rows is written transposed: dst[matrix][col][row], row stride
+ * dst_row_stride (>= rows_per_matrix), so V [B*H*L, D] becomes [B*H, D, L].
+ * No reference counterpart (see af3_amax).
+ */
+int af3_quantize_fp8_e4m3(const void* src, int32_t src_dtype, void* dst, int64_t rows, int64_t cols, int64_t src_row_stride,
+						  int32_t transpose_last2, int64_t rows_per_matrix, int64_t dst_row_stride, float pre_scale, const float* amax,
+						  float* descale_out, void* hip_stream);
+
+/*
+ * N-dimensional pad (ndim <= AF3_PAD_MAX_DIMS): copy src (shape src_shape, element strides
+ * src_strides) into the low corner of a contiguous dst of shape dst_shape (>= src_shape in
+ * every axis) and fill the rest with the 32-bit pattern `fill_bits` truncated to elem_size
+ * (1, 2 or 4 bytes).  The shape / stride arrays are host memory, read before the call returns.
+ * Replaces: pad_and_align_tensor / fast_memcpy -- src/csrc/tools.cpp:16-124.  The attention
+ * kernels never need it (tails are predicated in the kernel); it exists for callers that used
+ * the reference's helper directly.
+ */
+#define AF3_PAD_MAX_DIMS 6
+int af3_pad_nd(const void* src, void* dst, int32_t ndim, const int64_t* src_shape, const int64_t* src_strides, const int64_t* dst_shape,
+			   int32_t elem_size, uint32_t fill_bits, void* hip_stream);
+
+/*
+ * bf16 [M, N] -> per blk-wide column panel [N/blk][M/2][blk][2] (row pairs interleaved).
+ * Replaces: vnni_repack_tensor with type = XFORM_N2V -- src/csrc/tools.cpp:151-176,
+ * tpp::XformExtTPP::ref src/csrc/xsmm_functors.h:2100-2111.  The attention kernels do not
+ * consume this layout (their matrix operands are packed in the load path); it is kept for
+ * callers of the reference helper.  blk == 0 means blk = N.  M must be even, N % blk == 0.
+ */
+int af3_vnni_repack_bf16(const void* src, void* dst, int64_t M, int64_t N, int64_t blk, void* hip_stream);
+
+const char* af3_status_string(int status);
+/* ABI version of this header: bumped whenever a struct layout or signature changes. */
+int af3_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AF3_DPA_H */

@@ -1,0 +1,295 @@
+"""GPU parity tests: the HIP kernels, called through the Python drop-in (which goes through the
+C ABI of include/af3_dpa.h), against the CPU oracle on the same seeded inputs.
+
+Tolerances are the ones the task states, max-abs against the fp64 formula evaluated on the
+same (already rounded) inputs: 1e-4 for fp32, 2e-2 for bf16.  Cases too large for the oracle
+are checked on sampled batch rows and through size-independent properties.
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2}
+
+
+@pytest.fixture(scope="module")
+def af3():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import af3_kernels_amd
+    af3_kernels_amd._lib.load()   # raises if libaf3_dpa.so is missing: no fallback
+    return af3_kernels_amd
+
+
+def dev(*ts):
+    return [t.cuda() if t is not None else None for t in ts]
+
+
+def f32np(t):
+    return t.detach().float().cpu().numpy()
+
+
+def run_case(af3, oracle, q, k, v, mask, bias, tol=None, expect_kernel=None, **kw):
+    """q,k,v,bias: CPU torch tensors (fp32 or bf16); returns the max-abs error vs the formula."""
+    tol = TOL[q.dtype] if tol is None else tol
+    dq, dk, dv, dm, db = dev(q, k, v, mask, bias)
+    if expect_kernel is not None:
+        assert af3.selected_kernel(dq, dk, dv, dm, db) == expect_kernel
+    print(f"case B,H,L,D={tuple(q.shape)} dtype={q.dtype} mask={None if mask is None else tuple(mask.shape)}", flush=True)
+    out = af3.dot_product_attention_cpp(dq, dk, dv, dm, db, **kw)
+    torch.cuda.synchronize()
+    assert out.shape == q.shape and out.dtype == q.dtype and out.is_cuda
+    assert out.data_ptr() != dq.data_ptr()
+    want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), mask.numpy(), f32np(bias))
+    got = f32np(out)
+    assert np.isfinite(got).all()
+    err = float(np.abs(got - want).max())
+    assert err <= tol, f"max abs err {err} > {tol}"
+    return err
+
+
+def rand_inputs(B, H, L, D, dtype, seed=0, mask="none", mask_rank=2):
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = [torch.randn(B, H, L, D, generator=g).to(dtype) for _ in range(3)]
+    bias = torch.randn(H, L, L, generator=g).to(dtype)
+    if mask == "none":
+        m = torch.ones(B, L, dtype=torch.bool)
+    elif mask == "random":
+        m = torch.rand(B, L, generator=g) < 0.7
+        m[:, 0] = True
+    elif mask == "tail":
+        m = torch.ones(B, L, dtype=torch.bool)
+        m[:, L - max(1, L // 10):] = False
+    if mask_rank == 1:
+        m = m[0].clone()
+    return q, k, v, m, bias
+
+
+# ---- golden vectors -------------------------------------------------------------------------
+
+GOLDEN = sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "*.npz")))
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-4] for p in GOLDEN])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_golden_vectors(af3, path, dtype):
+    g = np.load(path)
+    if dtype == torch.bfloat16 and "cfg1" in path:
+        pytest.skip("cfg1 is the fp32 case (its inputs are not bf16-representable)")
+    q, k, v, bias = [torch.from_numpy(g[n]).to(dtype).cuda() for n in ("q", "k", "v", "bias")]
+    mask = torch.from_numpy(g["mask"]).cuda()
+    out = af3.dot_product_attention_cpp(q, k, v, mask, bias)
+    torch.cuda.synchronize()
+    err = np.abs(f32np(out) - g["expected"]).max()
+    assert err <= TOL[dtype], err
+
+
+def test_cfg1_fp32_plumbing_case(af3, oracle):
+    from af3_kernels_amd.synthetic import CASES, make_inputs
+    q, k, v, mask, bias = make_inputs(CASES["cfg1"])
+    err = run_case(af3, oracle, q, k, v, mask, bias, expect_kernel="fp32_fma")
+    assert err < 1e-5   # fp32 FMA with an fp32 softmax sits far inside the 1e-4 budget
+
+
+# ---- bf16 matrix-core kernel ----------------------------------------------------------------
+
+@pytest.mark.parametrize("B,H,L,D,mask,rank", [
+    (2, 4, 128, 32, "none", 2),
+    (3, 4, 384, 32, "tail", 2),      # triangle attention shape, tail padding
+    (2, 4, 768, 32, "random", 2),    # headline shape, random mask
+    (1, 16, 768, 24, "tail", 1),     # pair-biased single attention: head_dim 24, 1-D mask
+    (2, 16, 128, 48, "random", 2),   # diffusion shape of the reference harness, head_dim 48
+    (2, 2, 256, 64, "random", 2),
+    (2, 2, 192, 16, "tail", 2),
+    (3, 4, 37, 32, "random", 2),     # L = 37: the reference harness's small case (odd length)
+    (2, 4, 65, 32, "none", 1),
+    (1, 4, 1491, 32, "tail", 2),     # the reference harness's default length
+    (1, 2, 1000, 24, "random", 1),
+])
+def test_bf16_mfma_matches_formula(af3, oracle, B, H, L, D, mask, rank):
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=L + D, mask=mask, mask_rank=rank)
+    run_case(af3, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+
+
+def test_bf16_mfma_and_fp32_fma_kernels_agree(af3):
+    q, k, v, m, bias = dev(*rand_inputs(2, 4, 200, 32, torch.bfloat16, seed=5, mask="random"))
+    a = af3.dot_product_attention_cpp(q, k, v, m, bias)
+    b = torch.ops.af3_kernels.dpa_forward(q, k, v, m.view(torch.uint8), bias, 1, True)   # force the fp32-FMA kernel
+    torch.cuda.synchronize()
+    assert (a.float() - b.float()).abs().max().item() <= 2e-2
+
+
+def test_reference_flags_do_not_change_results(af3):
+    q, k, v, m, bias = dev(*rand_inputs(2, 4, 300, 32, torch.bfloat16, seed=6, mask="tail"))
+    a = af3.dot_product_attention_cpp(q, k, v, m, bias)
+    b = af3.dot_product_attention_cpp(q, k, v, m, bias, True, 64, 128)
+    assert torch.equal(a, b)
+
+
+def test_native_signature_op_takes_the_inverted_typed_mask(af3):
+    # what the reference wrapper hands to its extension: ~mask cast to q's dtype, [B,1,1,L]
+    q, k, v, m, bias = dev(*rand_inputs(2, 4, 96, 32, torch.bfloat16, seed=7, mask="random"))
+    inv = (~m)[:, None, None, :].to(q.dtype)
+    a = torch.ops.af3_kernels.dot_product_attention(q, k, v, inv, bias, False, 128, 1024)
+    b = af3.dot_product_attention_cpp(q, k, v, m, bias)
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_fully_dropped_row_is_mean_of_v_and_single_key_is_exact(af3, dtype):
+    B, H, L, D = 3, 2, 150, 32
+    q, k, v, m, bias = rand_inputs(B, H, L, D, dtype, seed=8)
+    m[1, :] = False                      # every key dropped -> uniform weights over all L keys
+    m[2, :] = False
+    m[2, 77] = True                      # exactly one live key -> that V row, exactly
+    dq, dk, dv, dm, db = dev(q, k, v, m, bias)
+    out = af3.dot_product_attention_cpp(dq, dk, dv, dm, db)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    mean = v[1].float().mean(dim=1, keepdim=True).expand(H, L, D)
+    assert (out[1].float().cpu() - mean).abs().max().item() <= (1e-5 if dtype == torch.float32 else 8e-3)
+    assert torch.equal(out[2].cpu(), v[2][:, 77:78, :].expand(H, L, D).contiguous())
+
+
+def test_values_at_dropped_keys_do_not_matter(af3):
+    q, k, v, m, bias = rand_inputs(2, 4, 130, 32, torch.bfloat16, seed=9, mask="random")
+    dq, dk, dv, dm, db = dev(q, k, v, m, bias)
+    a = af3.dot_product_attention_cpp(dq, dk, dv, dm, db)
+    k2, v2 = k.clone(), v.clone()
+    for b in range(2):
+        k2[b][:, ~m[b], :] = 50.0        # large finite logits at dropped keys
+        v2[b][:, ~m[b], :] = -1e4
+    b_ = af3.dot_product_attention_cpp(dq, k2.cuda(), v2.cuda(), dm, db)
+    assert torch.equal(a, b_)
+
+
+def test_strided_inputs_and_prepadded_bias(af3, oracle):
+    B, H, L, D, M = 2, 4, 100, 32, 128
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=10, mask="random")
+    big = torch.zeros(B, H, M, D + 32, dtype=torch.bfloat16)          # rows with a larger pitch
+    big[:, :, :L, :D] = q
+    qv = big.cuda()[:, :, :L, :D]
+    kv = k.cuda().transpose(0, 1).contiguous().transpose(0, 1)         # [B,H,L,D] view with permuted strides
+    padded = torch.full((H, M, M), 9.0, dtype=torch.bfloat16)          # garbage outside the L x L corner
+    padded[:, :L, :L] = bias
+    out = af3.dot_product_attention_cpp(qv, kv, v.cuda(), m.cuda(), padded.cuda())
+    want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), f32np(bias))
+    assert np.abs(f32np(out) - want).max() <= 2e-2
+
+
+def test_fp32_fma_kernel_shapes(af3, oracle):
+    for (B, H, L, D, mask) in [(1, 2, 700, 40, "random"), (2, 3, 37, 20, "tail"), (1, 1, 5, 3, "none"), (1, 2, 130, 128, "random")]:
+        q, k, v, m, bias = rand_inputs(B, H, L, D, torch.float32, seed=L, mask=mask)
+        run_case(af3, oracle, q, k, v, m, bias, expect_kernel="fp32_fma")
+    # bf16 storage whose head_dim is not a multiple of 8 also takes this kernel
+    q, k, v, m, bias = rand_inputs(2, 2, 90, 20, torch.bfloat16, seed=11, mask="random")
+    run_case(af3, oracle, q, k, v, m, bias, expect_kernel="fp32_fma")
+
+
+def test_fp32_bias_and_other_dtypes_are_cast_like_the_reference(af3, oracle):
+    q, k, v, m, bias = rand_inputs(2, 4, 64, 32, torch.bfloat16, seed=12, mask="tail")
+    out = af3.dot_product_attention_cpp(q.cuda(), k.float().cuda(), v.float().cuda(), m.float().cuda(), bias.float().cuda())
+    want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), f32np(bias))
+    assert out.dtype == torch.bfloat16 and np.abs(f32np(out) - want).max() <= 2e-2
+
+
+# ---- the benchmark configurations at their real sizes ---------------------------------------
+
+@pytest.mark.parametrize("name,sample_rows", [("cfg2", [0, 191, 383]), ("cfg3", [0]), ("cfg4", [0, 400, 767])])
+def test_named_configs_full_size(af3, oracle, name, sample_rows):
+    """Runs the whole configuration on the GPU; the oracle checks sampled batch rows (every batch
+    row is an independent problem sharing the bias), properties check the rest."""
+    from af3_kernels_amd.synthetic import CASES, make_inputs
+    case = CASES[name]
+    q, k, v, mask, bias = make_inputs(case)
+    dq, dk, dv, dm, db = dev(q, k, v, mask, bias)
+    assert af3.selected_kernel(dq, dk, dv, dm, db) == "bf16_mfma"
+    print(f"{name}: full size {tuple(q.shape)}", flush=True)
+    out = af3.dot_product_attention_cpp(dq, dk, dv, dm, db)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    for b in sample_rows:
+        mrow = mask if mask.dim() == 1 else mask[b:b + 1]
+        want = oracle.dpa_formula(f32np(q[b:b + 1]), f32np(k[b:b + 1]), f32np(v[b:b + 1]), mrow.numpy(), f32np(bias))
+        err = np.abs(f32np(out[b:b + 1]) - want).max()
+        assert err <= case.tol, (name, b, err)
+    # rows of the softmax sum to one: v = 1 gives 1 everywhere (checks every row of the full problem)
+    ones = af3.dot_product_attention_cpp(dq, dk, torch.ones_like(dv), dm, db)
+    assert (ones.float() - 1).abs().max().item() <= 8e-3
+    # a per-(head, query) shift of the bias leaves the result unchanged; the bias is first snapped to multiples of
+    # 1/8 so that bias + shift is exact in bf16 and the two runs see exactly shifted logits
+    coarse = (db.float() * 8).round() / 8
+    shift = torch.randint(-2, 3, (case.H, case.L, 1), device="cuda").float() * 4
+    base = af3.dot_product_attention_cpp(dq, dk, dv, dm, coarse.to(db.dtype))
+    shifted = af3.dot_product_attention_cpp(dq, dk, dv, dm, (coarse + shift).to(db.dtype))
+    assert (shifted.float() - base.float()).abs().max().item() <= 8e-3
+    # output is a convex combination of V rows
+    vmax = dv.float().amax(dim=2, keepdim=True)
+    vmin = dv.float().amin(dim=2, keepdim=True)
+    assert (out.float() <= vmax + 1e-2).all() and (out.float() >= vmin - 1e-2).all()
+
+
+# ---- element-wise kernels -------------------------------------------------------------------
+
+def test_convert_matches_torch_casts(af3):
+    g = torch.Generator().manual_seed(3)
+    x = torch.cat([torch.randn(100003, generator=g) * 7, torch.tensor([0.0, -0.0, 1.00390625, 1.0 + 2 ** -8, 1.0 + 3 * 2 ** -8, 3.3895e38, 1e-40, float("inf")])])
+    got = af3.convert(x.cuda(), torch.bfloat16)
+    assert torch.equal(got.cpu().view(torch.int16), x.to(torch.bfloat16).view(torch.int16))
+    back = af3.convert(got, torch.float32)
+    assert torch.equal(back.cpu(), x.to(torch.bfloat16).float())
+    codes = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    want = codes.float()
+    got = af3.convert(codes.cuda(), torch.float32).cpu()
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got), nan) and torch.equal(got[~nan], want[~nan])
+    assert torch.equal(af3.convert(codes.cuda(), torch.bfloat16).cpu()[~nan], want.to(torch.bfloat16)[~nan])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_quantize_fp8_per_tensor_scale(af3, dtype):
+    g = torch.Generator().manual_seed(4)
+    x = (torch.randn(3, 2, 40, 24, generator=g) * 3).to(dtype)
+    q8, descale = af3.quantize_fp8_e4m3(x.cuda(), pre_scale=0.5)
+    amax = x.float().abs().max().item() * 0.5
+    scale = 2.0 ** np.floor(np.log2(448.0 / amax))
+    assert descale.item() == pytest.approx(1.0 / scale, rel=0, abs=0)
+    want = (x.float() * 0.5 * scale).clamp(-448, 448).to(torch.float8_e4m3fn)
+    assert torch.equal(q8.cpu().view(torch.uint8), want.view(torch.uint8))
+    # transposed form: last two axes swapped
+    t8, d2 = af3.quantize_fp8_e4m3(x.cuda(), transpose_last2=True)
+    scale1 = 2.0 ** np.floor(np.log2(448.0 / (amax * 2)))
+    want_t = (x.float() * scale1).clamp(-448, 448).to(torch.float8_e4m3fn).transpose(-1, -2)
+    assert t8.shape == (3, 2, 24, 40) and torch.equal(t8.cpu().view(torch.uint8), want_t.contiguous().view(torch.uint8))
+    assert d2.item() == 1.0 / scale1
+
+
+def test_pad_and_vnni_repack(af3, oracle):
+    x = torch.arange(2 * 3 * 5, dtype=torch.float32).reshape(2, 3, 5).cuda()
+    y = af3.pad_and_align_tensor(x, (2, 4, 8), True, 1.0)
+    want = torch.ones(2, 4, 8)
+    want[:, :3, :5] = x.cpu()
+    assert torch.equal(y.cpu(), want)
+    assert af3.pad_and_align_tensor(x, (2, 3, 5)) is x                # already padded, contiguous, aligned: returned as is
+    b = torch.randn(4, 37, 37).to(torch.bfloat16).cuda()
+    pb = af3.pad_and_align_tensor(b, (4, 128, 128))
+    assert torch.equal(pb[:, :37, :37], b) and pb[:, 37:, :].abs().sum() == 0 and pb[:, :, 37:].abs().sum() == 0
+    w = torch.randn(16, 24).to(torch.bfloat16)
+    got = af3.vnni_repack_tensor(w.cuda(), 2, 8).cpu().view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got, oracle.vnni_repack(w.view(torch.int16).numpy().view(np.uint16), 8))
+    with pytest.raises(ValueError):
+        af3.vnni_repack_tensor(w.cuda(), 2, 7)
+
+
+def test_timers_report_calls(af3, capsys):
+    q, k, v, m, bias = dev(*rand_inputs(1, 2, 64, 32, torch.bfloat16, seed=1))
+    af3.reset_debug_timers()
+    for _ in range(3):
+        af3.dot_product_attention_cpp(q, k, v, m, bias)
+    af3.print_debug_timers()
+    assert "calls=3" in capsys.readouterr().out

@@ -1,0 +1,166 @@
+"""CPU-only checks: the oracle against the committed golden vectors, the C-ABI library's
+exported symbols and host-side validation (no kernel is launched here), and the host logic of
+the Python wrapper."""
+import ctypes
+import glob
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "*.npz")))
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-4] for p in GOLDEN])
+def test_oracle_reproduces_golden(oracle, path):
+    g = np.load(path)
+    got = oracle.dpa_formula(g["q"], g["k"], g["v"], g["mask"], g["bias"])
+    assert np.abs(got - g["expected"]).max() < 2e-6
+    ref = oracle.dpa_reference(g["q"], g["k"], g["v"], g["mask"], g["bias"], BLK_SZ=64 if g["q"].shape[2] % 64 == 0 else 128)
+    # the compiled reference dilutes an all-dropped row with its zero padding when L % BLK != 0 (tools.cpp pads V with 0,
+    # dot_product_attention.cpp:54 pads the mask with 1.0); everywhere else it agrees with the formula
+    B, L = g["q"].shape[0], g["q"].shape[2]
+    keep = np.broadcast_to(g["mask"].reshape(-1, L), (B, L)) if g["mask"].ndim == 1 else g["mask"]
+    rows = keep.any(1)
+    assert np.abs(ref[rows] - g["expected"][rows]).max() < 2e-5
+
+
+def test_golden_cfg1_is_the_named_case():
+    from af3_kernels_amd.synthetic import CASES, make_inputs
+    g = np.load(os.path.join(ROOT, "tests", "golden", "cfg1_fp32.npz"))
+    q, k, v, mask, bias = make_inputs(CASES["cfg1"])
+    assert q.shape == (2, 4, 128, 32) and bias.shape == (4, 128, 128) and mask.shape == (2, 128)
+    assert mask[0].all() and mask[1, :112].all() and not mask[1, 112:].any()
+    assert np.array_equal(q.numpy(), g["q"]) and np.array_equal(bias.numpy(), g["bias"])
+
+
+# ---- the C-ABI library ---------------------------------------------------------------------
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "af3_dpa.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(af3_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from af3_kernels_amd import _lib
+    lib = _lib.load()
+    names = declared_symbols()
+    assert "af3_dpa_forward" in names and len(names) >= 8
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/af3_dpa.h but not exported"
+    assert sorted(_lib.SYMBOLS) == names
+    assert lib.af3_abi_version() == _lib.ABI_VERSION
+    assert lib.af3_status_string(0) == b"ok"
+
+
+def test_params_struct_matches_header_layout():
+    from af3_kernels_amd._lib import DpaParams
+    # 6 pointers, 4 dims, 4*3 + 2 + 1 strides (int64), 4 int32, 4 floats, 2 int32, 1 pointer
+    assert ctypes.sizeof(DpaParams) == 6 * 8 + 4 * 8 + 15 * 8 + 4 * 4 + 4 * 4 + 2 * 4 + 8
+    assert DpaParams.device_descales.offset == ctypes.sizeof(DpaParams) - 8
+
+
+def _params(**kw):
+    from af3_kernels_amd._lib import DpaParams, AF3_BF16
+    p = DpaParams()
+    B, H, L, D = 2, 4, 64, 32
+    p.B, p.H, p.L, p.D = B, H, L, D
+    for name in ("q", "k", "v", "out"):
+        setattr(p, name, 0x1000)   # never dereferenced: validation fails first or select_kernel is host-only
+        setattr(p, name + "_stride", (ctypes.c_int64 * 3)(H * L * D, L * D, D))
+    p.io_dtype = p.out_dtype = p.mma_dtype = p.bias_dtype = AF3_BF16
+    p.softmax_scale = D ** -0.5
+    for k, v in kw.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_host_validation_returns_error_codes_instead_of_exiting():
+    from af3_kernels_amd import _lib
+    lib = _lib.load()
+    fwd = lib.af3_dpa_forward
+    assert fwd(None, None) == -1
+    assert fwd(ctypes.byref(_params(q=None)), None) == -1
+    assert fwd(ctypes.byref(_params(L=0)), None) == -3
+    assert fwd(ctypes.byref(_params(D=256)), None) == -5
+    assert fwd(ctypes.byref(_params(io_dtype=7)), None) == -2
+    assert fwd(ctypes.byref(_params(io_dtype=0)), None) == -2            # fp32 storage with bf16 arithmetic
+    assert fwd(ctypes.byref(_params(q_stride=(ctypes.c_int64 * 3)(1, 1, 8))), None) == -4   # rows overlap
+    assert fwd(ctypes.byref(_params(softmax_scale=0.0)), None) == -7
+    assert fwd(ctypes.byref(_params(bias=0x1000, bias_stride=(ctypes.c_int64 * 2)(64 * 64, 8))), None) == -4
+    for code in range(-8, 1):
+        assert lib.af3_status_string(code) != b"unknown status"
+    with pytest.raises(ValueError):
+        _lib.check(-3, "x")
+    with pytest.raises(RuntimeError):
+        _lib.check(-6, "x")
+
+
+def test_kernel_selection_is_host_only_and_follows_alignment():
+    from af3_kernels_amd import _lib
+    sel = _lib.load().af3_dpa_select_kernel
+    assert sel(ctypes.byref(_params())) == 1                              # bf16 MFMA
+    assert sel(ctypes.byref(_params(force_generic=1))) == 0
+    assert sel(ctypes.byref(_params(mma_dtype=0))) == 0                   # bf16 storage, fp32 arithmetic
+    assert sel(ctypes.byref(_params(q=0x1002))) == 0                      # misaligned rows -> fp32-FMA kernel
+    assert sel(ctypes.byref(_params(D=20))) == 0                          # head_dim not a multiple of 8
+    s96 = (ctypes.c_int64 * 3)(4 * 64 * 96, 64 * 96, 96)
+    assert sel(ctypes.byref(_params(D=96, q_stride=s96, k_stride=s96, v_stride=s96, out_stride=s96))) == 0   # head_dim > 64
+    assert sel(ctypes.byref(_params(D=96))) == -4                         # rows of 96 with stride 32 overlap
+    assert sel(ctypes.byref(_params(io_dtype=0, mma_dtype=0, out_dtype=0))) == 0
+    assert sel(ctypes.byref(_params(L=-1))) == -3
+
+
+def test_elementwise_entry_points_validate_on_the_host():
+    from af3_kernels_amd import _lib
+    lib = _lib.load()
+    assert lib.af3_convert(None, 0, None, 1, 0, None) == 0               # empty: nothing to do
+    assert lib.af3_convert(None, 0, None, 1, 8, None) == -1
+    assert lib.af3_convert(0x1000, 1, 0x2000, 2, 8, None) == -2          # bf16 -> fp8 goes through af3_quantize_fp8_e4m3
+    assert lib.af3_amax(0x1000, 2, 8, 0x2000, None) == -2
+    assert lib.af3_vnni_repack_bf16(0x1000, 0x2000, 16, 24, 7, None) == -7   # N % BLK_SZ != 0: the reference exits here
+    assert lib.af3_vnni_repack_bf16(0x1000, 0x2000, 15, 24, 8, None) == -7
+    arr = ctypes.c_int64 * 2
+    assert lib.af3_pad_nd(0x1000, 0x2000, 2, arr(4, 4), arr(4, 1), arr(2, 8), 4, 0, None) == -3   # shrinking
+    assert lib.af3_pad_nd(0x1000, 0x2000, 9, arr(4, 4), arr(4, 1), arr(4, 8), 4, 0, None) == -3
+    assert lib.af3_quantize_fp8_e4m3(0x1000, 1, 0x2000, 8, 6, 6, 0, 0, 6, 1.0, 0x3000, None, None) == -7    # cols % 4
+
+
+def test_wrapper_rejects_cpu_tensors_and_bad_shapes():
+    import af3_kernels_amd as af3
+    q = torch.randn(1, 2, 16, 8)
+    mask = torch.ones(16, dtype=torch.bool)
+    bias = torch.zeros(2, 16, 16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        af3.dot_product_attention_cpp(q, q, q, mask, bias)
+    with pytest.raises(ValueError):
+        af3.dot_product_attention_cpp(q.to(torch.float16), q, q, mask, bias)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        af3.vnni_repack_tensor(torch.zeros(4, 4, dtype=torch.bfloat16))
+
+
+def test_wrapper_signature_matches_the_reference():
+    import inspect
+    import af3_kernels_amd as af3
+    sig = inspect.signature(af3.dot_product_attention_cpp)
+    assert list(sig.parameters) == ["q", "k", "v", "mask", "bias", "use_flash_attention", "BLK_SZ", "FLASH_SZ"]
+    assert [sig.parameters[n].default for n in ("use_flash_attention", "BLK_SZ", "FLASH_SZ")] == [False, 128, 1024]
+    assert list(inspect.signature(af3.pad_and_align_tensor).parameters) == ["x", "shape", "need_init", "init", "alignment"]
+    assert list(inspect.signature(af3.vnni_repack_tensor).parameters) == ["x", "type", "BLK_SZ"]
+    assert list(inspect.signature(af3.print_debug_timers).parameters) == ["tid", "detailed"]
+    assert hasattr(torch.ops.af3_kernels, "dot_product_attention") and hasattr(torch.ops.af3_kernels, "dpa_forward")
+
+
+def test_mask_lifting_follows_the_reference_wrapper():
+    from af3_kernels_amd.ops import _lift_mask
+    m1 = torch.tensor([1, 0, 1, 1], dtype=torch.bool)
+    assert _lift_mask(m1, 4).shape == (1, 4) and _lift_mask(m1, 4).dtype == torch.uint8
+    m2 = torch.tensor([[1.0, 0.0, 2.0, 0.0]])
+    assert _lift_mask(m2, 4).tolist() == [[1, 0, 1, 0]]                  # truthy = attend
+    m4 = torch.ones(3, 1, 1, 4, dtype=torch.bool)
+    assert _lift_mask(m4, 4).shape == (3, 4)
+    assert _lift_mask(m1, 4).data_ptr() == m1.data_ptr()                 # bool masks are reinterpreted, not copied

@@ -25,6 +25,7 @@ class DpaParams(ctypes.Structure):
         ("softmax_scale", f32), ("q_descale", f32), ("k_descale", f32), ("v_descale", f32),
         ("force_generic", i32), ("reserved", i32),
         ("device_descales", vp),
+        ("workspace", vp), ("workspace_bytes", i64),
     ]
 
 
@@ -32,6 +33,7 @@ class DpaParams(ctypes.Structure):
 SYMBOLS = {
     "af3_dpa_forward": (ctypes.c_int, [ctypes.POINTER(DpaParams), vp]),
     "af3_dpa_select_kernel": (ctypes.c_int, [ctypes.POINTER(DpaParams)]),
+    "af3_dpa_workspace_bytes": (ctypes.c_int64, [ctypes.POINTER(DpaParams)]),
     "af3_convert": (ctypes.c_int, [vp, i32, vp, i32, i64, vp]),
     "af3_amax": (ctypes.c_int, [vp, i32, i64, vp, vp]),
     "af3_quantize_fp8_e4m3": (ctypes.c_int, [vp, i32, vp, i64, i64, i64, i32, i64, i64, f32, vp, vp, vp]),

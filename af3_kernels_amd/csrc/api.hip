@@ -51,6 +51,12 @@ int select_kernel(const af3_dpa_params& p) {
 
 }  // namespace
 
+extern "C" int64_t af3_dpa_workspace_bytes(const af3_dpa_params* params) {
+	const int rc = validate(params);
+	if(rc != AF3_OK) return rc;
+	return select_kernel(*params) == 1 ? mfma_bf16_workspace_bytes(*params) : 0;
+}
+
 extern "C" int af3_dpa_select_kernel(const af3_dpa_params* params) {
 	const int rc = validate(params);
 	if(rc != AF3_OK) return rc;

@@ -1,20 +1,22 @@
 // bf16 matrix-core attention kernel for gfx950 (CDNA4): out = softmax(q.k^T*scale + bias, mask).v
 //
-// Work split.  One workgroup = 4 wavefronts = 128 query rows of one (batch, head); each
-// wavefront owns 32 query rows and walks the key axis in tiles of 64 keys with an online
-// softmax.  K and V tiles are staged once per workgroup in LDS (double buffered); the bias tile
-// is not shared between wavefronts, so every lane loads its own 16-byte bias fragments straight
-// from global memory (L2-resident: the bias is shared by all batch rows).
+// Work split.  One workgroup = NW wavefronts (4, 2 or 1, chosen so that the launch fills the
+// chip) = NW*32 query rows of one (batch, head); each wavefront owns 32 query rows and walks the
+// key axis in tiles of 64 keys with an online softmax.  K and V tiles are staged once per
+// workgroup in LDS, double buffered, by buffer loads that write LDS directly (no register
+// staging, scalar tile offsets, hardware bounds check for rows past L).  The bias tile is not
+// shared between wavefronts, so every lane loads its own 16-byte bias fragments straight from
+// global memory (L2-resident: the bias is shared by all batch rows).
 //
 // Everything is computed "transposed" so that all per-query state is lane-local:
 //   S^T[key][q]  = K . Q^T      v_mfma_f32_32x32x16_bf16, A = K tile (LDS), B = Q (registers)
-//              += I . bias^T    same instruction with A = 0/1 identity fragment, B = bias
-//                               fragment as loaded: bf16 * 1.0 accumulates exactly in fp32, so
-//                               the bias add costs no vector-ALU work
+//              += I . bias^T    same shape with A = 0/1 identity fragment, B = bias fragment as
+//                               loaded: x * 1.0 accumulates exactly in fp32, so the bias add
+//                               costs no vector-ALU work
 //              += m . 1^T       one more MFMA whose A holds the additive key-mask value of each
 //                               key in contraction slot 0 and whose B holds 1.0 in slot 0
 //   In the 32x32 accumulator layout lane (q = lane%32, half = lane/32) holds 16 keys of one
-//   query row, so row max / exp / row sum are in-lane loops plus one half-wave swap.
+//   query row, so exp / row sum are in-lane loops.
 //   O^T[d][q]   += V^T . P^T    A = V^T fragment read with ds_read_b64_tr_b16 from the row-major
 //                               V tile, B = P^T = the accumulator registers converted to bf16
 //                               in place (the accumulator layout IS the B-operand layout).
@@ -22,66 +24,66 @@
 // register), which is this design's counterpart of the reference's VNNI repack
 // (src/csrc/tools.cpp:151-176).
 //
+// Two variants of the inner loop:
+//   natural  (no workspace)  logits in natural units, bias read in place through the identity
+//                            MFMA (exact), p = exp2(fma(s, log2 e, -m*log2 e)).
+//   log2     (workspace)     a prepass writes fp16(bias * log2 e) once per call in fragment order
+//                            (every bias load is then one coalesced 1 KB wave access; fp16 keeps
+//                            11 significant bits, 3 more than the bf16 bias itself), q is scaled
+//                            by scale*log2 e, and the reference maximum m rides the mask MFMA
+//                            (slot 1: A = 1.0, B = -m, m kept bf16-exact), so p = exp2(s) with no
+//                            per-element subtract or multiply at all.
+// Softmax bookkeeping is optimistic: only the very first sub-tile of a row computes a row
+// maximum.  Afterwards p is computed against the current reference and the row sum (needed
+// anyway) is checked; only if a sum is huge or not finite (a logit more than ~26 log2 units above
+// the reference) does the wavefront take a rare path that finds the maximum, moves the reference
+// and rescales the accumulators.  Probabilities may therefore exceed 1 (up to 2^30), which fp32
+// accumulators and bf16 P carry without loss.
+//
 // Reference semantics followed: src/csrc/dot_product_attention.cpp:88-122 (what is computed) and
 // :148-191 (the running max / sum recurrence); the harness formula
 // examples/dot_product_attention.py:20-43 for masking (dropped keys get weight 0, an all-dropped
 // row yields the mean of V).
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace af3 {
 
-constexpr int QT_WAVES = 4;              // wavefronts per workgroup
-constexpr int QT       = QT_WAVES * 32;  // query rows per workgroup
-constexpr int KT       = 64;             // keys per tile
-constexpr int MAX_L_MFMA = 16384;        // mask table (2 B/key) and tile list live in LDS
+constexpr int   KT         = 64;       // keys per tile
+constexpr int   MAX_L_MFMA = 8192;     // mask table (4 B/key) and tile list live in LDS
+constexpr float REF_SLACK  = 12.f;     // log2 units: a moved reference sits this close to the row maximum
+constexpr float PSUM_LIMIT = 0x1p30f;  // per-lane row-sum bound that triggers the rare path
+
+typedef __attribute__((ext_vector_type(2))) __bf16   bf16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+template <int V>
+using ic = std::integral_constant<int, V>;
 
 // ---- LDS layout -----------------------------------------------------------------------------
-// K tile: [KT rows][DP cols] bf16, 16-byte chunks XOR-swizzled so that the 8 lanes served in one
-// LDS cycle of a ds_read_b128 (8 consecutive rows, same logical chunk) hit distinct banks.
+// K tile: [KT rows][DP cols] bf16; the 16-byte chunks of a row are XOR-swizzled so that the 8
+// lanes served in one LDS cycle of a ds_read_b128 (8 consecutive rows, same logical chunk) hit
+// distinct banks.  The swizzle only depends on row % 8.
 template <int DP>
-__device__ __forceinline__ int k_lds_offset(int row, int chunk) {  // in bf16 elements
-	constexpr int CPR = DP / 8;
-	const int     sw  = (CPR == 4) ? ((row >> 1) & 3) : (row & 7);
-	return row * DP + ((chunk ^ sw) << 3);
+__device__ __forceinline__ int k_swizzle(int row) {
+	return (DP == 32) ? ((row >> 1) & 3) : (row & 7);
 }
-// V tile: [KT rows][DP cols] bf16 row-major.  For DP = 64 the two 64-byte halves of a row are
+// V tile: [KT rows][DP cols] bf16 row-major; for DP = 64 the two 64-byte halves of a row are
 // swapped on odd rows (keeps the transposed reads of 8 rows x 64 B spread over all banks).
 template <int DP>
-__device__ __forceinline__ int v_lds_offset(int row, int col) {
-	if(DP == 64) return row * DP + (col ^ ((row & 1) << 5));
-	return row * DP + col;
+__device__ __forceinline__ int v_swizzle(int row) {  // in 16-byte chunks
+	return (DP == 64) ? ((row & 1) << 2) : 0;
 }
 
-template <int DP>
-struct SmemLayout {
-	static constexpr int TILE_ELEMS = KT * DP;
-	uint16_t k[2][TILE_ELEMS];
-	uint16_t v[2][TILE_ELEMS];
-};
-
-// Load 8 consecutive bias values bias[row][key .. key+7] as 4 dwords (MFMA B fragment).
-// Elements at key >= L read as zero.  `vec_ok` = the row base and key are 16-byte aligned.
+// 8 consecutive bias values bias[row][key .. key+7], guarded: elements at key >= L read as zero.
 template <bool BIAS_F32>
-__device__ __forceinline__ u32x4 load_bias8(const void* bias_row, int64_t key, int64_t L, bool row_ok, bool vec_ok) {
-	u32x4 r = {0u, 0u, 0u, 0u};
-	if(!row_ok || key >= L) return r;
-	if(BIAS_F32) {
-		const float* b = static_cast<const float*>(bias_row) + key;
-		float f[8];
-#pragma unroll
-		for(int j = 0; j < 8; j++) f[j] = (key + j < L) ? b[j] : 0.f;
-#pragma unroll
-		for(int j = 0; j < 4; j++) r[j] = pack_bf16x2(f[2 * j], f[2 * j + 1]);
-		return r;
-	}
-	const uint16_t* b = static_cast<const uint16_t*>(bias_row) + key;
-	if(vec_ok && key + 8 <= L) return *reinterpret_cast<const u32x4*>(b);
+__device__ __forceinline__ void load_bias8_guarded(const void* bias_row, int64_t key, int64_t L, bool row_ok, float (&f)[8]) {
 #pragma unroll
 	for(int j = 0; j < 8; j++) {
-		const uint32_t e = (key + j < L) ? (uint32_t)b[j] : 0u;
-		r[j >> 1] |= e << ((j & 1) * 16);
+		f[j] = 0.f;
+		if(row_ok && key + j < L) f[j] = BIAS_F32 ? static_cast<const float*>(bias_row)[key + j] : bf16_bits_to_f32(static_cast<const uint16_t*>(bias_row)[key + j]);
 	}
-	return r;
 }
 
 __device__ __forceinline__ float half_swap_max(float x) {
@@ -95,20 +97,69 @@ __device__ __forceinline__ float half_swap_sum(float x) {
 	return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-// DP: head_dim padded to a multiple of 32 (32 or 64).  BIAS_F32: bias stored as fp32.
-template <int DP, bool BIAS_F32>
-__global__ void __launch_bounds__(QT_WAVES * 64, 2) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups) {
-	constexpr int NC  = DP / 16;  // contraction chunks of QK^T
-	constexpr int NDB = DP / 32;  // 32-row blocks of O^T
-	constexpr int CPR = DP / 8;   // 16-byte chunks per K/V row
-	constexpr int LOADS = KT * CPR / (QT_WAVES * 64);  // 16-byte chunks per thread per tile (1 or 2)
+// ---- bias prepass (log2 variant) ---------------------------------------------------------------
+// Workspace layout: [H][query block of 32][key tile of 64][fragment 4][lane 64] x 16 bytes: exactly
+// the B fragment lane (q = lane%32, g = lane/32) needs for the bias MFMA of fragment f = 2*sub+c2:
+// fp16(bias[q][64*kt + 16*f + 8*g + 0..7] * log2 e), zero outside the L x L corner.
+template <bool BIAS_F32>
+__global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restrict__ bias, u32x4* __restrict__ ws, int64_t H, int64_t L, int64_t stride_h,
+															 int64_t stride_q, int n_qblocks, int n_ktiles, bool vec_ok) {
+	const int64_t total = H * n_qblocks * (int64_t)n_ktiles * 256;
+	for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+		const int     lane = (int)(i & 63), frag = (int)((i >> 6) & 3);
+		const int64_t t    = i >> 8;
+		const int     kt   = (int)(t % n_ktiles);
+		const int64_t t2   = t / n_ktiles;
+		const int     qb   = (int)(t2 % n_qblocks);
+		const int64_t h    = t2 / n_qblocks;
+		const int64_t row  = (int64_t)qb * 32 + (lane & 31);
+		const int64_t key  = (int64_t)kt * KT + 16 * frag + 8 * (lane >> 5);
+		const int64_t esz  = BIAS_F32 ? 4 : 2;
+		const unsigned char* rowp = static_cast<const unsigned char*>(bias) + (h * stride_h + (row < L ? row : 0) * stride_q) * esz;
+		float f[8];
+		if(!BIAS_F32 && vec_ok && row < L && key + 8 <= L) {
+			const u32x4 raw = *reinterpret_cast<const u32x4*>(rowp + key * 2);
+#pragma unroll
+			for(int j = 0; j < 4; j++) f[2 * j] = bf16_bits_to_f32(raw[j] & 0xffffu), f[2 * j + 1] = bf16_bits_to_f32(raw[j] >> 16);
+		} else {
+			load_bias8_guarded<BIAS_F32>(rowp, key, L, row < L, f);
+		}
+		u32x4 o;
+#pragma unroll
+		for(int j = 0; j < 4; j++) {
+			// clamp to the fp16 range: exp2 of anything below -65504 is zero anyway
+			const float a = fminf(fmaxf(f[2 * j] * LOG2E, -65504.f), 65504.f), c = fminf(fmaxf(f[2 * j + 1] * LOG2E, -65504.f), 65504.f);
+			f16x2       h2 = {(_Float16)a, (_Float16)c};
+			o[j] = __builtin_bit_cast(uint32_t, h2);
+		}
+		ws[i] = o;
+	}
+}
 
-	extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-	SmemLayout<DP>& sm      = *reinterpret_cast<SmemLayout<DP>*>(smem_raw);
-	uint16_t* mask_tab      = reinterpret_cast<uint16_t*>(smem_raw + sizeof(SmemLayout<DP>));  // [n_ktiles*KT]
-	const int n_ktiles      = (int)((p.L + KT - 1) / KT);
-	int16_t*  live_list     = reinterpret_cast<int16_t*>(mask_tab + n_ktiles * KT);            // [n_ktiles]
-	__shared__ int s_nvalid;
+// DP: head_dim padded to a multiple of 32 (32 or 64).  NW: wavefronts per workgroup.  L2DOM: log2
+// variant (bias from the workspace, or no bias at all).  BIAS_F32: bias stored as fp32 (natural
+// variant only).
+template <int DP, int NW, bool L2DOM, bool BIAS_F32>
+// (at least 2 wavefronts per SIMD: keeps the register budget at 256 so that the compiler writes MFMA
+// results to ordinary VGPRs instead of AGPRs, which every softmax operand would have to be copied out of)
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP == 32 ? 3 : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups) {
+	constexpr int NC         = DP / 16;            // contraction chunks of QK^T
+	constexpr int NDB        = DP / 32;            // 32-row blocks of O^T
+	constexpr int CPR        = DP / 8;             // 16-byte chunks per K/V row
+	constexpr int TILE_BYTES = KT * DP * 2;
+	constexpr int NI         = TILE_BYTES / 1024;  // 1 KB wave loads per tile and tensor
+	constexpr int RPI        = 512 / DP;           // tile rows covered by one wave load
+	constexpr int QT         = NW * 32;
+	static_assert(NI % NW == 0, "tile loads must divide evenly over the wavefronts");
+
+	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+	// [K buf0][K buf1][V buf0][V buf1][mask table: (n_ktiles*64 + 64) dwords][live list]
+	unsigned char* const k_lds     = smem;
+	unsigned char* const v_lds     = smem + 2 * TILE_BYTES;
+	uint32_t* const      mask_tab  = reinterpret_cast<uint32_t*>(smem + 4 * TILE_BYTES);
+	const int            n_ktiles  = (int)((p.L + KT - 1) / KT);
+	int16_t* const       live_list = reinterpret_cast<int16_t*>(mask_tab + n_ktiles * KT + 64);
+	__shared__ int       s_nvalid, s_nlive;
 
 	// ---- workgroup -> (batch, head, query tile).  Workgroups are handed to the 8 XCDs round
 	// robin, so all query tiles of one (batch, head) are given ids that are congruent mod 8:
@@ -122,20 +173,29 @@ __global__ void __launch_bounds__(QT_WAVES * 64, 2) dpa_mfma_bf16_kernel(af3_dpa
 	if(group >= n_groups) return;
 	const int64_t b = group / p.H, h = group % p.H;
 
-	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-	const int n = lane & 31, half = lane >> 5;
+	const int     tid = threadIdx.x, lane = tid & 63;
+	const int     wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int     n = lane & 31, half = lane >> 5;
 	const int64_t L = p.L;
 	const int     D = (int)p.D;
 
-	// ---- key-mask table (bf16 additive values) and list of tiles with at least one live key ----
+	// ---- zero the K/V buffers: lanes of padded head columns never write them, and whatever a
+	// bounds-checked load leaves behind for rows past L must be finite (0 * stale NaN = NaN) ----
+	for(int i = tid; i < 4 * TILE_BYTES / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
+	// ---- key-mask table and list of tiles with at least one live key ----
+	// entry = bf16 additive mask value in the low half (contraction slot 0) and, in the log2
+	// variant, 1.0 in the high half (slot 1, multiplies -m_ref); the last 64 entries are zero
+	// (read by the lanes of the upper half-wave, whose contraction slots are unused).
 	if(tid == 0) s_nvalid = 0;
+	if(tid < 64) mask_tab[n_ktiles * KT + tid] = 0u;
 	__syncthreads();
 	const uint8_t* keep = p.key_mask ? p.key_mask + b * p.key_mask_stride_b : nullptr;
-	for(int kt = wave; kt < n_ktiles; kt += QT_WAVES) {
-		const int64_t key  = (int64_t)kt * KT + lane;
-		const bool    in   = key < L;
-		const bool    live = in && (keep ? keep[key] != 0 : true);
-		mask_tab[kt * KT + lane] = live ? (uint16_t)0 : (in ? MASK_DROPPED_BF16 : MASK_OUT_OF_RANGE_BF16);
+	for(int kt = wave; kt < n_ktiles; kt += NW) {
+		const int64_t  key  = (int64_t)kt * KT + lane;
+		const bool     in   = key < L;
+		const bool     live = in && (keep ? keep[key] != 0 : true);
+		const uint32_t mv   = live ? 0u : (in ? (uint32_t)MASK_DROPPED_BF16 : (uint32_t)MASK_OUT_OF_RANGE_BF16);
+		mask_tab[kt * KT + lane] = mv | (L2DOM ? 0x3F800000u : 0u);
 		const unsigned long long bal = __ballot(live);
 		if(lane == 0) {
 			live_list[kt] = bal ? 1 : 0;
@@ -143,207 +203,318 @@ __global__ void __launch_bounds__(QT_WAVES * 64, 2) dpa_mfma_bf16_kernel(af3_dpa
 		}
 	}
 	__syncthreads();
-	// Compact the flags into a list (serial; at most a few hundred tiles).  If no key of this
-	// batch row is live every tile is kept: the result is then the mean over all L keys.
-	__shared__ int s_nlive;
+	// Compact the flags into a list (serial; at most 128 tiles).  If no key of this batch row is
+	// live every tile is kept: the result is then the mean over all L keys.
 	if(tid == 0) {
 		const bool all = (s_nvalid == 0);
-		int cnt = 0;
+		int        cnt = 0;
 		for(int kt = 0; kt < n_ktiles; kt++)
 			if(all || live_list[kt]) live_list[cnt++] = (int16_t)kt;
 		s_nlive = cnt;
 	}
 	__syncthreads();
-	const int nlive = s_nlive;
+	const int nlive = __builtin_amdgcn_readfirstlane(s_nlive);
+	// A batch row without any live key: q and the bias are dropped so that every logit is exactly
+	// the mask constant and the weights come out uniform whatever the accumulation order.
+	const bool all_dropped = __builtin_amdgcn_readfirstlane(s_nvalid) == 0;
 
 	// ---- per-lane constants ----
 	const int64_t qrow   = (int64_t)qtile * QT + wave * 32 + n;
 	const bool    row_ok = qrow < L;
 
 	// Q fragments (B operand of S^T = K.Q^T): lane (q = n, g = half) holds q[q][16c + 8g .. +7]
-	// scaled by softmax_scale and rounded to bf16 (the reference also rounds the scaled q,
+	// scaled and rounded to bf16 (the reference also rounds the scaled q,
 	// src/csrc/dot_product_attention.cpp:95-98).
-	bf16x8 qf[NC];
+	const float qmul = all_dropped ? 0.f : (L2DOM ? p.softmax_scale * LOG2E : p.softmax_scale);
+	bf16x8      qf[NC];
 	{
 		const uint16_t* qp = static_cast<const uint16_t*>(p.q) + b * p.q_stride[0] + h * p.q_stride[1] + qrow * p.q_stride[2];
 #pragma unroll
 		for(int c = 0; c < NC; c++) {
-			const int d0 = 16 * c + 8 * half;
+			const int d0  = 16 * c + 8 * half;
 			u32x4     raw = {0u, 0u, 0u, 0u};
 			if(row_ok && d0 < D) raw = *reinterpret_cast<const u32x4*>(qp + d0);
 			u32x4 sc;
 #pragma unroll
-			for(int j = 0; j < 4; j++) {
-				const float lo = bf16_bits_to_f32(raw[j] & 0xffffu) * p.softmax_scale;
-				const float hi = bf16_bits_to_f32(raw[j] >> 16) * p.softmax_scale;
-				sc[j] = pack_bf16x2(lo, hi);
-			}
+			for(int j = 0; j < 4; j++) sc[j] = pack_bf16x2(bf16_bits_to_f32(raw[j] & 0xffffu) * qmul, bf16_bits_to_f32(raw[j] >> 16) * qmul);
 			qf[c] = __builtin_bit_cast(bf16x8, sc);
 		}
 	}
 	// Identity fragments (A operand of the bias MFMA): lane (m = n, g = half), slot j of chunk c2
-	// is 1.0 iff m == 16*c2 + 8*g + j.
-	bf16x8 idf[2];
+	// is 1.0 iff m == 16*c2 + 8*g + j.  bf16 1.0 for the natural variant, fp16 1.0 for the log2 one.
+	u32x4 idf[2];
 #pragma unroll
 	for(int c2 = 0; c2 < 2; c2++) {
 		u32x4     v = {0u, 0u, 0u, 0u};
 		const int j = n - 16 * c2 - 8 * half;
-		if(j >= 0 && j < 8) v[j >> 1] = 0x3F80u << ((j & 1) * 16);
-		idf[c2] = __builtin_bit_cast(bf16x8, v);
+		if(j >= 0 && j < 8) v[j >> 1] = (L2DOM ? 0x3C00u : 0x3F80u) << ((j & 1) * 16);
+		idf[c2] = v;
 	}
-	// B operand of the mask MFMA: 1.0 in contraction slot 0.
-	bf16x8 onef;
-	{
-		u32x4 v = {0u, 0u, 0u, 0u};
-		if(half == 0) v[0] = 0x3F80u;
-		onef = __builtin_bit_cast(bf16x8, v);
-	}
+	// B operand of the mask MFMA: slot 0 = 1.0 (multiplies the key's mask value), slot 1 = -m_ref
+	// (log2 variant; multiplies the 1.0 every key carries in slot 1 of A).
+	u32x4 maskB = {0u, 0u, 0u, 0u};
+	if(half == 0) maskB[0] = 0x3F80u;
+	u32x4 maskA = {0u, 0u, 0u, 0u};
 
+	const bool has_bias = p.bias != nullptr && !all_dropped;
+	// natural variant: direct bias access through per-lane row pointers
 	const unsigned char* bias_row = nullptr;
 	bool                 bias_vec = false;
-	if(p.bias) {
+	if(!L2DOM && has_bias) {
 		const int64_t esz = BIAS_F32 ? 4 : 2;
 		bias_row = static_cast<const unsigned char*>(p.bias) + (h * p.bias_stride[0] + (row_ok ? qrow : 0) * p.bias_stride[1]) * esz;
-		bias_vec = ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) && (p.bias_stride[0] % 8 == 0) && (p.bias_stride[1] % 8 == 0);
+		bias_vec = !BIAS_F32 && ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) && (p.bias_stride[0] % 8 == 0) && (p.bias_stride[1] % 8 == 0);
 	}
-	const bool has_bias = p.bias != nullptr;
+	// log2 variant: fragment-ordered workspace; the tile base is wave-uniform
+	const u32x4* ws_wave = nullptr;
+	if(L2DOM && has_bias) {
+		const int     n_qblocks = (int)((L + 31) / 32);
+		const int64_t qb        = (int64_t)qtile * NW + wave;
+		// query blocks beyond the last one only hold rows >= L; clamp so that loads stay in bounds
+		const int64_t qbc = qb < n_qblocks ? qb : n_qblocks - 1;
+		ws_wave = static_cast<const u32x4*>(p.workspace) + ((h * n_qblocks + qbc) * n_ktiles) * 256;
+	}
 
-	// ---- K/V tile loader: thread -> (row, chunk) of the tile ----
-	const uint16_t* kbase = static_cast<const uint16_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1];
-	const uint16_t* vbase = static_cast<const uint16_t*>(p.v) + b * p.v_stride[0] + h * p.v_stride[1];
-	u32x4 kreg[LOADS], vreg[LOADS];
-	auto  load_tile = [&](int kt) {
+	// ---- K/V tile loader: buffer loads that write LDS directly ----
+	// One wave load moves 1 KB: lane i -> LDS chunk i of the load's 1 KB window, i.e. tile row
+	// j*RPI + i/CPR, physical chunk i%CPR.  The lane picks the global chunk that belongs there
+	// under the swizzle; lanes of padded head columns (chunk*8 >= D) stay idle.
+	const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+		const_cast<uint16_t*>(static_cast<const uint16_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1]), 0, (int)(((L - 1) * p.k_stride[2] + D) * 2), 0x00020000);
+	const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+		const_cast<uint16_t*>(static_cast<const uint16_t*>(p.v) + b * p.v_stride[0] + h * p.v_stride[1]), 0, (int)(((L - 1) * p.v_stride[2] + D) * 2), 0x00020000);
+	const int  ld_row  = lane / CPR, ld_pc = lane % CPR;
+	const int  k_chunk = ld_pc ^ k_swizzle<DP>(ld_row);
+	const int  v_chunk = ld_pc ^ v_swizzle<DP>(ld_row);
+	const int  k_voff  = (int)(ld_row * p.k_stride[2] * 2) + k_chunk * 16;
+	const int  v_voff  = (int)(ld_row * p.v_stride[2] * 2) + v_chunk * 16;
+	const bool k_act   = k_chunk * 8 < D, v_act = v_chunk * 8 < D;
+	const int  k_tile_stride = (int)(KT * p.k_stride[2] * 2), v_tile_stride = (int)(KT * p.v_stride[2] * 2);
+	const int  k_ld_stride   = (int)(RPI * p.k_stride[2] * 2), v_ld_stride = (int)(RPI * p.v_stride[2] * 2);
+	auto       load_tile     = [&](int kt, int buf) {
 #pragma unroll
-		for(int i = 0; i < LOADS; i++) {
-			const int     id  = tid + i * QT_WAVES * 64;
-			const int     row = id / CPR, ch = id % CPR;
-			const int64_t key = (int64_t)kt * KT + row;
-			const bool    ok  = key < L && ch * 8 < D;
-			u32x4         z   = {0u, 0u, 0u, 0u};
-			kreg[i] = ok ? *reinterpret_cast<const u32x4*>(kbase + key * p.k_stride[2] + ch * 8) : z;
-			vreg[i] = ok ? *reinterpret_cast<const u32x4*>(vbase + key * p.v_stride[2] + ch * 8) : z;
+		for(int t = 0; t < NI / NW; t++) {
+			const int j = wave + NW * t;
+			if(k_act)
+				__builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (__attribute__((address_space(3))) void*)(k_lds + buf * TILE_BYTES + j * 1024), 16, k_voff,
+														 kt * k_tile_stride + j * k_ld_stride, 0, 0);
+			if(v_act)
+				__builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (__attribute__((address_space(3))) void*)(v_lds + buf * TILE_BYTES + j * 1024), 16, v_voff,
+														 kt * v_tile_stride + j * v_ld_stride, 0, 0);
 		}
 	};
-	auto store_tile = [&](int buf) {
-#pragma unroll
-		for(int i = 0; i < LOADS; i++) {
-			const int id  = tid + i * QT_WAVES * 64;
-			const int row = id / CPR, ch = id % CPR;
-			*reinterpret_cast<u32x4*>(&sm.k[buf][k_lds_offset<DP>(row, ch)]) = kreg[i];
-			*reinterpret_cast<u32x4*>(&sm.v[buf][v_lds_offset<DP>(row, ch * 8)]) = vreg[i];
-		}
-	};
-	// bias fragments of one 64-key tile: [sub-tile][c2]
-	u32x4 bnext[2][2];
+
+	// bias fragments of one 64-key tile: [2*sub + c2]
+	u32x4 bfrag[4];
 	auto  load_bias_tile = [&](int kt) {
+		if(!has_bias) return;
+		if(L2DOM) {
+			const u32x4* wp = ws_wave + (int64_t)kt * 256 + lane;
 #pragma unroll
-		for(int sub = 0; sub < 2; sub++)
+			for(int f = 0; f < 4; f++) bfrag[f] = wp[f * 64];
+			return;
+		}
+		const int64_t key0 = (int64_t)kt * KT + 8 * half;
+		if(bias_vec && (int64_t)(kt + 1) * KT <= L) {  // wave-uniform: whole tile in range, aligned rows
+			const uint16_t* bp = reinterpret_cast<const uint16_t*>(bias_row) + key0;
+			if(row_ok) {
 #pragma unroll
-			for(int c2 = 0; c2 < 2; c2++) {
-				const int64_t key = (int64_t)kt * KT + 32 * sub + 16 * c2 + 8 * half;
-				bnext[sub][c2] = load_bias8<BIAS_F32>(bias_row, key, L, row_ok && has_bias, bias_vec);
+				for(int f = 0; f < 4; f++) bfrag[f] = *reinterpret_cast<const u32x4*>(bp + 16 * f);
+			} else {
+#pragma unroll
+				for(int f = 0; f < 4; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
 			}
+		} else {
+#pragma unroll
+			for(int f = 0; f < 4; f++) {
+				float v8[8];
+				load_bias8_guarded<BIAS_F32>(bias_row, key0 + 16 * f, L, row_ok, v8);
+#pragma unroll
+				for(int j = 0; j < 4; j++) bfrag[f][j] = pack_bf16x2(v8[2 * j], v8[2 * j + 1]);
+			}
+		}
 	};
+
+	// ---- per-lane LDS read addresses (bytes, for buffer 0 / sub-tile 0; the rest are immediates) ----
+	int k_rd[NC];
+#pragma unroll
+	for(int c = 0; c < NC; c++) k_rd[c] = n * DP * 2 + (((2 * c + half) ^ k_swizzle<DP>(n)) << 4);
+	// V^T fragment reads: lane l: i = l%16, G = l/16 supplies the 8-byte chunk at tile row
+	// base + 4*(G/2) + i/4, column 32*db + 16*(G%2) + 4*(i%4); it receives 4 keys of column 32*db + l%32.
+	int v_rd[NDB];
+	{
+		const int i16 = lane & 15, G = lane >> 4;
+		const int row = 4 * (G >> 1) + (i16 >> 2);
+#pragma unroll
+		for(int db = 0; db < NDB; db++) {
+			const int col   = 32 * db + 16 * (G & 1) + 4 * (i16 & 3);
+			const int chunk = (col >> 3) ^ v_swizzle<DP>(row);
+			v_rd[db] = row * DP * 2 + chunk * 16 + (col & 7) * 2;
+		}
+	}
+	// mask table read address: lanes of the upper half-wave always read the zero entries
+	const int mask_rd     = (int)(4 * TILE_BYTES) + (half == 0 ? n * 4 : (n_ktiles * KT + n) * 4);
+	const int mask_stride = half == 0 ? KT * 4 : 0;
 
 	// ---- online-softmax state (per lane: one query row; the two halves hold disjoint keys) ----
-	const float c_log2 = LOG2E;  // logits are in natural units; exp(x) = exp2(x * log2 e)
-	float       m_run  = -INFINITY;
-	float       l_run  = 0.f;
-	f32x16      oacc[NDB];
+	float  m_ref = 0.f;  // reference maximum: log2 units and bf16-exact (log2 variant), natural units (natural variant)
+	float  mc    = 0.f;  // natural variant: m_ref * log2 e
+	float  l_run = 0.f;
+	f32x16 oacc[NDB];
 #pragma unroll
 	for(int db = 0; db < NDB; db++)
 #pragma unroll
 		for(int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+	const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
+
+	// S^T for one 32-key sub-tile of the tile in LDS buffer BUF
+	auto compute_s = [&](auto buf_c, auto sub_c, int mask_addr) -> f32x16 {
+		constexpr int BUF = decltype(buf_c)::value, SUB = decltype(sub_c)::value;
+		f32x16        s;
+#pragma unroll
+		for(int i = 0; i < 16; i++) s[i] = 0.f;
+#pragma unroll
+		for(int c = 0; c < NC; c++) {
+			const u32x4 kf = *reinterpret_cast<const u32x4*>(k_lds + k_rd[c] + BUF * TILE_BYTES + SUB * 32 * DP * 2);
+			s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf), qf[c], s, 0, 0, 0);
+		}
+		if(has_bias) {
+#pragma unroll
+			for(int c2 = 0; c2 < 2; c2++) {
+				if(L2DOM)
+					s = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, idf[c2]), __builtin_bit_cast(f16x8, bfrag[2 * SUB + c2]), s, 0, 0, 0);
+				else
+					s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, idf[c2]), __builtin_bit_cast(bf16x8, bfrag[2 * SUB + c2]), s, 0, 0, 0);
+			}
+		}
+		maskA[0] = *reinterpret_cast<const uint32_t*>(smem + mask_addr + SUB * 32 * 4);
+		s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), s, 0, 0, 0);
+		return s;
+	};
+
+	// p = exp2(s - reference) for 16 logits, packed to bf16 pairs; returns this lane's part of the row sum
+	auto exp_tile = [&](const f32x16& s, u32x4 (&pf)[2]) -> float {
+		float psum = 0.f;
+#pragma unroll
+		for(int i = 0; i < 16; i += 2) {
+			float p0, p1;
+			if(L2DOM) {
+				p0 = __builtin_amdgcn_exp2f(s[i]);
+				p1 = __builtin_amdgcn_exp2f(s[i + 1]);
+			} else {
+				p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], LOG2E, -mc));
+				p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], LOG2E, -mc));
+			}
+			const uint32_t pk = pack_bf16x2(p0, p1);
+			// row sum over the bf16-rounded probabilities (the values the PV product sees)
+			psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), ones2, psum, false);
+			pf[i >> 3][(i & 7) >> 1] = pk;
+		}
+		return psum;
+	};
+
+	// Move the reference of every row whose maximum is not within REF_SLACK of it (all rows when
+	// `force`), rescale what has been accumulated, and re-express s (and a sub-tile that was
+	// already issued against the old reference) relative to the new one.
+	auto rereference = [&](f32x16& s, f32x16* pending, bool force) {
+		float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+		for(int i = 3; i < 15; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
+		mx = half_swap_max(fmaxf(mx, s[15]));
+		float alpha;
+		if(L2DOM) {
+			// s already has m_ref subtracted (by the mask MFMA)
+			const bool  need  = force || mx > REF_SLACK;
+			const float m_new = need ? bf16_bits_to_f32(f32_to_bf16_bits(m_ref + mx)) : m_ref;
+			const float delta = m_new - m_ref;                      // exact: both are bf16 values
+			alpha = force ? 1.f : __builtin_amdgcn_exp2f(-delta);  // nothing is accumulated yet when forced (first sub-tile)
+#pragma unroll
+			for(int i = 0; i < 16; i++) s[i] -= delta;
+			if(pending) {
+#pragma unroll
+				for(int i = 0; i < 16; i++) (*pending)[i] -= delta;
+			}
+			m_ref = m_new;
+			if(half == 0) maskB[0] = 0x3F80u | (f32_to_bf16_bits(-m_new) << 16);
+		} else {
+			const bool  need  = force || mx > m_ref + REF_SLACK * 0.6931472f;
+			const float m_new = need ? mx : m_ref;
+			alpha = force ? 1.f : __builtin_amdgcn_exp2f((m_ref - m_new) * LOG2E);
+			m_ref = m_new;
+			mc    = m_new * LOG2E;
+		}
+		l_run *= alpha;
+#pragma unroll
+		for(int db = 0; db < NDB; db++)
+#pragma unroll
+			for(int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+	};
+
+	auto softmax_tile = [&](f32x16& s, bool first, u32x4 (&pf)[2], f32x16* pending) {
+		if(first) rereference(s, pending, true);  // wave-uniform
+		float psum = exp_tile(s, pf);
+		if(__ballot(!(psum < PSUM_LIMIT))) {  // also catches inf and NaN; rare
+			rereference(s, pending, false);
+			psum = exp_tile(s, pf);
+		}
+		l_run += psum;
+	};
+
+	// O^T += V^T . P^T for one sub-tile; V^T fragments come from transposing LDS reads
+	auto pv_tile = [&](auto buf_c, auto sub_c, const u32x4 (&pf)[2]) {
+		constexpr int BUF = decltype(buf_c)::value, SUB = decltype(sub_c)::value;
+#pragma unroll
+		for(int cp = 0; cp < 2; cp++) {
+#pragma unroll
+			for(int db = 0; db < NDB; db++) {
+				u32x4 vf;
+#pragma unroll
+				for(int t = 0; t < 2; t++) {
+					const int   off = BUF * TILE_BYTES + (32 * SUB + 16 * cp + 8 * t) * DP * 2;
+					const s16x4 r   = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(v_lds + v_rd[db] + off));
+					const u32x2 rr  = __builtin_bit_cast(u32x2, r);
+					vf[2 * t]       = rr[0];
+					vf[2 * t + 1]   = rr[1];
+				}
+				oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf[cp]), oacc[db], 0, 0, 0);
+			}
+		}
+	};
+
+	auto tile_iteration = [&](auto buf_c, int it) {
+		constexpr int BUF      = decltype(buf_c)::value;
+		const int     kt       = __builtin_amdgcn_readfirstlane((int)live_list[it]);
+		const bool    has_next = it + 1 < nlive;
+		const int     ktn      = has_next ? __builtin_amdgcn_readfirstlane((int)live_list[it + 1]) : kt;
+		if(has_next) load_tile(ktn, BUF ^ 1);
+		const int mask_addr = mask_rd + kt * mask_stride;
+		// both S^T chains are issued first so that the matrix pipe works on sub-tile 1 while the
+		// vector ALU does sub-tile 0's softmax
+		f32x16 s0 = compute_s(buf_c, ic<0>{}, mask_addr);
+		f32x16 s1 = compute_s(buf_c, ic<1>{}, mask_addr);
+		if(has_next) load_bias_tile(ktn);
+		u32x4 pf0[2], pf1[2];
+		softmax_tile(s0, it == 0, pf0, &s1);
+		pv_tile(buf_c, ic<0>{}, pf0);
+		softmax_tile(s1, false, pf1, nullptr);
+		pv_tile(buf_c, ic<1>{}, pf1);
+		// the next tile's K/V must have landed in LDS before anyone reads it
+		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+		__syncthreads();
+	};
 
 	// prologue: first tile
-	load_tile(live_list[0]);
-	load_bias_tile(live_list[0]);
-	store_tile(0);
+	__syncthreads();  // zero fill done
+	load_tile(__builtin_amdgcn_readfirstlane((int)live_list[0]), 0);
+#pragma unroll
+	for(int f = 0; f < 4; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
+	load_bias_tile(__builtin_amdgcn_readfirstlane((int)live_list[0]));
+	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 	__syncthreads();
 
-	for(int it = 0; it < nlive; it++) {
-		const int  kt       = live_list[it];
-		const int  buf      = it & 1;
-		const bool has_next = it + 1 < nlive;
-		u32x4      bcur[2][2];
-#pragma unroll
-		for(int sub = 0; sub < 2; sub++)
-#pragma unroll
-			for(int c2 = 0; c2 < 2; c2++) bcur[sub][c2] = bnext[sub][c2];
-		if(has_next) {
-			const int ktn = live_list[it + 1];
-			load_tile(ktn);
-			load_bias_tile(ktn);
-		}
-
-#pragma unroll
-		for(int sub = 0; sub < 2; sub++) {
-			// ---- S^T = K.Q^T + bias + mask for 32 keys x 32 queries ----
-			f32x16 s;
-#pragma unroll
-			for(int i = 0; i < 16; i++) s[i] = 0.f;
-#pragma unroll
-			for(int c = 0; c < NC; c++) {
-				const u32x4 kf = *reinterpret_cast<const u32x4*>(&sm.k[buf][k_lds_offset<DP>(32 * sub + n, 2 * c + half)]);
-				s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf), qf[c], s, 0, 0, 0);
-			}
-#pragma unroll
-			for(int c2 = 0; c2 < 2; c2++)
-				s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(idf[c2], __builtin_bit_cast(bf16x8, bcur[sub][c2]), s, 0, 0, 0);
-			{
-				u32x4 mv = {0u, 0u, 0u, 0u};
-				const uint32_t mval = mask_tab[kt * KT + 32 * sub + n];
-				mv[0] = half == 0 ? mval : 0u;
-				s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, mv), onef, s, 0, 0, 0);
-			}
-			// ---- online softmax: accumulator register i of lane (q, half) is key 8*(i/4) + 4*half + i%4 ----
-			float mx = s[0];
-#pragma unroll
-			for(int i = 1; i < 16; i++) mx = fmaxf(mx, s[i]);
-			mx = half_swap_max(mx);
-			const float m_new = fmaxf(m_run, mx);
-			const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c_log2);
-			const float mc    = m_new * c_log2;
-			m_run = m_new;
-			float psum = 0.f;
-			u32x4 pf[2];
-#pragma unroll
-			for(int i = 0; i < 16; i += 2) {
-				const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c_log2, -mc));
-				const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], c_log2, -mc));
-				psum += p0 + p1;
-				pf[i >> 3][(i & 7) >> 1] = pack_bf16x2(p0, p1);
-			}
-			l_run = l_run * alpha + psum;
-#pragma unroll
-			for(int db = 0; db < NDB; db++)
-#pragma unroll
-				for(int i = 0; i < 16; i++) oacc[db][i] *= alpha;
-			// ---- O^T += V^T . P^T ; V^T fragments come from transposing LDS reads ----
-#pragma unroll
-			for(int cp = 0; cp < 2; cp++) {
-#pragma unroll
-				for(int db = 0; db < NDB; db++) {
-					// lane l: i = l%16, G = l/16 ; supplies the 8-byte chunk at row keybase + i/4,
-					// column 32*db + 16*(G%2) + 4*(i%4); receives 4 keys of head column 32*db + l%32.
-					const int i16 = lane & 15, G = lane >> 4;
-					const int col = 32 * db + 16 * (G & 1) + 4 * (i16 & 3);
-					u32x4     vf;
-#pragma unroll
-					for(int t = 0; t < 2; t++) {
-						const int   row = 32 * sub + 16 * cp + 8 * t + 4 * (G >> 1) + (i16 >> 2);
-						const s16x4 r   = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-							(__attribute__((address_space(3))) s16x4*)(&sm.v[buf][v_lds_offset<DP>(row, col)]));
-						const u32x2 rr = __builtin_bit_cast(u32x2, r);
-						vf[2 * t]     = rr[0];
-						vf[2 * t + 1] = rr[1];
-					}
-					oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf[cp]), oacc[db], 0, 0, 0);
-				}
-			}
-		}
-		if(has_next) store_tile(buf ^ 1);
-		__syncthreads();
+	for(int it = 0; it < nlive; it += 2) {
+		tile_iteration(ic<0>{}, it);
+		if(it + 1 < nlive) tile_iteration(ic<1>{}, it + 1);
 	}
 
 	// ---- epilogue: O^T register i of block db is head column 32*db + 8*(i/4) + 4*half + i%4 ----
@@ -378,6 +549,8 @@ bool mfma_bf16_eligible(const af3_dpa_params& p) {
 	if(!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v)) return false;
 	for(int i = 0; i < 3; i++)
 		if(p.q_stride[i] % 8 || p.k_stride[i] % 8 || p.v_stride[i] % 8) return false;
+	// buffer addressing of one (batch, head) slab uses 32-bit byte offsets
+	if(p.L * p.k_stride[2] * 2 >= 0x7fffffffLL || p.L * p.v_stride[2] * 2 >= 0x7fffffffLL) return false;
 	if(p.out_dtype == AF3_BF16) {
 		if((reinterpret_cast<uintptr_t>(p.out) & 7) || p.out_stride[0] % 4 || p.out_stride[1] % 4 || p.out_stride[2] % 4) return false;
 	} else {
@@ -386,24 +559,64 @@ bool mfma_bf16_eligible(const af3_dpa_params& p) {
 	return true;
 }
 
-template <int DP, bool BIAS_F32>
+static int64_t ws_bytes_needed(const af3_dpa_params& p) {
+	const int64_t n_qblocks = (p.L + 31) / 32, n_ktiles = (p.L + KT - 1) / KT;
+	return p.H * n_qblocks * n_ktiles * 256 * 16;
+}
+
+// The rewrite costs one extra pass over the bias; it pays off as soon as two batch rows share it.
+int64_t mfma_bf16_workspace_bytes(const af3_dpa_params& p) {
+	if(!mfma_bf16_eligible(p) || !p.bias || p.B < 2) return 0;
+	return ws_bytes_needed(p);
+}
+
+template <int DP, int NW, bool L2DOM, bool BIAS_F32>
 static int launch_one(const af3_dpa_params& p, hipStream_t s) {
+	constexpr int QT       = NW * 32;
 	const int     n_qtiles = (int)((p.L + QT - 1) / QT);
 	const int     n_ktiles = (int)((p.L + KT - 1) / KT);
 	const int64_t n_groups = p.B * p.H;
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
-	const size_t smem = sizeof(SmemLayout<DP>) + (size_t)n_ktiles * KT * 2 + (size_t)n_ktiles * 2 + 16;
-	auto         kern = dpa_mfma_bf16_kernel<DP, BIAS_F32>;
-	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(QT_WAVES * 64), smem, s, p, n_qtiles, n_groups);
+	const size_t smem = (size_t)4 * KT * DP * 2 + ((size_t)n_ktiles * KT + 64) * 4 + (size_t)n_ktiles * 2 + 16;
+	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BIAS_F32>;
+	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, n_qtiles, n_groups);
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }
 
-int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s) {
-	const bool bf32 = p.bias && p.bias_dtype == AF3_F32;
-	if(p.D <= 32) return bf32 ? launch_one<32, true>(p, s) : launch_one<32, false>(p, s);
-	return bf32 ? launch_one<64, true>(p, s) : launch_one<64, false>(p, s);
+template <int DP, bool L2DOM, bool BIAS_F32>
+static int launch_nw(const af3_dpa_params& p, hipStream_t s) {
+	// the largest workgroup that still gives the 256 CUs a few workgroups each
+	const int64_t groups = p.B * p.H;
+	if(groups * ((p.L + 127) / 128) >= 768) return launch_one<DP, 4, L2DOM, BIAS_F32>(p, s);
+	if(groups * ((p.L + 63) / 64) >= 768) return launch_one<DP, 2, L2DOM, BIAS_F32>(p, s);
+	return launch_one<DP, 1, L2DOM, BIAS_F32>(p, s);
 }
 
-// The fp8 kernel is built in its own translation unit.
+int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s) {
+	const bool bf32   = p.bias && p.bias_dtype == AF3_F32;
+	const bool use_ws = p.bias && p.workspace && mfma_bf16_workspace_bytes(p) > 0 && p.workspace_bytes >= ws_bytes_needed(p) &&
+						(reinterpret_cast<uintptr_t>(p.workspace) & 15) == 0;
+	if(use_ws) {
+		const int      n_qblocks = (int)((p.L + 31) / 32), n_ktiles = (int)((p.L + KT - 1) / KT);
+		const int64_t  total     = p.H * n_qblocks * (int64_t)n_ktiles * 256;
+		const unsigned g         = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
+		const bool     vec_ok    = ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) && (p.bias_stride[0] % 8 == 0) && (p.bias_stride[1] % 8 == 0);
+		if(bf32)
+			hipLaunchKernelGGL(bias_prepass_kernel<true>, dim3(g), dim3(256), 0, s, p.bias, static_cast<u32x4*>(p.workspace), p.H, p.L, p.bias_stride[0], p.bias_stride[1],
+							   n_qblocks, n_ktiles, vec_ok);
+		else
+			hipLaunchKernelGGL(bias_prepass_kernel<false>, dim3(g), dim3(256), 0, s, p.bias, static_cast<u32x4*>(p.workspace), p.H, p.L, p.bias_stride[0], p.bias_stride[1],
+							   n_qblocks, n_ktiles, vec_ok);
+		if(hipGetLastError() != hipSuccess) return AF3_ERR_LAUNCH;
+	}
+	const bool l2dom = use_ws || !p.bias;
+	if(p.D <= 32) {
+		if(l2dom) return launch_nw<32, true, false>(p, s);
+		return bf32 ? launch_nw<32, false, true>(p, s) : launch_nw<32, false, false>(p, s);
+	}
+	if(l2dom) return launch_nw<64, true, false>(p, s);
+	return bf32 ? launch_nw<64, false, true>(p, s) : launch_nw<64, false, false>(p, s);
+}
+
 }  // namespace af3

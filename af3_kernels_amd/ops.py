@@ -146,11 +146,17 @@ def _dpa_forward_impl(q, k, v, keep, bias, mma_dtype: int, force_generic: bool) 
     if q.numel() == 0:
         return out
     p = _fill_params(q, k, v, keep, bias, out, mma_dtype, force_generic)
+    lib = _lib.load()
+    ws_bytes = lib.af3_dpa_workspace_bytes(ctypes.byref(p))
+    if ws_bytes > 0:
+        # scratch for the kernel's bias rewrite; torch's caching allocator makes this a pointer bump
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+        p.workspace, p.workspace_bytes = ws.data_ptr(), ws_bytes
     with torch.cuda.device(q.device):
         if _timers.enabled:
             s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             s.record()
-        _lib.check(_lib.load().af3_dpa_forward(ctypes.byref(p), _stream_ptr(q.device)), "af3_dpa_forward")
+        _lib.check(lib.af3_dpa_forward(ctypes.byref(p), _stream_ptr(q.device)), "af3_dpa_forward")
         if _timers.enabled:
             e.record()
             B, H, L, D = q.shape

@@ -96,6 +96,12 @@ typedef struct af3_dpa_params {
 	 * af3_quantize_fp8_e4m3; when non-NULL they override the three host values above, so a
 	 * quantise -> attend sequence needs no device-to-host copy. */
 	const float*   device_descales;
+	/* Optional scratch in device memory, at least af3_dpa_workspace_bytes() long and 256-byte
+	 * aligned.  With it the bf16 kernel first rewrites the bias once (scaled by log2 e and laid
+	 * out in matrix-operand order, shared by all B batch rows) and then runs its fastest variant;
+	 * without it (NULL) the bias is read in place.  Contents are overwritten by every call. */
+	void*          workspace;
+	int64_t        workspace_bytes;
 } af3_dpa_params;
 
 /*
@@ -109,6 +115,10 @@ typedef struct af3_dpa_params {
  * always an online-softmax kernel and its tiling is fixed by the hardware).
  */
 int af3_dpa_forward(const af3_dpa_params* params, void* hip_stream);
+
+/* Bytes of workspace the call would use (0 when a workspace would not help, e.g. B == 1,
+ * no bias, or a kernel that does not take one); negative = af3_status error.  Host only. */
+int64_t af3_dpa_workspace_bytes(const af3_dpa_params* params);
 
 /* Which kernel af3_dpa_forward would run for these arguments: 0 = fp32-FMA kernel,
  * 1 = bf16 MFMA kernel, 2 = fp8 MFMA kernel; negative = af3_status error.  Host only. */

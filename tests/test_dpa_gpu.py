@@ -227,7 +227,7 @@ def test_named_configs_full_size(af3, oracle, name, sample_rows):
     shift = torch.randint(-2, 3, (case.H, case.L, 1), device="cuda").float() * 4
     base = af3.dot_product_attention_cpp(dq, dk, dv, dm, coarse.to(db.dtype))
     shifted = af3.dot_product_attention_cpp(dq, dk, dv, dm, (coarse + shift).to(db.dtype))
-    assert (shifted.float() - base.float()).abs().max().item() <= 8e-3
+    assert (shifted.float() - base.float()).abs().max().item() <= 2e-2   # one bf16 ulp of an output near 2
     # output is a convex combination of V rows
     vmax = dv.float().amax(dim=2, keepdim=True)
     vmin = dv.float().amin(dim=2, keepdim=True)

@@ -59,9 +59,9 @@ def test_library_exports_every_declared_symbol():
 
 def test_params_struct_matches_header_layout():
     from af3_kernels_amd._lib import DpaParams
-    # 6 pointers, 4 dims, 4*3 + 2 + 1 strides (int64), 4 int32, 4 floats, 2 int32, 1 pointer
-    assert ctypes.sizeof(DpaParams) == 6 * 8 + 4 * 8 + 15 * 8 + 4 * 4 + 4 * 4 + 2 * 4 + 8
-    assert DpaParams.device_descales.offset == ctypes.sizeof(DpaParams) - 8
+    # 6 pointers, 4 dims, 4*3 + 2 + 1 strides (int64), 4 int32, 4 floats, 2 int32, 2 pointers, 1 int64
+    assert ctypes.sizeof(DpaParams) == 6 * 8 + 4 * 8 + 15 * 8 + 4 * 4 + 4 * 4 + 2 * 4 + 8 + 8 + 8
+    assert DpaParams.workspace_bytes.offset == ctypes.sizeof(DpaParams) - 8
 
 
 def _params(**kw):

@@ -3,7 +3,7 @@
 // Work split.  One workgroup = NW wavefronts (4, 2 or 1, chosen so that the launch fills the
 // chip) = NW*32 query rows of one (batch, head); each wavefront owns 32 query rows and walks the
 // key axis in tiles of 64 keys with an online softmax.  K and V tiles are staged once per
-// workgroup in LDS, double buffered, by buffer loads that write LDS directly (no register
+// workgroup in LDS, triple buffered, by buffer loads that write LDS directly (no register
 // staging, scalar tile offsets, hardware bounds check for rows past L).  The bias tile is not
 // shared between wavefronts, so every lane loads its own 16-byte bias fragments straight from
 // global memory (L2-resident: the bias is shared by all batch rows).
@@ -142,7 +142,7 @@ __global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restric
 template <int DP, int NW, bool L2DOM, bool BIAS_F32>
 // (at least 2 wavefronts per SIMD: keeps the register budget at 256 so that the compiler writes MFMA
 // results to ordinary VGPRs instead of AGPRs, which every softmax operand would have to be copied out of)
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP == 32 ? 3 : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups) {
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP == 32 ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups) {
 	constexpr int NC         = DP / 16;            // contraction chunks of QK^T
 	constexpr int NDB        = DP / 32;            // 32-row blocks of O^T
 	constexpr int CPR        = DP / 8;             // 16-byte chunks per K/V row
@@ -153,10 +153,10 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	static_assert(NI % NW == 0, "tile loads must divide evenly over the wavefronts");
 
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-	// [K buf0][K buf1][V buf0][V buf1][mask table: (n_ktiles*64 + 64) dwords][live list]
+	// [K x3][V x3][mask table: (n_ktiles*64 + 64) dwords][live list]
 	unsigned char* const k_lds     = smem;
-	unsigned char* const v_lds     = smem + 2 * TILE_BYTES;
-	uint32_t* const      mask_tab  = reinterpret_cast<uint32_t*>(smem + 4 * TILE_BYTES);
+	unsigned char* const v_lds     = smem + 3 * TILE_BYTES;
+	uint32_t* const      mask_tab  = reinterpret_cast<uint32_t*>(smem + 6 * TILE_BYTES);
 	const int            n_ktiles  = (int)((p.L + KT - 1) / KT);
 	int16_t* const       live_list = reinterpret_cast<int16_t*>(mask_tab + n_ktiles * KT + 64);
 	__shared__ int       s_nvalid, s_nlive;
@@ -181,7 +181,8 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 
 	// ---- zero the K/V buffers: lanes of padded head columns never write them, and whatever a
 	// bounds-checked load leaves behind for rows past L must be finite (0 * stale NaN = NaN) ----
-	for(int i = tid; i < 4 * TILE_BYTES / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
+	if(D != DP || L % KT != 0)
+		for(int i = tid; i < 6 * TILE_BYTES / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
 	// ---- key-mask table and list of tiles with at least one live key ----
 	// entry = bf16 additive mask value in the low half (contraction slot 0) and, in the log2
 	// variant, 1.0 in the high half (slot 1, multiplies -m_ref); the last 64 entries are zero
@@ -203,14 +204,22 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		}
 	}
 	__syncthreads();
-	// Compact the flags into a list (serial; at most 128 tiles).  If no key of this batch row is
-	// live every tile is kept: the result is then the mean over all L keys.
-	if(tid == 0) {
+	// Compact the flags into a list of live tile indices (wavefront 0, 64 tiles per pass: rank =
+	// number of live tiles below).  If no key of this batch row is live every tile is kept: the
+	// result is then the mean over all L keys.
+	if(wave == 0) {
 		const bool all = (s_nvalid == 0);
 		int        cnt = 0;
-		for(int kt = 0; kt < n_ktiles; kt++)
-			if(all || live_list[kt]) live_list[cnt++] = (int16_t)kt;
-		s_nlive = cnt;
+		for(int base = 0; base < n_ktiles; base += 64) {
+			const int  kt   = base + lane;
+			const bool keepit = kt < n_ktiles && (all || live_list[kt] != 0);
+			const unsigned long long bal = __ballot(keepit);
+			const int rank = __builtin_amdgcn_mbcnt_hi((unsigned)(bal >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)bal, 0));
+			__builtin_amdgcn_wave_barrier();  // all flags of this pass are read before any index is written (cnt + rank <= kt)
+			if(keepit) live_list[cnt + rank] = (int16_t)kt;
+			cnt += __builtin_popcountll(bal);
+		}
+		if(lane == 0) s_nlive = cnt;
 	}
 	__syncthreads();
 	const int nlive = __builtin_amdgcn_readfirstlane(s_nlive);
@@ -304,14 +313,15 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		}
 	};
 
-	// bias fragments of one 64-key tile: [2*sub + c2]
+	// bias fragments of one 64-key tile: [2*sub + c2]; loaded one sub-tile (two fragments) at a time
 	u32x4 bfrag[4];
-	auto  load_bias_tile = [&](int kt) {
+	auto  load_bias_frags = [&](int kt, auto sub_c) {
+		constexpr int SUB = decltype(sub_c)::value;
 		if(!has_bias) return;
 		if(L2DOM) {
 			const u32x4* wp = ws_wave + (int64_t)kt * 256 + lane;
 #pragma unroll
-			for(int f = 0; f < 4; f++) bfrag[f] = wp[f * 64];
+			for(int f = 2 * SUB; f < 2 * SUB + 2; f++) bfrag[f] = wp[f * 64];
 			return;
 		}
 		const int64_t key0 = (int64_t)kt * KT + 8 * half;
@@ -319,14 +329,14 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			const uint16_t* bp = reinterpret_cast<const uint16_t*>(bias_row) + key0;
 			if(row_ok) {
 #pragma unroll
-				for(int f = 0; f < 4; f++) bfrag[f] = *reinterpret_cast<const u32x4*>(bp + 16 * f);
+				for(int f = 2 * SUB; f < 2 * SUB + 2; f++) bfrag[f] = *reinterpret_cast<const u32x4*>(bp + 16 * f);
 			} else {
 #pragma unroll
-				for(int f = 0; f < 4; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
+				for(int f = 2 * SUB; f < 2 * SUB + 2; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
 			}
 		} else {
 #pragma unroll
-			for(int f = 0; f < 4; f++) {
+			for(int f = 2 * SUB; f < 2 * SUB + 2; f++) {
 				float v8[8];
 				load_bias8_guarded<BIAS_F32>(bias_row, key0 + 16 * f, L, row_ok, v8);
 #pragma unroll
@@ -353,7 +363,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		}
 	}
 	// mask table read address: lanes of the upper half-wave always read the zero entries
-	const int mask_rd     = (int)(4 * TILE_BYTES) + (half == 0 ? n * 4 : (n_ktiles * KT + n) * 4);
+	const int mask_rd     = (int)(6 * TILE_BYTES) + (half == 0 ? n * 4 : (n_ktiles * KT + n) * 4);
 	const int mask_stride = half == 0 ? KT * 4 : 0;
 
 	// ---- online-softmax state (per lane: one query row; the two halves hold disjoint keys) ----
@@ -365,53 +375,6 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	for(int db = 0; db < NDB; db++)
 #pragma unroll
 		for(int i = 0; i < 16; i++) oacc[db][i] = 0.f;
-	const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
-
-	// S^T for one 32-key sub-tile of the tile in LDS buffer BUF
-	auto compute_s = [&](auto buf_c, auto sub_c, int mask_addr) -> f32x16 {
-		constexpr int BUF = decltype(buf_c)::value, SUB = decltype(sub_c)::value;
-		f32x16        s;
-#pragma unroll
-		for(int i = 0; i < 16; i++) s[i] = 0.f;
-#pragma unroll
-		for(int c = 0; c < NC; c++) {
-			const u32x4 kf = *reinterpret_cast<const u32x4*>(k_lds + k_rd[c] + BUF * TILE_BYTES + SUB * 32 * DP * 2);
-			s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf), qf[c], s, 0, 0, 0);
-		}
-		if(has_bias) {
-#pragma unroll
-			for(int c2 = 0; c2 < 2; c2++) {
-				if(L2DOM)
-					s = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, idf[c2]), __builtin_bit_cast(f16x8, bfrag[2 * SUB + c2]), s, 0, 0, 0);
-				else
-					s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, idf[c2]), __builtin_bit_cast(bf16x8, bfrag[2 * SUB + c2]), s, 0, 0, 0);
-			}
-		}
-		maskA[0] = *reinterpret_cast<const uint32_t*>(smem + mask_addr + SUB * 32 * 4);
-		s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), s, 0, 0, 0);
-		return s;
-	};
-
-	// p = exp2(s - reference) for 16 logits, packed to bf16 pairs; returns this lane's part of the row sum
-	auto exp_tile = [&](const f32x16& s, u32x4 (&pf)[2]) -> float {
-		float psum = 0.f;
-#pragma unroll
-		for(int i = 0; i < 16; i += 2) {
-			float p0, p1;
-			if(L2DOM) {
-				p0 = __builtin_amdgcn_exp2f(s[i]);
-				p1 = __builtin_amdgcn_exp2f(s[i + 1]);
-			} else {
-				p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], LOG2E, -mc));
-				p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], LOG2E, -mc));
-			}
-			const uint32_t pk = pack_bf16x2(p0, p1);
-			// row sum over the bf16-rounded probabilities (the values the PV product sees)
-			psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), ones2, psum, false);
-			pf[i >> 3][(i & 7) >> 1] = pk;
-		}
-		return psum;
-	};
 
 	// Move the reference of every row whose maximum is not within REF_SLACK of it (all rows when
 	// `force`), rescale what has been accumulated, and re-express s (and a sub-tile that was
@@ -450,72 +413,187 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			for(int i = 0; i < 16; i++) oacc[db][i] *= alpha;
 	};
 
-	auto softmax_tile = [&](f32x16& s, bool first, u32x4 (&pf)[2], f32x16* pending) {
-		if(first) rereference(s, pending, true);  // wave-uniform
-		float psum = exp_tile(s, pf);
-		if(__ballot(!(psum < PSUM_LIMIT))) {  // also catches inf and NaN; rare
-			rereference(s, pending, false);
-			psum = exp_tile(s, pf);
+	// p = exp2(s - reference) for logits [I0, I0+N) of a sub-tile, packed to bf16 pairs, and this
+	// lane's part of the row sum.  (Plain fp32 adds: on gfx950 v_dot2c_f32_bf16 on the packed pairs
+	// would halve the instruction count but does not execute concurrently with MFMA, adds do.)
+	auto exp_part = [&](const f32x16& s, u32x4 (&pf)[2], float& psum, auto i0_c, auto n_c) {
+		constexpr int I0 = decltype(i0_c)::value, N = decltype(n_c)::value;
+#pragma unroll
+		for(int i = I0; i < I0 + N; i += 2) {
+			float p0, p1;
+			if(L2DOM) {
+				p0 = __builtin_amdgcn_exp2f(s[i]);
+				p1 = __builtin_amdgcn_exp2f(s[i + 1]);
+			} else {
+				p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], LOG2E, -mc));
+				p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], LOG2E, -mc));
+			}
+			psum += p0 + p1;
+			pf[i >> 3][(i & 7) >> 1] = pack_bf16x2(p0, p1);
 		}
-		l_run += psum;
 	};
 
-	// O^T += V^T . P^T for one sub-tile; V^T fragments come from transposing LDS reads
-	auto pv_tile = [&](auto buf_c, auto sub_c, const u32x4 (&pf)[2]) {
-		constexpr int BUF = decltype(buf_c)::value, SUB = decltype(sub_c)::value;
+	// One pipeline stage.  On entry `sc` holds the finished S^T of sub-tile j, `pprev`/`vprev` the
+	// P^T and V^T fragments of sub-tile j-1.  The stage interleaves, one matrix instruction per
+	// handful of vector instructions so that both pipes stay busy within this wavefront:
+	//     matrix pipe                         vector ALU
+	//     O^T += V^T . P^T   (sub-tile j-1)   exp2 / pack of sub-tile j
+	//     S^T of sub-tile j+1 (K.Q^T, bias,   row sum of sub-tile j
+	//                          mask)
+	// and leaves S^T(j+1) in `sc`, P^T(j) in `pprev`, V^T(j) fragments in `vprev`.
+	// k_off / v_off: byte offsets of the LDS buffers holding sub-tile j+1's K rows and sub-tile j's V rows;
+	// SUBN / SUBC: which half of those tiles; FB: first bias fragment of sub-tile j+1.
+	f32x16 sc;
+	u32x4  pprev[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
+	u32x4  vprev[2][NDB];
 #pragma unroll
-		for(int cp = 0; cp < 2; cp++) {
+	for(int cp = 0; cp < 2; cp++)
 #pragma unroll
-			for(int db = 0; db < NDB; db++) {
-				u32x4 vf;
+		for(int db = 0; db < NDB; db++) vprev[cp][db] = u32x4{0u, 0u, 0u, 0u};
+
+	auto read_kfrag = [&](int k_off, int sub, int c) -> u32x4 { return *reinterpret_cast<const u32x4*>(k_lds + k_rd[c] + k_off + sub * 32 * DP * 2); };
+	auto read_vfrags = [&](int v_off, int sub) {
+#pragma unroll
+		for(int cp = 0; cp < 2; cp++)
+#pragma unroll
+			for(int db = 0; db < NDB; db++)
 #pragma unroll
 				for(int t = 0; t < 2; t++) {
-					const int   off = BUF * TILE_BYTES + (32 * SUB + 16 * cp + 8 * t) * DP * 2;
+					const int   off = v_off + (32 * sub + 16 * cp + 8 * t) * DP * 2;
 					const s16x4 r   = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(v_lds + v_rd[db] + off));
 					const u32x2 rr  = __builtin_bit_cast(u32x2, r);
-					vf[2 * t]       = rr[0];
-					vf[2 * t + 1]   = rr[1];
+					vprev[cp][db][2 * t]     = rr[0];
+					vprev[cp][db][2 * t + 1] = rr[1];
 				}
-				oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf[cp]), oacc[db], 0, 0, 0);
-			}
+	};
+	auto bias_mfma = [&](f32x16 s, int f) -> f32x16 {
+		if(L2DOM) return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, idf[f & 1]), __builtin_bit_cast(f16x8, bfrag[f]), s, 0, 0, 0);
+		return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, idf[f & 1]), __builtin_bit_cast(bf16x8, bfrag[f]), s, 0, 0, 0);
+	};
+	// plain (not interleaved) S^T of one sub-tile; used once, for the very first sub-tile
+	auto compute_s_plain = [&](int k_off, int sub, int mask_addr, int fb) -> f32x16 {
+		f32x16 s;
+#pragma unroll
+		for(int i = 0; i < 16; i++) s[i] = 0.f;
+#pragma unroll
+		for(int c = 0; c < NC; c++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, read_kfrag(k_off, sub, c)), qf[c], s, 0, 0, 0);
+		s = bias_mfma(s, fb);
+		s = bias_mfma(s, fb + 1);
+		maskA[0] = *reinterpret_cast<const uint32_t*>(smem + mask_addr + sub * 32 * 4);
+		return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), s, 0, 0, 0);
+	};
+
+	auto stage = [&](auto subn_c, int k_off, int mask_addr_next, int v_off, auto subc_c) {
+		constexpr int SUBN = decltype(subn_c)::value, SUBC = decltype(subc_c)::value, FB = 2 * SUBN;
+		// operands of S^T(j+1) from LDS
+		u32x4 kf[NC];
+#pragma unroll
+		for(int c = 0; c < NC; c++) kf[c] = read_kfrag(k_off, SUBN, c);
+		maskA[0] = *reinterpret_cast<const uint32_t*>(smem + mask_addr_next + SUBN * 32 * 4);
+		u32x4  pcur[2];
+		f32x16 sn;
+#pragma unroll
+		for(int i = 0; i < 16; i++) sn[i] = 0.f;
+		// One matrix instruction, then a handful of vector instructions, and so on: a dependent
+		// MFMA chain would otherwise stall the wavefront for the full 32-cycle pass of each link.
+		// The scheduling barriers keep the compiler from regrouping the chunks.
+#define AF3_CHUNK_END() __builtin_amdgcn_sched_barrier(0)
+		AF3_CHUNK_END();
+		// O^T += V^T . P^T of the previous sub-tile, exp2 of this one
+		float psum = 0.f;
+#pragma unroll
+		for(int db = 0; db < NDB; db++)
+			oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[0][db]), __builtin_bit_cast(bf16x8, pprev[0]), oacc[db], 0, 0, 0);
+		exp_part(sc, pcur, psum, ic<0>{}, ic<2>{});
+		AF3_CHUNK_END();
+#pragma unroll
+		for(int db = 0; db < NDB; db++)
+			oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[1][db]), __builtin_bit_cast(bf16x8, pprev[1]), oacc[db], 0, 0, 0);
+		exp_part(sc, pcur, psum, ic<2>{}, ic<2>{});
+		AF3_CHUNK_END();
+		// S^T of the next sub-tile
+		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[0]), qf[0], sn, 0, 0, 0);
+		// V^T fragments of this sub-tile for the next stage's PV product: issued as soon as the two PV
+		// MFMAs above have consumed the previous fragments, a whole stage before their use
+		read_vfrags(v_off, SUBC);
+		exp_part(sc, pcur, psum, ic<4>{}, ic<2>{});
+		AF3_CHUNK_END();
+		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[1]), qf[1], sn, 0, 0, 0);
+		exp_part(sc, pcur, psum, ic<6>{}, ic<2>{});
+		AF3_CHUNK_END();
+#pragma unroll
+		for(int c = 2; c < NC; c++) sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[c]), qf[c], sn, 0, 0, 0);
+		// (the bias MFMAs run unconditionally -- on zero fragments when there is no bias -- so that the
+		// whole stage stays one basic block)
+		sn = bias_mfma(sn, FB);
+		exp_part(sc, pcur, psum, ic<8>{}, ic<2>{});
+		AF3_CHUNK_END();
+		sn = bias_mfma(sn, FB + 1);
+		exp_part(sc, pcur, psum, ic<10>{}, ic<2>{});
+		AF3_CHUNK_END();
+		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), sn, 0, 0, 0);
+		exp_part(sc, pcur, psum, ic<12>{}, ic<4>{});
+		AF3_CHUNK_END();
+#undef AF3_CHUNK_END
+		if(__ballot(!(psum < PSUM_LIMIT))) {  // a logit far above the reference (or inf / NaN): rare
+			rereference(sc, &sn, false);
+			psum = 0.f;
+			exp_part(sc, pcur, psum, ic<0>{}, ic<16>{});
 		}
+		l_run += psum;
+		sc       = sn;
+		pprev[0] = pcur[0];
+		pprev[1] = pcur[1];
 	};
 
-	auto tile_iteration = [&](auto buf_c, int it) {
-		constexpr int BUF      = decltype(buf_c)::value;
-		const int     kt       = __builtin_amdgcn_readfirstlane((int)live_list[it]);
-		const bool    has_next = it + 1 < nlive;
-		const int     ktn      = has_next ? __builtin_amdgcn_readfirstlane((int)live_list[it + 1]) : kt;
-		if(has_next) load_tile(ktn, BUF ^ 1);
-		const int mask_addr = mask_rd + kt * mask_stride;
-		// both S^T chains are issued first so that the matrix pipe works on sub-tile 1 while the
-		// vector ALU does sub-tile 0's softmax
-		f32x16 s0 = compute_s(buf_c, ic<0>{}, mask_addr);
-		f32x16 s1 = compute_s(buf_c, ic<1>{}, mask_addr);
-		if(has_next) load_bias_tile(ktn);
-		u32x4 pf0[2], pf1[2];
-		softmax_tile(s0, it == 0, pf0, &s1);
-		pv_tile(buf_c, ic<0>{}, pf0);
-		softmax_tile(s1, false, pf1, nullptr);
-		pv_tile(buf_c, ic<1>{}, pf1);
-		// the next tile's K/V must have landed in LDS before anyone reads it
-		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-		__syncthreads();
-	};
-
-	// prologue: first tile
+	// ---- prologue: first two tiles, first sub-tile's S^T and its row maximum ----
+	const int kt0 = __builtin_amdgcn_readfirstlane((int)live_list[0]);
 	__syncthreads();  // zero fill done
-	load_tile(__builtin_amdgcn_readfirstlane((int)live_list[0]), 0);
+	load_tile(kt0, 0);
+	if(nlive > 1) load_tile(__builtin_amdgcn_readfirstlane((int)live_list[1]), 1);
 #pragma unroll
 	for(int f = 0; f < 4; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
-	load_bias_tile(__builtin_amdgcn_readfirstlane((int)live_list[0]));
+	load_bias_frags(kt0, ic<0>{});
+	load_bias_frags(kt0, ic<1>{});
 	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 	__syncthreads();
+	sc = compute_s_plain(0, 0, mask_rd + kt0 * mask_stride, 0);
+	rereference(sc, nullptr, true);
+	if(nlive > 1) load_bias_frags(__builtin_amdgcn_readfirstlane((int)live_list[1]), ic<0>{});
 
-	for(int it = 0; it < nlive; it += 2) {
-		tile_iteration(ic<0>{}, it);
-		if(it + 1 < nlive) tile_iteration(ic<1>{}, it + 1);
+	int buf = 0;  // LDS buffer of tile `it` (it % 3)
+	// tile indices of iterations it, it+1, it+2 are carried in scalar registers; the list entry for
+	// it+3 is fetched at the top of an iteration and only consumed at its end
+	auto live_at = [&](int i) -> int { return (int)live_list[i < nlive ? i : nlive - 1]; };
+	int kt = kt0, kt1 = __builtin_amdgcn_readfirstlane(live_at(1)), kt2 = __builtin_amdgcn_readfirstlane(live_at(2));
+	for(int it = 0; it < nlive; it++) {
+		const int kt3_v = live_at(it + 3);
+		const int bufn = buf == 2 ? 0 : buf + 1, bufnn = bufn == 2 ? 0 : bufn + 1;
+		// sub-tile (it, 0): next is (it, 1) in the same buffer
+		stage(ic<1>{}, buf * TILE_BYTES, mask_rd + kt * mask_stride, buf * TILE_BYTES, ic<0>{});
+		load_bias_frags(kt1, ic<1>{});
+		// Tile it+1 (issued one iteration ago) must have landed, and every wavefront must be done
+		// with tile it-1, whose buffer tile it+2 is about to overwrite.
+		// (vmcnt counts loads in issue order; in the log2 variant exactly four bias-fragment loads were
+		// issued after that tile's LDS-direct loads and may stay in flight)
+		if(L2DOM && has_bias) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+		else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+		__syncthreads();
+		if(it + 2 < nlive) load_tile(kt2, bufnn);
+		// sub-tile (it, 1): next is (it+1, 0) in the next buffer (harmless stale data after the last tile)
+		stage(ic<0>{}, bufn * TILE_BYTES, mask_rd + kt1 * mask_stride, buf * TILE_BYTES, ic<1>{});
+		load_bias_frags(kt2, ic<0>{});
+		buf = bufn;
+		kt  = kt1;
+		kt1 = kt2;
+		kt2 = __builtin_amdgcn_readfirstlane(kt3_v);
 	}
+	// the last sub-tile's PV product
+#pragma unroll
+	for(int cp = 0; cp < 2; cp++)
+#pragma unroll
+		for(int db = 0; db < NDB; db++)
+			oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[cp][db]), __builtin_bit_cast(bf16x8, pprev[cp]), oacc[db], 0, 0, 0);
 
 	// ---- epilogue: O^T register i of block db is head column 32*db + 8*(i/4) + 4*half + i%4 ----
 	const float l_tot = half_swap_sum(l_run);
@@ -578,7 +656,7 @@ static int launch_one(const af3_dpa_params& p, hipStream_t s) {
 	const int64_t n_groups = p.B * p.H;
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
-	const size_t smem = (size_t)4 * KT * DP * 2 + ((size_t)n_ktiles * KT + 64) * 4 + (size_t)n_ktiles * 2 + 16;
+	const size_t smem = (size_t)6 * KT * DP * 2 + ((size_t)n_ktiles * KT + 64) * 4 + (size_t)n_ktiles * 2 + 16;
 	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BIAS_F32>;
 	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, n_qtiles, n_groups);
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;

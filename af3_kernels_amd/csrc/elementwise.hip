@@ -130,15 +130,18 @@ __global__ void __launch_bounds__(EW_THREADS) quantize_e4m3_kernel(const void* _
 		}
 	} else {
 		// one thread = 4 consecutive rows of one column, written as 4 consecutive bytes of dst[matrix][col][row..row+3]
-		const int64_t rq = rows_per_matrix >> 2, n_mat = rows / rows_per_matrix, total = n_mat * rq * cols;
+		// (rows past the end of a matrix quantise to zero)
+		const int64_t rq = (rows_per_matrix + 3) >> 2, n_mat = rows / rows_per_matrix, total = n_mat * rq * cols;
 		for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += stride) {
 			const int64_t c   = i % cols;
 			const int64_t r4  = (i / cols) % rq;
 			const int64_t mat = i / (cols * rq);
 			const int64_t r   = mat * rows_per_matrix + (r4 << 2);
+			const int64_t left = rows_per_matrix - (r4 << 2);
+			const float   f0 = ld(r, c), f1 = left > 1 ? ld(r + 1, c) : 0.f, f2 = left > 2 ? ld(r + 2, c) : 0.f, f3 = left > 3 ? ld(r + 3, c) : 0.f;
 			uint32_t      w   = 0;
-			w = __builtin_amdgcn_cvt_pk_fp8_f32(ld(r, c), ld(r + 1, c), w, false);
-			w = __builtin_amdgcn_cvt_pk_fp8_f32(ld(r + 2, c), ld(r + 3, c), w, true);
+			w = __builtin_amdgcn_cvt_pk_fp8_f32(f0, f1, w, false);
+			w = __builtin_amdgcn_cvt_pk_fp8_f32(f2, f3, w, true);
 			*reinterpret_cast<uint32_t*>(dst + (mat * cols + c) * dst_row_stride + (r4 << 2)) = w;
 		}
 	}
@@ -217,8 +220,8 @@ extern "C" int af3_quantize_fp8_e4m3(const void* src, int32_t sd, void* dst, int
 	if(!src || !dst) return AF3_ERR_NULL_POINTER;
 	if(src_row_stride < cols) return AF3_ERR_BAD_STRIDE;
 	if(transpose_last2) {
-		if(rows_per_matrix <= 0 || rows % rows_per_matrix != 0 || rows_per_matrix % 4 != 0) return AF3_ERR_BAD_ARGUMENT;
-		if(dst_row_stride < rows_per_matrix || dst_row_stride % 4 != 0) return AF3_ERR_BAD_STRIDE;
+		if(rows_per_matrix <= 0 || rows % rows_per_matrix != 0) return AF3_ERR_BAD_ARGUMENT;
+		if(dst_row_stride < (rows_per_matrix + 3) / 4 * 4 || dst_row_stride % 4 != 0) return AF3_ERR_BAD_STRIDE;
 	} else {
 		if(cols % 4 != 0) return AF3_ERR_BAD_ARGUMENT;
 		if(dst_row_stride < cols || dst_row_stride % 4 != 0) return AF3_ERR_BAD_STRIDE;

@@ -291,7 +291,9 @@ def quantize_fp8_e4m3(x: torch.Tensor, pre_scale: float = 1.0, transpose_last2: 
             _lib.check(lib.af3_quantize_fp8_e4m3(x.data_ptr(), _DTYPE_CODE[x.dtype], full.data_ptr(), rows, cols, cols, 1, rows_per_matrix, lpad,
                                                  pre_scale, amax.data_ptr(), descale_out.data_ptr(), st), "af3_quantize_fp8_e4m3")
         else:
-            out = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+            # 16 bytes of slack behind the last row: the fp8 attention kernel fetches rows in 16-byte chunks
+            flat = torch.zeros(x.numel() + 16, dtype=torch.uint8, device=x.device)
+            out = flat[:x.numel()].view(torch.float8_e4m3fn).view(x.shape)
             _lib.check(lib.af3_quantize_fp8_e4m3(x.data_ptr(), _DTYPE_CODE[x.dtype], out.data_ptr(), rows, cols, cols, 0, 0, cols,
                                                  pre_scale, amax.data_ptr(), descale_out.data_ptr(), st), "af3_quantize_fp8_e4m3")
     return out, descale_out

@@ -59,7 +59,9 @@ typedef enum af3_dtype {
  *   io_dtype     : element type of q, k, v.  AF3_F32, AF3_BF16, or AF3_FP8_E4M3 (then q, k
  *                  are e4m3 bytes [B,H,L,D] and v is e4m3 bytes laid out TRANSPOSED as
  *                  [B, H, D, L] -- v_stride then holds strides for B, H and D, innermost (L) 1 --
- *                  as written by af3_quantize_fp8_e4m3 with transpose_last2 = 1).
+ *                  as written by af3_quantize_fp8_e4m3 with transpose_last2 = 1).  K rows are
+ *                  fetched in 16-byte chunks: when D % 16 != 0 the k allocation must extend at
+ *                  least 8 readable bytes past its last row.
  *   bias_dtype   : AF3_F32 or AF3_BF16.          out_dtype : AF3_F32 or AF3_BF16.
  *   mma_dtype    : arithmetic of the two products: AF3_F32 (fp32 FMA), AF3_BF16 (bf16 MFMA,
  *                  fp32 accumulate) or AF3_FP8_E4M3 (e4m3 MFMA, fp32 accumulate).

@@ -141,6 +141,28 @@ float af3o_quantize_e4m3(const float* in, uint8_t* out, int64_t n) {
 	}
 	return scale;
 }
+/* The shipped quantiser's variant: scale = 2^floor(log2(448 / (amax * |pre_scale|))) (1 when amax == 0),
+ * q = e4m3(x * pre_scale * scale).  Power-of-two scales keep descale products exact. */
+float af3o_quantize_e4m3_pow2(const float* in, uint8_t* out, int64_t n, float pre_scale) {
+	float amax = 0.0f;
+	for(int64_t i = 0; i < n; i++) {
+		float a = fabsf(in[i]);
+		if(a > amax) {
+			amax = a;
+		}
+	}
+	float a     = amax * fabsf(pre_scale);
+	float scale = 1.0f;
+	if(a > 0.0f && a < INFINITY) {
+		int e;
+		frexpf(448.0f / a, &e);
+		scale = ldexpf(1.0f, e - 1);
+	}
+	for(int64_t i = 0; i < n; i++) {
+		out[i] = af3o_f32_to_e4m3_bits(in[i] * pre_scale * scale);
+	}
+	return scale;
+}
 void af3o_dequantize_e4m3(const uint8_t* in, float* out, int64_t n, float inv_scale) {
 	for(int64_t i = 0; i < n; i++) {
 		out[i] = af3o_e4m3_bits_to_f32(in[i]) * inv_scale;

@@ -43,6 +43,8 @@ def lib():
         L.af3o_convert_bf16_to_f32.argtypes = [u16, fp, i64]
         L.af3o_quantize_e4m3.argtypes = [fp, u8, i64]
         L.af3o_quantize_e4m3.restype = ctypes.c_float
+        L.af3o_quantize_e4m3_pow2.argtypes = [fp, u8, i64, ctypes.c_float]
+        L.af3o_quantize_e4m3_pow2.restype = ctypes.c_float
         L.af3o_dequantize_e4m3.argtypes = [u8, fp, i64, ctypes.c_float]
         L.af3o_f32_to_e4m3_bits.argtypes = [ctypes.c_float]
         L.af3o_f32_to_e4m3_bits.restype = ctypes.c_uint8
@@ -122,6 +124,15 @@ def quantize_e4m3(x):
     out = np.empty(x.shape, np.uint8)
     scale = lib().af3o_quantize_e4m3(xp, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), x.size)
     return out, float(scale)
+
+
+def fake_quantize_e4m3_pow2(x, pre_scale=1.0):
+    """x -> e4m3 with the shipped quantiser's power-of-two per-tensor scale -> back to float32
+    (including the pre_scale): what the fp8 kernels actually see."""
+    x, xp = _f(x)
+    bits = np.empty(x.shape, np.uint8)
+    scale = lib().af3o_quantize_e4m3_pow2(xp, bits.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), x.size, pre_scale)
+    return dequantize_e4m3(bits, 1.0 / scale)
 
 
 def dequantize_e4m3(bits, inv_scale=1.0):

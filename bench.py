@@ -26,7 +26,7 @@ def cpu_baseline(case, budget_s=12.0):
     batch x head x 128-row query tiles like src/csrc/dot_product_attention.cpp:88-91), timed on
     this host with the reference harness's protocol (2 warm-ups, then timed calls, wall clock:
     examples/dot_product_attention.py:87,130-148) on a bounded sample of the same workload."""
-    import numpy as np
+    import torch
     from af3_kernels_amd.synthetic import make_inputs
     from oracle import af3_oracle
     dtype = af3_oracle.F32 if case.io_dtype == "fp32" else af3_oracle.BF16
@@ -35,11 +35,19 @@ def cpu_baseline(case, budget_s=12.0):
     batch = min(case.B, 2)
     per_row = 4.0 * case.H * case.L * case.L * case.D
 
-    def run(nb):
-        q, k, v, mask, bias = [t.float().numpy() if t.dtype != __import__("torch").bool else t.numpy() for t in make_inputs(case, batch=nb)]
-        af3_oracle.dpa_reference(q[:1], k[:1], v[:1], mask[:1] if mask.ndim == 2 else mask, bias, dtype=dtype)   # warm-up
-        t0 = time.time()
+    cache = {}
+
+    def run_once(nb):
+        if nb not in cache:
+            cache.clear()
+            cache[nb] = [t.float().numpy() if t.dtype != torch.bool else t.numpy() for t in make_inputs(case, batch=nb)]
+        q, k, v, mask, bias = cache[nb]
         af3_oracle.dpa_reference(q, k, v, mask, bias, dtype=dtype)
+
+    def run(nb):
+        run_once(min(nb, 1))     # warm-up
+        t0 = time.time()
+        run_once(nb)
         return time.time() - t0
 
     t = run(batch)
@@ -48,16 +56,42 @@ def cpu_baseline(case, budget_s=12.0):
     if target > batch:
         batch = target
         t = run(batch)
+    reps = 1
+    if t < budget_s * 0.6:   # the whole workload fits the budget several times over: repeat it like the reference harness's COUNT loop
+        reps = max(1, int(budget_s / max(t, 1e-3)))
+        t0 = time.time()
+        for _ in range(reps):
+            run_once(batch)
+        t = (time.time() - t0) / reps
+    # second CPU figure: the harness formula (examples/dot_product_attention.py:20-43) in torch on the CPU, same dtype,
+    # 2 warm-ups then timed calls, on a few batch rows
+    tq, tk, tv, tmask, tbias = make_inputs(case, batch=min(case.B, 8))
+
+    def torch_formula():
+        logits = torch.matmul(tq * case.D ** -0.5, tk.transpose(-1, -2)) + tbias
+        m = tmask[None, None, None, :] if tmask.dim() == 1 else tmask[:, None, None, :]
+        return torch.matmul(torch.softmax(logits.masked_fill(~m, -1e9), dim=-1), tv)
+
+    for _ in range(2):
+        torch_formula()
+    n_t, t0 = 0, time.time()
+    while time.time() - t0 < 3.0:
+        torch_formula()
+        n_t += 1
+    torch_tflops = per_row * tq.shape[0] * n_t / (time.time() - t0) / 1e12
     return {"value": round(per_row * batch / t / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"{batch} of {case.B} batch rows of {case.name} (same H, L, D, bias and mask), {t:.2f} s wall, OpenMP restatement of the reference algorithm in {case.io_dtype}",
+            "torch_cpu_formula_tflops": round(torch_tflops, 5), "torch_threads": torch.get_num_threads(),
+            "sample": f"{batch} of {case.B} batch rows of {case.name} (same H, L, D, bias and mask) x {reps} repeats, {t:.2f} s wall each, "
+                      f"OpenMP restatement of the reference algorithm in {case.io_dtype}",
             "ms_full_workload_extrapolated": round(t / batch * case.B * 1e3, 1)}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    # long enough for the GPU to settle at its sustained clock (a 0.5 ms kernel needs a few hundred launches)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--case", default="cfg4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()

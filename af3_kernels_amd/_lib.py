@@ -26,6 +26,7 @@ class DpaParams(ctypes.Structure):
         ("force_generic", i32), ("reserved", i32),
         ("device_descales", vp),
         ("workspace", vp), ("workspace_bytes", i64),
+        ("q_lo", vp), ("k_lo", vp),
     ]
 
 
@@ -36,7 +37,7 @@ SYMBOLS = {
     "af3_dpa_workspace_bytes": (ctypes.c_int64, [ctypes.POINTER(DpaParams)]),
     "af3_convert": (ctypes.c_int, [vp, i32, vp, i32, i64, vp]),
     "af3_amax": (ctypes.c_int, [vp, i32, i64, vp, vp]),
-    "af3_quantize_fp8_e4m3": (ctypes.c_int, [vp, i32, vp, i64, i64, i64, i32, i64, i64, f32, vp, vp, vp]),
+    "af3_quantize_fp8_e4m3": (ctypes.c_int, [vp, i32, vp, i64, i64, i64, i32, i64, i64, f32, vp, vp, vp, vp]),
     "af3_pad_nd": (ctypes.c_int, [vp, vp, i32, ctypes.POINTER(i64), ctypes.POINTER(i64), ctypes.POINTER(i64), i32, ctypes.c_uint32, vp]),
     "af3_vnni_repack_bf16": (ctypes.c_int, [vp, vp, i64, i64, i64, vp]),
     "af3_status_string": (ctypes.c_char_p, [ctypes.c_int]),

@@ -150,7 +150,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	constexpr int NI         = TILE_BYTES / 1024;  // 1 KB wave loads per tile and tensor
 	constexpr int RPI        = 512 / DP;           // tile rows covered by one wave load
 	constexpr int QT         = NW * 32;
-	static_assert(NI % NW == 0, "tile loads must divide evenly over the wavefronts");
+	static_assert((2 * NI) % NW == 0 || NI % NW == 0, "tile loads must divide evenly over the wavefronts");
 
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 	// [K x3][V x3][mask table: (n_ktiles*64 + 64) dwords][live list]
@@ -301,15 +301,29 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	const int  k_tile_stride = (int)(KT * p.k_stride[2] * 2), v_tile_stride = (int)(KT * p.v_stride[2] * 2);
 	const int  k_ld_stride   = (int)(RPI * p.k_stride[2] * 2), v_ld_stride = (int)(RPI * p.v_stride[2] * 2);
 	auto       load_tile     = [&](int kt, int buf) {
+		if(NW <= NI) {
 #pragma unroll
-		for(int t = 0; t < NI / NW; t++) {
-			const int j = wave + NW * t;
-			if(k_act)
-				__builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (__attribute__((address_space(3))) void*)(k_lds + buf * TILE_BYTES + j * 1024), 16, k_voff,
-														 kt * k_tile_stride + j * k_ld_stride, 0, 0);
-			if(v_act)
-				__builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (__attribute__((address_space(3))) void*)(v_lds + buf * TILE_BYTES + j * 1024), 16, v_voff,
-														 kt * v_tile_stride + j * v_ld_stride, 0, 0);
+			for(int t = 0; t < NI / NW; t++) {
+				const int j = wave + NW * t;
+				if(k_act)
+					__builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (__attribute__((address_space(3))) void*)(k_lds + buf * TILE_BYTES + j * 1024), 16, k_voff,
+															 kt * k_tile_stride + j * k_ld_stride, 0, 0);
+				if(v_act)
+					__builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (__attribute__((address_space(3))) void*)(v_lds + buf * TILE_BYTES + j * 1024), 16, v_voff,
+															 kt * v_tile_stride + j * v_ld_stride, 0, 0);
+			}
+		} else {
+			// more wavefronts than 1 KB pieces per tensor: the first NI wavefronts fetch K, the next NI fetch V
+			if(wave < NI) {
+				if(k_act)
+					__builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (__attribute__((address_space(3))) void*)(k_lds + buf * TILE_BYTES + wave * 1024), 16, k_voff,
+															 kt * k_tile_stride + wave * k_ld_stride, 0, 0);
+			} else if(wave < 2 * NI) {
+				const int j = wave - NI;
+				if(v_act)
+					__builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (__attribute__((address_space(3))) void*)(v_lds + buf * TILE_BYTES + j * 1024), 16, v_voff,
+															 kt * v_tile_stride + j * v_ld_stride, 0, 0);
+			}
 		}
 	};
 

@@ -39,13 +39,15 @@ __device__ __forceinline__ float hswap_sum(float x) {
 }
 
 // DP: head_dim padded to 32 or 64 (bytes per K row in LDS, rows of the V^T tile).
-template <int DP>
+// COMP: compensated logits q8.k8 + q8.k_lo + q_lo.k8 (the residual tensors recover the e4m3 rounding of q and k).
+template <int DP, bool COMP>
 __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2))) dpa_mfma_fp8_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups) {
 	constexpr int NC       = DP / 16;       // contraction chunks of QK^T
 	constexpr int NDB      = DP / 32;       // 32-row blocks of O^T
-	constexpr int K_TILE   = KT8 * DP;      // bytes
+	constexpr int K_TILE1  = KT8 * DP;      // bytes of one K tile
+	constexpr int K_TILE   = K_TILE1 * (COMP ? 2 : 1);  // hi tile followed by the residual tile
 	constexpr int V_TILE   = DP * KT8;      // bytes: [DP rows d][64 keys]
-	constexpr int K_LOADS  = K_TILE / 1024; // 1 KB wave loads per K tile (2 or 4)
+	constexpr int K_LOADS  = K_TILE1 / 1024; // 1 KB wave loads per K tile (2 or 4)
 	constexpr int V_LOADS  = V_TILE / 1024;
 
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -128,6 +130,17 @@ __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2
 			qf[c] = __builtin_bit_cast(long, w);
 		}
 	}
+	long qlo[NC];
+	if(COMP) {
+		const uint8_t* qp = static_cast<const uint8_t*>(p.q_lo) + b * p.q_stride[0] + h * p.q_stride[1] + qrow * p.q_stride[2];
+#pragma unroll
+		for(int c = 0; c < NC; c++) {
+			const int d0 = 16 * c + 8 * half;
+			u32v2     w  = {0u, 0u};
+			if(row_ok && d0 < D && !all_dropped) w = *reinterpret_cast<const u32v2*>(qp + d0);
+			qlo[c] = __builtin_bit_cast(long, w);
+		}
+	}
 	// identity fragments scaled by 1/alpha (power of two times 1/softmax_scale folded by the caller: exact in bf16
 	// when alpha is a power of two)
 	bf16x8 idf[2];
@@ -158,6 +171,8 @@ __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2
 	// V^T: lane i of load j -> row d = j*16 + i/4, 16-byte chunk i%4 of the 64-key row
 	const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
 		const_cast<uint8_t*>(static_cast<const uint8_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1]), 0, (int)((L - 1) * p.k_stride[2] + (D + 15) / 16 * 16), 0x00020000);  // rows are fetched in 16-byte chunks
+	const __amdgpu_buffer_rsrc_t klo_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+		const_cast<uint8_t*>(static_cast<const uint8_t*>(COMP ? p.k_lo : p.k) + b * p.k_stride[0] + h * p.k_stride[1]), 0, (int)((L - 1) * p.k_stride[2] + (D + 15) / 16 * 16), 0x00020000);
 	const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
 		const_cast<uint8_t*>(static_cast<const uint8_t*>(p.v) + b * p.v_stride[0] + h * p.v_stride[1]), 0, (int)((D - 1) * p.v_stride[2] + p.v_stride[2]), 0x00020000);
 	constexpr int KCPR = DP / 16;       // 16-byte chunks per K row
@@ -171,9 +186,13 @@ __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2
 #pragma unroll
 		for(int t = 0; t < (K_LOADS + NW8 - 1) / NW8; t++) {
 			const int j = wave + NW8 * t;
-			if(j < K_LOADS && k_act)
+			if(j < K_LOADS && k_act) {
 				__builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (__attribute__((address_space(3))) void*)(k_lds + buf * K_TILE + j * 1024), 16, k_voff,
 														 (int)((kt * KT8 + j * KRPI) * p.k_stride[2]), 0, 0);
+				if(COMP)
+					__builtin_amdgcn_raw_ptr_buffer_load_lds(klo_rsrc, (__attribute__((address_space(3))) void*)(k_lds + buf * K_TILE + K_TILE1 + j * 1024), 16, k_voff,
+															 (int)((kt * KT8 + j * KRPI) * p.k_stride[2]), 0, 0);
+			}
 		}
 #pragma unroll
 		for(int t = 0; t < (V_LOADS + NW8 - 1) / NW8; t++) {
@@ -251,6 +270,11 @@ __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2
 			for(int c = 0; c < NC; c++) {
 				const long kf = *reinterpret_cast<const long*>(k_lds + buf * K_TILE + k_rd + sub * 32 * DP + 16 * c);
 				s = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(kf, qf[c], s, 0, 0, 0);
+				if(COMP) {
+					const long kl = *reinterpret_cast<const long*>(k_lds + buf * K_TILE + K_TILE1 + k_rd + sub * 32 * DP + 16 * c);
+					s = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(kl, qf[c], s, 0, 0, 0);
+					s = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(kf, qlo[c], s, 0, 0, 0);
+				}
 			}
 #pragma unroll
 			for(int c2 = 0; c2 < 2; c2++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(idf[c2], __builtin_bit_cast(bf16x8, bcur[2 * sub + c2]), s, 0, 0, 0);
@@ -323,15 +347,15 @@ __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2
 	}
 }
 
-template <int DP>
+template <int DP, bool COMP>
 int launch8(const af3_dpa_params& p, hipStream_t s) {
 	const int     n_qtiles = (int)((p.L + NW8 * 32 - 1) / (NW8 * 32));
 	const int     n_ktiles = (int)((p.L + KT8 - 1) / KT8);
 	const int64_t n_groups = p.B * p.H;
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
-	const size_t smem = (size_t)4 * KT8 * DP + ((size_t)n_ktiles * KT8 + 64) * 4 + (size_t)n_ktiles * 2 + 16;
-	hipLaunchKernelGGL(dpa_mfma_fp8_kernel<DP>, dim3((unsigned)blocks), dim3(NW8 * 64), smem, s, p, n_qtiles, n_groups);
+	const size_t smem = (size_t)(COMP ? 6 : 4) * KT8 * DP + ((size_t)n_ktiles * KT8 + 64) * 4 + (size_t)n_ktiles * 2 + 16;
+	hipLaunchKernelGGL((dpa_mfma_fp8_kernel<DP, COMP>), dim3((unsigned)blocks), dim3(NW8 * 64), smem, s, p, n_qtiles, n_groups);
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }
 
@@ -343,6 +367,8 @@ bool mfma_fp8_eligible(const af3_dpa_params& p) {
 	if(p.bias && p.bias_dtype != AF3_BF16) return false;
 	// q rows are read 8 bytes at a time, K / V^T rows in 16-byte chunks at 4-byte aligned offsets
 	if((reinterpret_cast<uintptr_t>(p.q) & 7) || (reinterpret_cast<uintptr_t>(p.k) & 3) || (reinterpret_cast<uintptr_t>(p.v) & 15)) return false;
+	if((p.q_lo != nullptr) != (p.k_lo != nullptr)) return false;  // both residuals or none
+	if((reinterpret_cast<uintptr_t>(p.q_lo) & 7) || (reinterpret_cast<uintptr_t>(p.k_lo) & 3)) return false;
 	for(int i = 0; i < 3; i++)
 		if(p.q_stride[i] % 8 || p.k_stride[i] % 4 || p.v_stride[i] % 16) return false;
 	if(p.L * p.k_stride[2] >= 0x7fffffffLL || p.D * p.v_stride[2] >= 0x7fffffffLL) return false;
@@ -354,6 +380,10 @@ bool mfma_fp8_eligible(const af3_dpa_params& p) {
 	return true;
 }
 
-int launch_dpa_mfma_fp8(const af3_dpa_params& p, hipStream_t s) { return p.D <= 32 ? launch8<32>(p, s) : launch8<64>(p, s); }
+int launch_dpa_mfma_fp8(const af3_dpa_params& p, hipStream_t s) {
+	const bool comp = p.q_lo != nullptr && p.k_lo != nullptr;
+	if(p.D <= 32) return comp ? launch8<32, true>(p, s) : launch8<32, false>(p, s);
+	return comp ? launch8<64, true>(p, s) : launch8<64, false>(p, s);
+}
 
 }  // namespace af3

@@ -81,17 +81,36 @@ __global__ void __launch_bounds__(EW_THREADS) cvt_e4m3_kernel(const uint8_t* __r
 }
 
 // ---- per-tensor amax -------------------------------------------------------------------------
+// 16-byte loads, wave then workgroup reduction, one atomic per workgroup (a few hundred atomics on
+// the one result word instead of one per wavefront).
 template <bool SRC_BF16>
 __global__ void __launch_bounds__(EW_THREADS) amax_kernel(const void* __restrict__ src, int64_t n, float* amax_out) {
-	const int64_t stride = (int64_t)gridDim.x * EW_THREADS;
-	float         a      = 0.f;
-	for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += stride) {
+	__shared__ float part[EW_THREADS / 64];
+	const int64_t stride = (int64_t)gridDim.x * EW_THREADS, tid0 = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x;
+	constexpr int PER  = SRC_BF16 ? 8 : 4;  // elements per 16-byte load
+	const bool    vec  = (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+	const int64_t nvec = vec ? n / PER : 0;
+	float         a    = 0.f;  // fmaxf drops NaN operands: a NaN element does not poison the scale
+	for(int64_t i = tid0; i < nvec; i += stride) {
+		const u32x4 w = static_cast<const u32x4*>(src)[i];
+#pragma unroll
+		for(int j = 0; j < 4; j++) {
+			if(SRC_BF16) a = fmaxf(a, fmaxf(fabsf(bf16_bits_to_f32(w[j] & 0xffffu)), fabsf(bf16_bits_to_f32(w[j] >> 16))));
+			else a = fmaxf(a, fabsf(__uint_as_float(w[j])));
+		}
+	}
+	for(int64_t i = nvec * PER + tid0; i < n; i += stride) {
 		const float f = SRC_BF16 ? bf16_bits_to_f32(static_cast<const uint16_t*>(src)[i]) : static_cast<const float*>(src)[i];
-		a = fmaxf(a, fabsf(f));  // fmaxf drops NaN operands: a NaN element does not poison the scale
+		a = fmaxf(a, fabsf(f));
 	}
 	for(int o = 32; o > 0; o >>= 1) a = fmaxf(a, __shfl_xor(a, o));
-	// non-negative floats order like their bit patterns
-	if((threadIdx.x & 63) == 0) atomicMax(reinterpret_cast<unsigned int*>(amax_out), __float_as_uint(a));
+	if((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = a;
+	__syncthreads();
+	if(threadIdx.x == 0) {
+		for(int w = 1; w < EW_THREADS / 64; w++) a = fmaxf(a, part[w]);
+		// non-negative floats order like their bit patterns
+		atomicMax(reinterpret_cast<unsigned int*>(amax_out), __float_as_uint(a));
+	}
 }
 
 // scale = 2^floor(log2(448 / (amax*pre_scale))); the power of two keeps every descale product exact.
@@ -108,7 +127,7 @@ __device__ __forceinline__ float fp8_pow2_scale(float amax, float pre_scale) {
 template <bool SRC_BF16>
 __global__ void __launch_bounds__(EW_THREADS) quantize_e4m3_kernel(const void* __restrict__ src, uint8_t* __restrict__ dst, int64_t rows, int64_t cols,
 																	 int64_t src_row_stride, int transpose, int64_t rows_per_matrix, int64_t dst_row_stride,
-																	 float pre_scale, const float* amax, float* descale_out) {
+																	 float pre_scale, const float* amax, float* descale_out, uint8_t* __restrict__ dst_lo) {
 	const float scale = fp8_pow2_scale(*amax, pre_scale);
 	if(blockIdx.x == 0 && threadIdx.x == 0 && descale_out) *descale_out = 1.f / scale;
 	const float   mul    = pre_scale * scale;
@@ -118,15 +137,25 @@ __global__ void __launch_bounds__(EW_THREADS) quantize_e4m3_kernel(const void* _
         const float   f = SRC_BF16 ? bf16_bits_to_f32(static_cast<const uint16_t*>(src)[i]) : static_cast<const float*>(src)[i];
         return fminf(fmaxf(f * mul, -448.f), 448.f);
 	};
+	// residual word: e4m3 of (scaled value - decoded hi), the rounding error of hi at the same scale
+	auto residual = [&](float f0, float f1, float f2, float f3, uint32_t hi) -> uint32_t {
+		const auto lo01 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), lo23 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+		uint32_t   w    = 0;
+		w = __builtin_amdgcn_cvt_pk_fp8_f32(f0 - lo01[0], f1 - lo01[1], w, false);
+		w = __builtin_amdgcn_cvt_pk_fp8_f32(f2 - lo23[0], f3 - lo23[1], w, true);
+		return w;
+	};
 	if(!transpose) {
 		// one thread = 4 consecutive columns of one row (cols % 4 == 0 is checked by the launcher)
 		const int64_t cq = cols >> 2, total = rows * cq;
 		for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += stride) {
 			const int64_t r = i / cq, c = (i % cq) << 2;
+			const float   f0 = ld(r, c), f1 = ld(r, c + 1), f2 = ld(r, c + 2), f3 = ld(r, c + 3);
 			uint32_t      w = 0;
-			w = __builtin_amdgcn_cvt_pk_fp8_f32(ld(r, c), ld(r, c + 1), w, false);
-			w = __builtin_amdgcn_cvt_pk_fp8_f32(ld(r, c + 2), ld(r, c + 3), w, true);
+			w = __builtin_amdgcn_cvt_pk_fp8_f32(f0, f1, w, false);
+			w = __builtin_amdgcn_cvt_pk_fp8_f32(f2, f3, w, true);
 			*reinterpret_cast<uint32_t*>(dst + r * dst_row_stride + c) = w;
+			if(dst_lo) *reinterpret_cast<uint32_t*>(dst_lo + r * dst_row_stride + c) = residual(f0, f1, f2, f3, w);
 		}
 	} else {
 		// one thread = 4 consecutive rows of one column, written as 4 consecutive bytes of dst[matrix][col][row..row+3]
@@ -143,6 +172,7 @@ __global__ void __launch_bounds__(EW_THREADS) quantize_e4m3_kernel(const void* _
 			w = __builtin_amdgcn_cvt_pk_fp8_f32(f0, f1, w, false);
 			w = __builtin_amdgcn_cvt_pk_fp8_f32(f2, f3, w, true);
 			*reinterpret_cast<uint32_t*>(dst + (mat * cols + c) * dst_row_stride + (r4 << 2)) = w;
+			if(dst_lo) *reinterpret_cast<uint32_t*>(dst_lo + (mat * cols + c) * dst_row_stride + (r4 << 2)) = residual(f0, f1, f2, f3, w);
 		}
 	}
 }
@@ -206,14 +236,15 @@ extern "C" int af3_amax(const void* src, int32_t sd, int64_t n, float* amax_out,
 	if(!amax_out || (n > 0 && !src)) return AF3_ERR_NULL_POINTER;
 	if(n == 0) return AF3_OK;
 	hipStream_t s = static_cast<hipStream_t>(stream);
-	if(sd == AF3_F32) hipLaunchKernelGGL(amax_kernel<false>, dim3(ew_blocks(n, 2048)), dim3(EW_THREADS), 0, s, src, n, amax_out);
-	else if(sd == AF3_BF16) hipLaunchKernelGGL(amax_kernel<true>, dim3(ew_blocks(n, 2048)), dim3(EW_THREADS), 0, s, src, n, amax_out);
+	if(sd == AF3_F32) hipLaunchKernelGGL(amax_kernel<false>, dim3(ew_blocks((n + 7) / 8, 512)), dim3(EW_THREADS), 0, s, src, n, amax_out);
+	else if(sd == AF3_BF16) hipLaunchKernelGGL(amax_kernel<true>, dim3(ew_blocks((n + 7) / 8, 512)), dim3(EW_THREADS), 0, s, src, n, amax_out);
 	else return AF3_ERR_BAD_DTYPE;
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }
 
 extern "C" int af3_quantize_fp8_e4m3(const void* src, int32_t sd, void* dst, int64_t rows, int64_t cols, int64_t src_row_stride, int32_t transpose_last2,
-									 int64_t rows_per_matrix, int64_t dst_row_stride, float pre_scale, const float* amax, float* descale_out, void* stream) {
+									 int64_t rows_per_matrix, int64_t dst_row_stride, float pre_scale, const float* amax, float* descale_out, void* dst_residual,
+									 void* stream) {
 	if(rows < 0 || cols < 0) return AF3_ERR_BAD_SHAPE;
 	if(!amax) return AF3_ERR_NULL_POINTER;
 	if(rows == 0 || cols == 0) return AF3_OK;
@@ -226,15 +257,15 @@ extern "C" int af3_quantize_fp8_e4m3(const void* src, int32_t sd, void* dst, int
 		if(cols % 4 != 0) return AF3_ERR_BAD_ARGUMENT;
 		if(dst_row_stride < cols || dst_row_stride % 4 != 0) return AF3_ERR_BAD_STRIDE;
 	}
-	if(reinterpret_cast<uintptr_t>(dst) & 3) return AF3_ERR_BAD_ARGUMENT;
+	if((reinterpret_cast<uintptr_t>(dst) & 3) || (reinterpret_cast<uintptr_t>(dst_residual) & 3)) return AF3_ERR_BAD_ARGUMENT;
 	hipStream_t    s = static_cast<hipStream_t>(stream);
 	const unsigned g = ew_blocks(rows * cols / 4);
 	if(sd == AF3_F32)
 		hipLaunchKernelGGL(quantize_e4m3_kernel<false>, dim3(g), dim3(EW_THREADS), 0, s, src, static_cast<uint8_t*>(dst), rows, cols, src_row_stride, (int)transpose_last2,
-						   rows_per_matrix, dst_row_stride, pre_scale, amax, descale_out);
+						   rows_per_matrix, dst_row_stride, pre_scale, amax, descale_out, static_cast<uint8_t*>(dst_residual));
 	else if(sd == AF3_BF16)
 		hipLaunchKernelGGL(quantize_e4m3_kernel<true>, dim3(g), dim3(EW_THREADS), 0, s, src, static_cast<uint8_t*>(dst), rows, cols, src_row_stride, (int)transpose_last2,
-						   rows_per_matrix, dst_row_stride, pre_scale, amax, descale_out);
+						   rows_per_matrix, dst_row_stride, pre_scale, amax, descale_out, static_cast<uint8_t*>(dst_residual));
 	else
 		return AF3_ERR_BAD_DTYPE;
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;

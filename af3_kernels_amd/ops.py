@@ -266,11 +266,13 @@ def convert(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
-def quantize_fp8_e4m3(x: torch.Tensor, pre_scale: float = 1.0, transpose_last2: bool = False, descale_out: Optional[torch.Tensor] = None):
+def quantize_fp8_e4m3(x: torch.Tensor, pre_scale: float = 1.0, transpose_last2: bool = False, descale_out: Optional[torch.Tensor] = None,
+                      with_residual: bool = False):
     """Per-tensor scaled quantisation to OCP e4m3: returns (fp8 tensor, descale) where descale is
     a 1-element device float and real ~= fp8 * descale.  The scale is the largest power of two
     that keeps amax * pre_scale <= 448.  With transpose_last2 the last two axes are swapped in
-    the output and the new innermost axis is padded to a multiple of 16 bytes."""
+    the output and the new innermost axis is padded to a multiple of 16 bytes.  With with_residual a third
+    value is returned: e4m3(x * pre_scale * scale - fp8), the rounding error at the same scale."""
     _require_device(x)
     if x.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("quantize_fp8_e4m3 takes float32 or bfloat16")
@@ -288,32 +290,44 @@ def quantize_fp8_e4m3(x: torch.Tensor, pre_scale: float = 1.0, transpose_last2: 
             lpad = (rows_per_matrix + 15) // 16 * 16
             full = torch.zeros(x.shape[:-2] + (cols, lpad), dtype=torch.float8_e4m3fn, device=x.device)
             out = full[..., :rows_per_matrix]
+            full_lo = torch.zeros_like(full) if with_residual else None
+            lo = full_lo[..., :rows_per_matrix] if with_residual else None
             _lib.check(lib.af3_quantize_fp8_e4m3(x.data_ptr(), _DTYPE_CODE[x.dtype], full.data_ptr(), rows, cols, cols, 1, rows_per_matrix, lpad,
-                                                 pre_scale, amax.data_ptr(), descale_out.data_ptr(), st), "af3_quantize_fp8_e4m3")
+                                                 pre_scale, amax.data_ptr(), descale_out.data_ptr(), full_lo.data_ptr() if with_residual else None, st),
+                       "af3_quantize_fp8_e4m3")
         else:
             # 16 bytes of slack behind the last row: the fp8 attention kernel fetches rows in 16-byte chunks
             flat = torch.zeros(x.numel() + 16, dtype=torch.uint8, device=x.device)
             out = flat[:x.numel()].view(torch.float8_e4m3fn).view(x.shape)
+            flat_lo = torch.zeros_like(flat) if with_residual else None
+            lo = flat_lo[:x.numel()].view(torch.float8_e4m3fn).view(x.shape) if with_residual else None
             _lib.check(lib.af3_quantize_fp8_e4m3(x.data_ptr(), _DTYPE_CODE[x.dtype], out.data_ptr(), rows, cols, cols, 0, 0, cols,
-                                                 pre_scale, amax.data_ptr(), descale_out.data_ptr(), st), "af3_quantize_fp8_e4m3")
-    return out, descale_out
+                                                 pre_scale, amax.data_ptr(), descale_out.data_ptr(), lo.data_ptr() if with_residual else None, st),
+                       "af3_quantize_fp8_e4m3")
+    return (out, descale_out, lo) if with_residual else (out, descale_out)
 
 
-def dot_product_attention_fp8(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+def dot_product_attention_fp8(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor, bias: torch.Tensor,
+                              compensated: bool = True) -> torch.Tensor:
     """Attention with both products on the e4m3 matrix cores (fp32 accumulation): q, k, v are
     quantised per tensor (q with D^-1/2 folded in, v written transposed), the bias stays bf16,
-    the output has q's dtype.  No reference counterpart (the reference has no fp8 path)."""
+    the output has q's dtype.  With `compensated` (default) q and k also carry their e4m3 rounding
+    residuals and the logits are q8.k8 + q8.k_lo + q_lo.k8 (three e4m3 MFMAs per chunk), which is
+    what keeps the result within 6e-2 of the fp32 formula; without it only q8.k8 is computed.
+    No reference counterpart (the reference has no fp8 path)."""
     _require_device(q, k, v, mask, bias)
     B, H, L, D = q.shape
     descales = torch.empty(3, dtype=torch.float32, device=q.device)
-    q8, _ = quantize_fp8_e4m3(q, pre_scale=float(D) ** -0.5, descale_out=descales[0:1])
-    k8, _ = quantize_fp8_e4m3(k, descale_out=descales[1:2])
+    q8, _, q_lo = quantize_fp8_e4m3(q, pre_scale=float(D) ** -0.5, descale_out=descales[0:1], with_residual=True)
+    k8, _, k_lo = quantize_fp8_e4m3(k, descale_out=descales[1:2], with_residual=True)
     v8t, _ = quantize_fp8_e4m3(v, transpose_last2=True, descale_out=descales[2:3])
     keep = _lift_mask(mask, L) if mask is not None else None
     bias = _inner_contig(bias.to(torch.bfloat16)) if bias is not None else None
     _check_shapes(q8, k8, v8t, keep, bias, v_transposed=True)
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     p = _fill_params(q8, k8, v8t, keep, bias, out, AF3_FP8_E4M3, False, descales=descales, softmax_scale=1.0)
+    if compensated:
+        p.q_lo, p.k_lo = q_lo.data_ptr(), k_lo.data_ptr()
     with torch.cuda.device(q.device):
         _lib.check(_lib.load().af3_dpa_forward(ctypes.byref(p), _stream_ptr(q.device)), "af3_dpa_forward(fp8)")
     return out

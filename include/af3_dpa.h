@@ -104,6 +104,12 @@ typedef struct af3_dpa_params {
 	 * without it (NULL) the bias is read in place.  Contents are overwritten by every call. */
 	void*          workspace;
 	int64_t        workspace_bytes;
+	/* Optional (fp8 only): residual tensors q_lo = e4m3(q*s - q8), k_lo = e4m3(k*s - k8) at the same
+	 * scale and with the same strides as q and k (af3_quantize_fp8_e4m3 writes them).  When both
+	 * are given the logits are q8.k8 + q8.k_lo + q_lo.k8: three e4m3 MFMAs per contraction chunk
+	 * that recover about six mantissa bits for q and k. */
+	const void*    q_lo;
+	const void*    k_lo;
 } af3_dpa_params;
 
 /*
@@ -150,11 +156,13 @@ int af3_amax(const void* src, int32_t src_dtype, int64_t n, float* amax_out, voi
  * row stride src_row_stride; with transpose_last2 != 0, every consecutive block of
  * `rows_per_matrix` rows is written transposed: dst[matrix][col][row], row stride
  * dst_row_stride (>= rows_per_matrix), so V [B*H*L, D] becomes [B*H, D, L].
+ * dst_residual (optional, same layout as dst): e4m3(src * pre_scale * scale - dst), the rounding
+ * error of dst at the same scale, for the compensated product of af3_dpa_forward.
  * No reference counterpart (see af3_amax).
  */
 int af3_quantize_fp8_e4m3(const void* src, int32_t src_dtype, void* dst, int64_t rows, int64_t cols, int64_t src_row_stride,
 						  int32_t transpose_last2, int64_t rows_per_matrix, int64_t dst_row_stride, float pre_scale, const float* amax,
-						  float* descale_out, void* hip_stream);
+						  float* descale_out, void* dst_residual, void* hip_stream);
 
 /*
  * N-dimensional pad (ndim <= AF3_PAD_MAX_DIMS): copy src (shape src_shape, element strides

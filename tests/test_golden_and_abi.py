@@ -59,9 +59,9 @@ def test_library_exports_every_declared_symbol():
 
 def test_params_struct_matches_header_layout():
     from af3_kernels_amd._lib import DpaParams
-    # 6 pointers, 4 dims, 4*3 + 2 + 1 strides (int64), 4 int32, 4 floats, 2 int32, 2 pointers, 1 int64
-    assert ctypes.sizeof(DpaParams) == 6 * 8 + 4 * 8 + 15 * 8 + 4 * 4 + 4 * 4 + 2 * 4 + 8 + 8 + 8
-    assert DpaParams.workspace_bytes.offset == ctypes.sizeof(DpaParams) - 8
+    # 6 pointers, 4 dims, 4*3 + 2 + 1 strides (int64), 4 int32, 4 floats, 2 int32, 2 pointers, 1 int64, 2 pointers
+    assert ctypes.sizeof(DpaParams) == 6 * 8 + 4 * 8 + 15 * 8 + 4 * 4 + 4 * 4 + 2 * 4 + 8 + 8 + 8 + 8 + 8
+    assert DpaParams.k_lo.offset == ctypes.sizeof(DpaParams) - 8
 
 
 def _params(**kw):
@@ -127,7 +127,7 @@ def test_elementwise_entry_points_validate_on_the_host():
     arr = ctypes.c_int64 * 2
     assert lib.af3_pad_nd(0x1000, 0x2000, 2, arr(4, 4), arr(4, 1), arr(2, 8), 4, 0, None) == -3   # shrinking
     assert lib.af3_pad_nd(0x1000, 0x2000, 9, arr(4, 4), arr(4, 1), arr(4, 8), 4, 0, None) == -3
-    assert lib.af3_quantize_fp8_e4m3(0x1000, 1, 0x2000, 8, 6, 6, 0, 0, 6, 1.0, 0x3000, None, None) == -7    # cols % 4
+    assert lib.af3_quantize_fp8_e4m3(0x1000, 1, 0x2000, 8, 6, 6, 0, 0, 6, 1.0, 0x3000, None, None, None) == -7    # cols % 4
 
 
 def test_wrapper_rejects_cpu_tensors_and_bad_shapes():

@@ -138,8 +138,10 @@ __global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restric
 
 // DP: head_dim padded to a multiple of 32 (32 or 64).  NW: wavefronts per workgroup.  L2DOM: log2
 // variant (bias from the workspace, or no bias at all).  BIAS_F32: bias stored as fp32 (natural
-// variant only).
-template <int DP, int NW, bool L2DOM, bool BIAS_F32>
+// variant only).  SPLIT: for launches too small to fill the chip -- the NW wavefronts of a workgroup
+// share ONE block of 32 query rows and split its key tiles round robin (each with private LDS
+// buffers, no barrier in the loop); their partial (O, m, l) are merged through LDS at the end.
+template <int DP, int NW, bool L2DOM, bool BIAS_F32, bool SPLIT>
 // (at least 2 wavefronts per SIMD: keeps the register budget at 256 so that the compiler writes MFMA
 // results to ordinary VGPRs instead of AGPRs, which every softmax operand would have to be copied out of)
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP == 32 ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups) {
@@ -149,14 +151,16 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	constexpr int TILE_BYTES = KT * DP * 2;
 	constexpr int NI         = TILE_BYTES / 1024;  // 1 KB wave loads per tile and tensor
 	constexpr int RPI        = 512 / DP;           // tile rows covered by one wave load
-	constexpr int QT         = NW * 32;
+	constexpr int QT         = SPLIT ? 32 : NW * 32;
+	constexpr int LDS_SETS   = SPLIT ? NW : 1;  // private K/V buffer sets
 	static_assert((2 * NI) % NW == 0 || NI % NW == 0, "tile loads must divide evenly over the wavefronts");
 
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 	// [K x3][V x3][mask table: (n_ktiles*64 + 64) dwords][live list]
-	unsigned char* const k_lds     = smem;
-	unsigned char* const v_lds     = smem + 3 * TILE_BYTES;
-	uint32_t* const      mask_tab  = reinterpret_cast<uint32_t*>(smem + 6 * TILE_BYTES);
+	const int            tid_pre   = threadIdx.x;
+	unsigned char* const k_lds     = smem + (SPLIT ? __builtin_amdgcn_readfirstlane(tid_pre >> 6) * 6 * TILE_BYTES : 0);
+	unsigned char* const v_lds     = k_lds + 3 * TILE_BYTES;
+	uint32_t* const      mask_tab  = reinterpret_cast<uint32_t*>(smem + LDS_SETS * 6 * TILE_BYTES);
 	const int            n_ktiles  = (int)((p.L + KT - 1) / KT);
 	int16_t* const       live_list = reinterpret_cast<int16_t*>(mask_tab + n_ktiles * KT + 64);
 	__shared__ int       s_nvalid, s_nlive;
@@ -182,7 +186,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	// ---- zero the K/V buffers: lanes of padded head columns never write them, and whatever a
 	// bounds-checked load leaves behind for rows past L must be finite (0 * stale NaN = NaN) ----
 	if(D != DP || L % KT != 0)
-		for(int i = tid; i < 6 * TILE_BYTES / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
+		for(int i = tid; i < LDS_SETS * 6 * TILE_BYTES / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
 	// ---- key-mask table and list of tiles with at least one live key ----
 	// entry = bf16 additive mask value in the low half (contraction slot 0) and, in the log2
 	// variant, 1.0 in the high half (slot 1, multiplies -m_ref); the last 64 entries are zero
@@ -228,7 +232,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	const bool all_dropped = __builtin_amdgcn_readfirstlane(s_nvalid) == 0;
 
 	// ---- per-lane constants ----
-	const int64_t qrow   = (int64_t)qtile * QT + wave * 32 + n;
+	const int64_t qrow   = (int64_t)qtile * QT + (SPLIT ? 0 : wave * 32) + n;
 	const bool    row_ok = qrow < L;
 
 	// Q fragments (B operand of S^T = K.Q^T): lane (q = n, g = half) holds q[q][16c + 8g .. +7]
@@ -278,7 +282,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	const u32x4* ws_wave = nullptr;
 	if(L2DOM && has_bias) {
 		const int     n_qblocks = (int)((L + 31) / 32);
-		const int64_t qb        = (int64_t)qtile * NW + wave;
+		const int64_t qb        = SPLIT ? (int64_t)qtile : (int64_t)qtile * NW + wave;
 		// query blocks beyond the last one only hold rows >= L; clamp so that loads stay in bounds
 		const int64_t qbc = qb < n_qblocks ? qb : n_qblocks - 1;
 		ws_wave = static_cast<const u32x4*>(p.workspace) + ((h * n_qblocks + qbc) * n_ktiles) * 256;
@@ -301,7 +305,18 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	const int  k_tile_stride = (int)(KT * p.k_stride[2] * 2), v_tile_stride = (int)(KT * p.v_stride[2] * 2);
 	const int  k_ld_stride   = (int)(RPI * p.k_stride[2] * 2), v_ld_stride = (int)(RPI * p.v_stride[2] * 2);
 	auto       load_tile     = [&](int kt, int buf) {
-		if(NW <= NI) {
+		if(SPLIT) {
+			// this wavefront fetches whole tiles into its private buffers
+#pragma unroll
+			for(int j = 0; j < NI; j++) {
+				if(k_act)
+					__builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (__attribute__((address_space(3))) void*)(k_lds + buf * TILE_BYTES + j * 1024), 16, k_voff,
+															 kt * k_tile_stride + j * k_ld_stride, 0, 0);
+				if(v_act)
+					__builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (__attribute__((address_space(3))) void*)(v_lds + buf * TILE_BYTES + j * 1024), 16, v_voff,
+															 kt * v_tile_stride + j * v_ld_stride, 0, 0);
+			}
+		} else if(NW <= NI) {
 #pragma unroll
 			for(int t = 0; t < NI / NW; t++) {
 				const int j = wave + NW * t;
@@ -377,7 +392,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		}
 	}
 	// mask table read address: lanes of the upper half-wave always read the zero entries
-	const int mask_rd     = (int)(6 * TILE_BYTES) + (half == 0 ? n * 4 : (n_ktiles * KT + n) * 4);
+	const int mask_rd     = (int)(LDS_SETS * 6 * TILE_BYTES) + (half == 0 ? n * 4 : (n_ktiles * KT + n) * 4);
 	const int mask_stride = half == 0 ? KT * 4 : 0;
 
 	// ---- online-softmax state (per lane: one query row; the two halves hold disjoint keys) ----
@@ -560,47 +575,52 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		pprev[1] = pcur[1];
 	};
 
-	// ---- prologue: first two tiles, first sub-tile's S^T and its row maximum ----
-	const int kt0 = __builtin_amdgcn_readfirstlane((int)live_list[0]);
-	__syncthreads();  // zero fill done
-	load_tile(kt0, 0);
-	if(nlive > 1) load_tile(__builtin_amdgcn_readfirstlane((int)live_list[1]), 1);
-#pragma unroll
-	for(int f = 0; f < 4; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
-	load_bias_frags(kt0, ic<0>{});
-	load_bias_frags(kt0, ic<1>{});
-	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-	__syncthreads();
-	sc = compute_s_plain(0, 0, mask_rd + kt0 * mask_stride, 0);
-	rereference(sc, nullptr, true);
-	if(nlive > 1) load_bias_frags(__builtin_amdgcn_readfirstlane((int)live_list[1]), ic<0>{});
+	// ---- which live tiles this wavefront walks: all of them, or every NW-th one when splitting ----
+	const int my_first = SPLIT ? wave : 0, my_step = SPLIT ? NW : 1;
+	const int my_n     = SPLIT ? (nlive > wave ? (nlive - wave + NW - 1) / NW : 0) : nlive;
+	auto live_at = [&](int j) -> int { return (int)live_list[my_first + (j < my_n ? j : my_n - 1) * my_step]; };
 
-	int buf = 0;  // LDS buffer of tile `it` (it % 3)
-	// tile indices of iterations it, it+1, it+2 are carried in scalar registers; the list entry for
-	// it+3 is fetched at the top of an iteration and only consumed at its end
-	auto live_at = [&](int i) -> int { return (int)live_list[i < nlive ? i : nlive - 1]; };
-	int kt = kt0, kt1 = __builtin_amdgcn_readfirstlane(live_at(1)), kt2 = __builtin_amdgcn_readfirstlane(live_at(2));
-	for(int it = 0; it < nlive; it++) {
-		const int kt3_v = live_at(it + 3);
-		const int bufn = buf == 2 ? 0 : buf + 1, bufnn = bufn == 2 ? 0 : bufn + 1;
-		// sub-tile (it, 0): next is (it, 1) in the same buffer
-		stage(ic<1>{}, buf * TILE_BYTES, mask_rd + kt * mask_stride, buf * TILE_BYTES, ic<0>{});
-		load_bias_frags(kt1, ic<1>{});
-		// Tile it+1 (issued one iteration ago) must have landed, and every wavefront must be done
-		// with tile it-1, whose buffer tile it+2 is about to overwrite.
-		// (vmcnt counts loads in issue order; in the log2 variant exactly four bias-fragment loads were
-		// issued after that tile's LDS-direct loads and may stay in flight)
-		if(L2DOM && has_bias) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-		else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-		__syncthreads();
-		if(it + 2 < nlive) load_tile(kt2, bufnn);
-		// sub-tile (it, 1): next is (it+1, 0) in the next buffer (harmless stale data after the last tile)
-		stage(ic<0>{}, bufn * TILE_BYTES, mask_rd + kt1 * mask_stride, buf * TILE_BYTES, ic<1>{});
-		load_bias_frags(kt2, ic<0>{});
-		buf = bufn;
-		kt  = kt1;
-		kt1 = kt2;
-		kt2 = __builtin_amdgcn_readfirstlane(kt3_v);
+	if(my_n > 0) {
+		// ---- prologue: first two tiles, first sub-tile's S^T and its row maximum ----
+		const int kt0 = __builtin_amdgcn_readfirstlane(live_at(0));
+		load_tile(kt0, 0);
+		if(my_n > 1) load_tile(__builtin_amdgcn_readfirstlane(live_at(1)), 1);
+#pragma unroll
+		for(int f = 0; f < 4; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
+		load_bias_frags(kt0, ic<0>{});
+		load_bias_frags(kt0, ic<1>{});
+		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+		if(!SPLIT) __syncthreads();
+		sc = compute_s_plain(0, 0, mask_rd + kt0 * mask_stride, 0);
+		rereference(sc, nullptr, true);
+		if(my_n > 1) load_bias_frags(__builtin_amdgcn_readfirstlane(live_at(1)), ic<0>{});
+
+		int buf = 0;  // LDS buffer of tile `it` (it % 3)
+		// tile indices of iterations it, it+1, it+2 are carried in scalar registers; the list entry for
+		// it+3 is fetched at the top of an iteration and only consumed at its end
+		int kt = kt0, kt1 = __builtin_amdgcn_readfirstlane(live_at(1)), kt2 = __builtin_amdgcn_readfirstlane(live_at(2));
+		for(int it = 0; it < my_n; it++) {
+			const int kt3_v = live_at(it + 3);
+			const int bufn = buf == 2 ? 0 : buf + 1, bufnn = bufn == 2 ? 0 : bufn + 1;
+			// sub-tile (it, 0): next is (it, 1) in the same buffer
+			stage(ic<1>{}, buf * TILE_BYTES, mask_rd + kt * mask_stride, buf * TILE_BYTES, ic<0>{});
+			load_bias_frags(kt1, ic<1>{});
+			// Tile it+1 (issued one iteration ago) must have landed, and every wavefront must be done
+			// with tile it-1, whose buffer tile it+2 is about to overwrite.
+			// (vmcnt counts loads in issue order; in the log2 variant exactly four bias-fragment loads were
+			// issued after that tile's LDS-direct loads and may stay in flight)
+			if(L2DOM && has_bias) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+			else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+			if(!SPLIT) __syncthreads();
+			if(it + 2 < my_n) load_tile(kt2, bufnn);
+			// sub-tile (it, 1): next is (it+1, 0) in the next buffer (harmless stale data after the last tile)
+			stage(ic<0>{}, bufn * TILE_BYTES, mask_rd + kt1 * mask_stride, buf * TILE_BYTES, ic<1>{});
+			load_bias_frags(kt2, ic<0>{});
+			buf = bufn;
+			kt  = kt1;
+			kt1 = kt2;
+			kt2 = __builtin_amdgcn_readfirstlane(kt3_v);
+		}
 	}
 	// the last sub-tile's PV product
 #pragma unroll
@@ -608,6 +628,44 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 #pragma unroll
 		for(int db = 0; db < NDB; db++)
 			oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[cp][db]), __builtin_bit_cast(bf16x8, pprev[cp]), oacc[db], 0, 0, 0);
+
+	if(SPLIT) {
+		// ---- merge the partial results of the NW wavefronts (same 32 query rows, disjoint keys) ----
+		asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+		__syncthreads();  // all K/V buffers are dead: reuse the front of LDS
+		float* const mred = reinterpret_cast<float*>(smem);        // [NW][32] reference maxima
+		float* const obuf = mred + NW * 32;                        // [NW][16*NDB + 1][64]
+		if(half == 0) mred[wave * 32 + n] = my_n > 0 ? m_ref : -INFINITY;
+		__syncthreads();
+		float mstar = mred[n];
+#pragma unroll
+		for(int w = 1; w < NW; w++) mstar = fmaxf(mstar, mred[w * 32 + n]);
+		const float scale_w = my_n > 0 ? __builtin_amdgcn_exp2f((m_ref - mstar) * (L2DOM ? 1.f : LOG2E)) : 0.f;
+		l_run *= scale_w;
+#pragma unroll
+		for(int db = 0; db < NDB; db++)
+#pragma unroll
+			for(int i = 0; i < 16; i++) oacc[db][i] *= scale_w;
+		if(wave > 0) {
+			float* mine = obuf + wave * (16 * NDB + 1) * 64 + lane;
+#pragma unroll
+			for(int db = 0; db < NDB; db++)
+#pragma unroll
+				for(int i = 0; i < 16; i++) mine[(db * 16 + i) * 64] = oacc[db][i];
+			mine[16 * NDB * 64] = l_run;
+		}
+		__syncthreads();
+		if(wave > 0) return;
+#pragma unroll
+		for(int w = 1; w < NW; w++) {
+			const float* theirs = obuf + w * (16 * NDB + 1) * 64 + lane;
+#pragma unroll
+			for(int db = 0; db < NDB; db++)
+#pragma unroll
+				for(int i = 0; i < 16; i++) oacc[db][i] += theirs[(db * 16 + i) * 64];
+			l_run += theirs[16 * NDB * 64];
+		}
+	}
 
 	// ---- epilogue: O^T register i of block db is head column 32*db + 8*(i/4) + 4*half + i%4 ----
 	const float l_tot = half_swap_sum(l_run);
@@ -662,16 +720,19 @@ int64_t mfma_bf16_workspace_bytes(const af3_dpa_params& p) {
 	return ws_bytes_needed(p);
 }
 
-template <int DP, int NW, bool L2DOM, bool BIAS_F32>
+template <int DP, int NW, bool L2DOM, bool BIAS_F32, bool SPLIT = false>
 static int launch_one(const af3_dpa_params& p, hipStream_t s) {
-	constexpr int QT       = NW * 32;
+	constexpr int QT       = SPLIT ? 32 : NW * 32;
 	const int     n_qtiles = (int)((p.L + QT - 1) / QT);
 	const int     n_ktiles = (int)((p.L + KT - 1) / KT);
 	const int64_t n_groups = p.B * p.H;
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
-	const size_t smem = (size_t)6 * KT * DP * 2 + ((size_t)n_ktiles * KT + 64) * 4 + (size_t)n_ktiles * 2 + 16;
-	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BIAS_F32>;
+	const size_t smem = (size_t)(SPLIT ? NW : 1) * 6 * KT * DP * 2 + ((size_t)n_ktiles * KT + 64) * 4 + (size_t)n_ktiles * 2 + 16;
+	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BIAS_F32, SPLIT>;
+	if(smem > 64 * 1024) {  // beyond the default dynamic-LDS limit: raise it for this kernel (idempotent, host side)
+		if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
+	}
 	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, n_qtiles, n_groups);
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }
@@ -682,6 +743,13 @@ static int launch_nw(const af3_dpa_params& p, hipStream_t s) {
 	const int64_t groups = p.B * p.H;
 	if(groups * ((p.L + 127) / 128) >= 768) return launch_one<DP, 4, L2DOM, BIAS_F32>(p, s);
 	if(groups * ((p.L + 63) / 64) >= 768) return launch_one<DP, 2, L2DOM, BIAS_F32>(p, s);
+	// Small launches: one 32-row block per workgroup, its key tiles split over 2 or 4 wavefronts so that
+	// more of the 1024 SIMDs have work.  The private LDS buffers limit a compute unit to one 4-wave or
+	// three 2-wave workgroups, so each split is only taken while the whole grid is resident at once
+	// (measured: beyond that the second round of workgroups costs more than the split gains).
+	const int64_t blocks1 = groups * ((p.L + 31) / 32), ktiles = (p.L + KT - 1) / KT;
+	if(DP == 32 && ktiles >= 4 && blocks1 <= 256) return launch_one<DP, 4, L2DOM, BIAS_F32, true>(p, s);
+	if(ktiles >= 2 && blocks1 <= (L2DOM ? 768 : 512)) return launch_one<DP, 2, L2DOM, BIAS_F32, true>(p, s);
 	return launch_one<DP, 1, L2DOM, BIAS_F32>(p, s);
 }
 

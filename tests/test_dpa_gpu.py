@@ -116,6 +116,30 @@ def test_bf16_mfma_matches_formula(af3, oracle, B, H, L, D, mask, rank):
     run_case(af3, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
 
 
+@pytest.mark.parametrize("B,H,L,D,live", [
+    (1, 2, 300, 24, None),     # 20 query blocks, 5 key tiles: four wavefronts share a block, one gets two tiles
+    (1, 2, 300, 32, 40),       # only the first tile is live: three of the four wavefronts have no tile at all
+    (1, 4, 520, 32, (260, 330)),  # live keys in the middle: tiles 4 and 5 only
+    (1, 2, 320, 64, None),     # head_dim 64: two wavefronts per block
+    (2, 2, 100, 32, None),     # two key tiles, bias through the fragment-ordered workspace
+    (1, 1, 2048, 32, None),    # 64 blocks x 32 tiles
+])
+def test_small_grids_split_keys_over_wavefronts(af3, oracle, B, H, L, D, live):
+    """Launches with few query blocks split each block's key tiles over the wavefronts of a workgroup
+    and merge the partial softmax states; every split must agree with the formula."""
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=3 * L + D)
+    if isinstance(live, int):
+        m[:, live:] = False
+    elif live is not None:
+        m[:] = False
+        m[:, live[0]:live[1]] = True
+    run_case(af3, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+    dq, dk, dv, dm, _ = dev(q, k, v, m, bias)
+    out = af3.dot_product_attention_cpp(dq, dk, dv, dm, torch.zeros(H, L, L, dtype=torch.bfloat16, device="cuda"))
+    want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), np.zeros((H, L, L), np.float32))
+    assert np.abs(f32np(out) - want).max() <= TOL[torch.bfloat16]
+
+
 def test_bf16_mfma_and_fp32_fma_kernels_agree(af3):
     q, k, v, m, bias = dev(*rand_inputs(2, 4, 200, 32, torch.bfloat16, seed=5, mask="random"))
     a = af3.dot_product_attention_cpp(q, k, v, m, bias)

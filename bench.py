@@ -19,6 +19,11 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "fp32": 157.3}   # MI355X dense matrix peaks
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the attention kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch) scaled by what the same counters read for a 256 MiB device copy
+# (FETCH x2.0, WRITE x1.0); the runs are summarised in profiles/dpa_mfma_bf16_cfg4_hbm_traffic.txt.
+# Counters cannot be read from inside this script, so workloads without such a run report null.
+MEASURED_TRAFFIC_BYTES = {"cfg4": 648.3e6}
 
 
 def cpu_baseline(case, budget_s=12.0):
@@ -139,6 +144,7 @@ def main():
                     "bias_stream_GBps": round(case.H * case.L * case.L * 2 / (kernel_ms * 1e-3) / 1e9, 1)}
     else:
         roofline = {"bound": "mfma", "achieved": round(k_tflops, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(k_tflops / peak, 4), "traffic": None}
+    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(case.name)
     roofline["kernel"] = kernel
     roofline["kernel_ms_avg"] = round(kernel_ms, 4)
     roofline["kernel_ms_median"] = round(per_launch[len(per_launch) // 2], 4)

@@ -53,6 +53,7 @@ namespace af3 {
 constexpr int   KT         = 64;       // keys per tile
 constexpr int   MAX_L_MFMA = 8192;     // mask table (4 B/key) and tile list live in LDS
 constexpr float REF_SLACK  = 12.f;     // log2 units: a moved reference sits this close to the row maximum
+constexpr bool  ROWSUM_MFMA = true;  // row sums of P on the matrix pipe instead of 16 vector adds per sub-tile
 constexpr float PSUM_LIMIT = 0x1p30f;  // per-lane row-sum bound that triggers the rare path
 
 typedef __attribute__((ext_vector_type(2))) __bf16   bf16x2;
@@ -287,6 +288,9 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		const int64_t qbc = qb < n_qblocks ? qb : n_qblocks - 1;
 		ws_wave = static_cast<const u32x4*>(p.workspace) + ((h * n_qblocks + qbc) * n_ktiles) * 256;
 	}
+	// (scalar base + per-lane 16-byte offset + scalar tile offset: no 64-bit pointer in vector registers)
+	const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(ws_wave), 0, ws_wave ? n_ktiles * 4096 : 0, 0x00020000);
+	const int                    ws_voff = lane * 16;
 
 	// ---- K/V tile loader: buffer loads that write LDS directly ----
 	// One wave load moves 1 KB: lane i -> LDS chunk i of the load's 1 KB window, i.e. tile row
@@ -343,14 +347,19 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	};
 
 	// bias fragments of one 64-key tile: [2*sub + c2]; loaded one sub-tile (two fragments) at a time
+	// Natural variant: four fragments in flight, each sub-tile's pair requested two stages before its
+	// use.  Log2 variant (BIAS_LATE): one pair only -- the registers are the scarce resource at four
+	// wavefronts per SIMD -- requested inside the previous stage, right after the matrix
+	// instructions that consume the pair before it.
+	constexpr bool BIAS_LATE = L2DOM;
 	u32x4 bfrag[4];
 	auto  load_bias_frags = [&](int kt, auto sub_c) {
 		constexpr int SUB = decltype(sub_c)::value;
 		if(!has_bias) return;
 		if(L2DOM) {
-			const u32x4* wp = ws_wave + (int64_t)kt * 256 + lane;
 #pragma unroll
-			for(int f = 2 * SUB; f < 2 * SUB + 2; f++) bfrag[f] = wp[f * 64];
+			for(int c2 = 0; c2 < 2; c2++)
+				bfrag[c2] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, ws_voff + (2 * SUB + c2) * 1024, kt * 4096, 0));
 			return;
 		}
 		const int64_t key0 = (int64_t)kt * KT + 8 * half;
@@ -399,6 +408,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	float  m_ref = 0.f;  // reference maximum: log2 units and bf16-exact (log2 variant), natural units (natural variant)
 	float  mc    = 0.f;  // natural variant: m_ref * log2 e
 	float  l_run = 0.f;
+	f32x4  lacc  = {0.f, 0.f, 0.f, 0.f};  // ROWSUM_MFMA: [0] = this lane's row sum (complete, same in both halves)
 	f32x16 oacc[NDB];
 #pragma unroll
 	for(int db = 0; db < NDB; db++)
@@ -436,6 +446,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			mc    = m_new * LOG2E;
 		}
 		l_run *= alpha;
+		lacc[0] *= alpha;
 #pragma unroll
 		for(int db = 0; db < NDB; db++)
 #pragma unroll
@@ -457,7 +468,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 				p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], LOG2E, -mc));
 				p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], LOG2E, -mc));
 			}
-			psum += p0 + p1;
+			if(!ROWSUM_MFMA) psum += p0 + p1;
 			pf[i >> 3][(i & 7) >> 1] = pack_bf16x2(p0, p1);
 		}
 	};
@@ -480,6 +491,22 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 #pragma unroll
 		for(int db = 0; db < NDB; db++) vprev[cp][db] = u32x4{0u, 0u, 0u, 0u};
 
+	// Row sums on the matrix pipe: a 16x16x32 MFMA whose A operand is a 0/1 pattern adds the 16 packed
+	// probabilities of a fragment (both half-waves) for every query; with this pattern register 0 of
+	// the result holds, in every lane, the sum for that lane's own query row.  As a B operand of the
+	// 16x16x32 shape the P fragment's lane l is column l%16, contraction group l/16, and holds query
+	// l%32: groups 0,2 belong to queries 0..15, groups 1,3 to queries 16..31.  Output register 0 of
+	// lane l is row 4*(l/16): rows 0 and 8 select the even groups, rows 4 and 12 the odd ones.
+	u32x4 ones_a;
+	{
+		const int  i16 = lane & 15, kg = lane >> 4;
+		const bool on  = ((i16 == 0 || i16 == 8) && (kg & 1) == 0) || ((i16 == 4 || i16 == 12) && (kg & 1) == 1);
+		const uint32_t w = on ? 0x3F803F80u : 0u;
+		ones_a = u32x4{w, w, w, w};
+	}
+	auto rowsum_mfma = [&](const u32x4& pf) {
+		lacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ones_a), __builtin_bit_cast(bf16x8, pf), lacc, 0, 0, 0);
+	};
 	auto read_kfrag = [&](int k_off, int sub, int c) -> u32x4 { return *reinterpret_cast<const u32x4*>(k_lds + k_rd[c] + k_off + sub * 32 * DP * 2); };
 	auto read_vfrags = [&](int v_off, int sub) {
 #pragma unroll
@@ -496,7 +523,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 				}
 	};
 	auto bias_mfma = [&](f32x16 s, int f) -> f32x16 {
-		if(L2DOM) return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, idf[f & 1]), __builtin_bit_cast(f16x8, bfrag[f]), s, 0, 0, 0);
+		if(L2DOM) return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, idf[f & 1]), __builtin_bit_cast(f16x8, bfrag[f & 1]), s, 0, 0, 0);
 		return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, idf[f & 1]), __builtin_bit_cast(bf16x8, bfrag[f]), s, 0, 0, 0);
 	};
 	// plain (not interleaved) S^T of one sub-tile; used once, for the very first sub-tile
@@ -512,7 +539,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), s, 0, 0, 0);
 	};
 
-	auto stage = [&](auto subn_c, int k_off, int mask_addr_next, int v_off, auto subc_c) {
+	auto stage = [&](auto subn_c, int k_off, int mask_addr_next, int v_off, auto subc_c, int bias_kt, auto bias_sub_c) {
 		constexpr int SUBN = decltype(subn_c)::value, SUBC = decltype(subc_c)::value, FB = 2 * SUBN;
 		// operands of S^T(j+1) from LDS
 		u32x4 kf[NC];
@@ -555,21 +582,37 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		// (the bias MFMAs run unconditionally -- on zero fragments when there is no bias -- so that the
 		// whole stage stays one basic block)
 		sn = bias_mfma(sn, FB);
+		const float l_before = lacc[0];
+		if(ROWSUM_MFMA) rowsum_mfma(pcur[0]);
 		exp_part(sc, pcur, psum, ic<8>{}, ic<2>{});
 		AF3_CHUNK_END();
 		sn = bias_mfma(sn, FB + 1);
 		exp_part(sc, pcur, psum, ic<10>{}, ic<2>{});
 		AF3_CHUNK_END();
+		if(BIAS_LATE) load_bias_frags(bias_kt, bias_sub_c);  // pair of the sub-tile after the next one
 		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), sn, 0, 0, 0);
 		exp_part(sc, pcur, psum, ic<12>{}, ic<4>{});
 		AF3_CHUNK_END();
 #undef AF3_CHUNK_END
-		if(__ballot(!(psum < PSUM_LIMIT))) {  // a logit far above the reference (or inf / NaN): rare
-			rereference(sc, &sn, false);
-			psum = 0.f;
-			exp_part(sc, pcur, psum, ic<0>{}, ic<16>{});
+		if(ROWSUM_MFMA) {
+			rowsum_mfma(pcur[1]);
+			// The running sum stays below L * 2^REF_SLACK <= 2^25 while every probability respects the
+			// reference, so this also catches a single probability near or beyond the limit (inf, NaN).
+			if(__ballot(!(lacc[0] < PSUM_LIMIT))) {  // rare
+				lacc[0] = l_before;
+				rereference(sc, &sn, false);
+				exp_part(sc, pcur, psum, ic<0>{}, ic<16>{});
+				rowsum_mfma(pcur[0]);
+				rowsum_mfma(pcur[1]);
+			}
+		} else {
+			if(__ballot(!(psum < PSUM_LIMIT))) {  // a logit far above the reference (or inf / NaN): rare
+				rereference(sc, &sn, false);
+				psum = 0.f;
+				exp_part(sc, pcur, psum, ic<0>{}, ic<16>{});
+			}
+			l_run += psum;
 		}
-		l_run += psum;
 		sc       = sn;
 		pprev[0] = pcur[0];
 		pprev[1] = pcur[1];
@@ -588,12 +631,13 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 #pragma unroll
 		for(int f = 0; f < 4; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
 		load_bias_frags(kt0, ic<0>{});
-		load_bias_frags(kt0, ic<1>{});
+		if(!BIAS_LATE) load_bias_frags(kt0, ic<1>{});
 		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 		if(!SPLIT) __syncthreads();
 		sc = compute_s_plain(0, 0, mask_rd + kt0 * mask_stride, 0);
 		rereference(sc, nullptr, true);
-		if(my_n > 1) load_bias_frags(__builtin_amdgcn_readfirstlane(live_at(1)), ic<0>{});
+		if(BIAS_LATE) load_bias_frags(kt0, ic<1>{});
+		else if(my_n > 1) load_bias_frags(__builtin_amdgcn_readfirstlane(live_at(1)), ic<0>{});
 
 		int buf = 0;  // LDS buffer of tile `it` (it % 3)
 		// tile indices of iterations it, it+1, it+2 are carried in scalar registers; the list entry for
@@ -603,8 +647,8 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			const int kt3_v = live_at(it + 3);
 			const int bufn = buf == 2 ? 0 : buf + 1, bufnn = bufn == 2 ? 0 : bufn + 1;
 			// sub-tile (it, 0): next is (it, 1) in the same buffer
-			stage(ic<1>{}, buf * TILE_BYTES, mask_rd + kt * mask_stride, buf * TILE_BYTES, ic<0>{});
-			load_bias_frags(kt1, ic<1>{});
+			stage(ic<1>{}, buf * TILE_BYTES, mask_rd + kt * mask_stride, buf * TILE_BYTES, ic<0>{}, kt1, ic<0>{});
+			if(!BIAS_LATE) load_bias_frags(kt1, ic<1>{});
 			// Tile it+1 (issued one iteration ago) must have landed, and every wavefront must be done
 			// with tile it-1, whose buffer tile it+2 is about to overwrite.
 			// (vmcnt counts loads in issue order; in the log2 variant exactly four bias-fragment loads were
@@ -614,8 +658,8 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			if(!SPLIT) __syncthreads();
 			if(it + 2 < my_n) load_tile(kt2, bufnn);
 			// sub-tile (it, 1): next is (it+1, 0) in the next buffer (harmless stale data after the last tile)
-			stage(ic<0>{}, bufn * TILE_BYTES, mask_rd + kt1 * mask_stride, buf * TILE_BYTES, ic<1>{});
-			load_bias_frags(kt2, ic<0>{});
+			stage(ic<0>{}, bufn * TILE_BYTES, mask_rd + kt1 * mask_stride, buf * TILE_BYTES, ic<1>{}, kt1, ic<1>{});
+			if(!BIAS_LATE) load_bias_frags(kt2, ic<0>{});
 			buf = bufn;
 			kt  = kt1;
 			kt1 = kt2;
@@ -642,6 +686,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		for(int w = 1; w < NW; w++) mstar = fmaxf(mstar, mred[w * 32 + n]);
 		const float scale_w = my_n > 0 ? __builtin_amdgcn_exp2f((m_ref - mstar) * (L2DOM ? 1.f : LOG2E)) : 0.f;
 		l_run *= scale_w;
+		lacc[0] *= scale_w;
 #pragma unroll
 		for(int db = 0; db < NDB; db++)
 #pragma unroll
@@ -652,7 +697,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			for(int db = 0; db < NDB; db++)
 #pragma unroll
 				for(int i = 0; i < 16; i++) mine[(db * 16 + i) * 64] = oacc[db][i];
-			mine[16 * NDB * 64] = l_run;
+			mine[16 * NDB * 64] = ROWSUM_MFMA ? lacc[0] : l_run;
 		}
 		__syncthreads();
 		if(wave > 0) return;
@@ -664,11 +709,12 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 #pragma unroll
 				for(int i = 0; i < 16; i++) oacc[db][i] += theirs[(db * 16 + i) * 64];
 			l_run += theirs[16 * NDB * 64];
+			lacc[0] += theirs[16 * NDB * 64];
 		}
 	}
 
 	// ---- epilogue: O^T register i of block db is head column 32*db + 8*(i/4) + 4*half + i%4 ----
-	const float l_tot = half_swap_sum(l_run);
+	const float l_tot = ROWSUM_MFMA ? lacc[0] : half_swap_sum(l_run);
 	const float inv   = 1.f / l_tot;
 	if(row_ok) {
 		const int64_t ooff = b * p.out_stride[0] + h * p.out_stride[1] + qrow * p.out_stride[2];

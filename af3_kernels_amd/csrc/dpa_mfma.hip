@@ -264,11 +264,14 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		if(j >= 0 && j < 8) v[j >> 1] = (L2DOM ? 0x3C00u : 0x3F80u) << ((j & 1) * 16);
 		idf[c2] = v;
 	}
-	// B operand of the mask MFMA: slot 0 = 1.0 (multiplies the key's mask value), slot 1 = -m_ref
-	// (log2 variant; multiplies the 1.0 every key carries in slot 1 of A).
+	// B operand of the mask MFMA: slot 0 = 1.0 (multiplies the key's mask value); log2 variant: slots 1
+	// and 2 = the reference maximum as -(m_hi + m_lo), two bf16 terms (16 significant bits, so that a
+	// reference of large magnitude -- a row whose biases are all hugely negative -- is still subtracted
+	// to within a fraction of a unit), multiplying the 1.0 that every key carries in slots 1 and 2 of A.
 	u32x4 maskB = {0u, 0u, 0u, 0u};
 	if(half == 0) maskB[0] = 0x3F80u;
 	u32x4 maskA = {0u, 0u, 0u, 0u};
+	if(L2DOM && half == 0) maskA[1] = 0x3F80u;  // slot 2; slots 0 and 1 come from the mask table
 
 	const bool has_bias = p.bias != nullptr && !all_dropped;
 	// natural variant: direct bias access through per-lane row pointers
@@ -427,8 +430,11 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		if(L2DOM) {
 			// s already has m_ref subtracted (by the mask MFMA)
 			const bool  need  = force || mx > REF_SLACK;
-			const float m_new = need ? bf16_bits_to_f32(f32_to_bf16_bits(m_ref + mx)) : m_ref;
-			const float delta = m_new - m_ref;                      // exact: both are bf16 values
+			const float m_want = m_ref + mx;
+			const float m_hi   = bf16_bits_to_f32(f32_to_bf16_bits(need ? m_want : m_ref));
+			const float m_lo   = bf16_bits_to_f32(f32_to_bf16_bits((need ? m_want : m_ref) - m_hi));
+			const float m_new  = m_hi + m_lo;  // exactly what the mask MFMA will subtract (unchanged when !need)
+			const float delta  = m_new - m_ref;
 			alpha = force ? 1.f : __builtin_amdgcn_exp2f(-delta);  // nothing is accumulated yet when forced (first sub-tile)
 #pragma unroll
 			for(int i = 0; i < 16; i++) s[i] -= delta;
@@ -437,7 +443,10 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 				for(int i = 0; i < 16; i++) (*pending)[i] -= delta;
 			}
 			m_ref = m_new;
-			if(half == 0) maskB[0] = 0x3F80u | (f32_to_bf16_bits(-m_new) << 16);
+			if(half == 0) {
+				maskB[0] = 0x3F80u | (f32_to_bf16_bits(-m_hi) << 16);
+				maskB[1] = f32_to_bf16_bits(-m_lo);
+			}
 		} else {
 			const bool  need  = force || mx > m_ref + REF_SLACK * 0.6931472f;
 			const float m_new = need ? mx : m_ref;

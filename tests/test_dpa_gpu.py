@@ -225,6 +225,52 @@ def test_fp32_bias_and_other_dtypes_are_cast_like_the_reference(af3, oracle):
     assert out.dtype == torch.bfloat16 and np.abs(f32np(out) - want).max() <= 2e-2
 
 
+@pytest.mark.parametrize("B,H,L,D", [(1, 1, 1, 8), (2, 3, 1, 32), (1, 5, 33, 8), (3, 7, 129, 40), (1, 1, 64, 64)])
+def test_tiny_and_odd_shapes(af3, oracle, B, H, L, D):
+    """L = 1 (softmax of one key), head_dim 8, odd head counts, lengths one past a tile edge."""
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=7 * L + D, mask="none")
+    run_case(af3, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+
+
+def test_logits_far_above_the_first_tile_move_the_reference(af3, oracle):
+    """The matrix-core kernel fixes its softmax reference from the first 32 keys of a row and only
+    moves it when a later logit exceeds it by a wide margin.  Rows whose large logits come late (and
+    grow from tile to tile) must take that path and still match the formula."""
+    B, H, L, D = 2, 2, 512, 32
+    q, k, v, m, bias0 = rand_inputs(B, H, L, D, torch.bfloat16, seed=99)
+    # B >= 2: bias through the fp16 log2-domain workspace, whose rounding error grows with |bias|
+    # (2^-12 * |bias| * log2 e in the logit), so this case keeps |bias| moderate: +20 across the row
+    # (29 in log2 units, two to three reference moves at a margin of 12), an isolated spike, and one
+    # row of hugely negative but equal biases (reference of large magnitude, 16-bit subtraction).
+    bias = (bias0.float() + torch.linspace(-8.0, 12.0, L)[None, None, :]).to(torch.bfloat16)
+    bias[:, 5, 300] = 40.0
+    bias[:, 7, :] = -3.0e4
+    run_case(af3, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+    # B = 1: bias read in place (exact), natural-domain reference in fp32: +100 across the row and a spike of 120
+    bias = (bias0.float() + torch.linspace(-40.0, 60.0, L)[None, None, :]).to(torch.bfloat16)
+    bias[:, 5, 300] = 120.0
+    bias[:, 7, :] = -3.0e4
+    bias[:, 9, :40] = -1.0e9          # masking expressed through the bias: the first tile of the row is dead
+    run_case(af3, oracle, q[:1], k[:1], v[:1], m[:1], bias, expect_kernel="bf16_mfma")
+
+
+def test_length_beyond_the_matrix_core_limit_uses_the_fma_kernel(af3):
+    """L > 8192 is outside the matrix-core kernel's mask table; the call must still work (fp32-FMA
+    kernel) -- checked through rows summing to one and against a torch reference on a slice."""
+    B, H, L, D = 1, 1, 8200, 32
+    g = torch.Generator().manual_seed(1)
+    q, k, v = [torch.randn(B, H, L, D, generator=g).to(torch.bfloat16).cuda() for _ in range(3)]
+    bias = torch.zeros(H, L, L, dtype=torch.bfloat16, device="cuda")
+    m = torch.ones(B, L, dtype=torch.bool, device="cuda")
+    m[:, 8000:] = False
+    assert af3.selected_kernel(q, k, v, m, bias) == "fp32_fma"
+    out = af3.dot_product_attention_cpp(q, k, v, m, bias)
+    s = (q[0, 0, :64].float() * D ** -0.5) @ k[0, 0].float().T
+    s[:, 8000:] = -1e9
+    want = torch.softmax(s, -1) @ v[0, 0].float()
+    assert (out[0, 0, :64].float() - want).abs().max().item() <= 2e-2
+
+
 # ---- the benchmark configurations at their real sizes ---------------------------------------
 
 @pytest.mark.parametrize("name,sample_rows", [("cfg2", [0, 191, 383]), ("cfg3", [0]), ("cfg4", [0, 400, 767])])

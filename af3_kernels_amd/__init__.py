@@ -19,11 +19,12 @@ from .ops import (  # noqa: F401
     quantize_fp8_e4m3,
     reset_debug_timers,
     selected_kernel,
+    set_exact_bias,
     vnni_repack_tensor,
 )
 
 __all__ = [
     "dot_product_attention_cpp", "dot_product_attention_fp8", "pad_and_align_tensor", "vnni_repack_tensor",
     "reset_debug_timers", "print_debug_timers", "print_debug_thread_imbalance", "convert", "quantize_fp8_e4m3",
-    "selected_kernel",
+    "selected_kernel", "set_exact_bias",
 ]

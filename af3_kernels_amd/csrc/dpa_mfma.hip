@@ -137,6 +137,24 @@ __global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restric
 	}
 }
 
+// 16 bytes per lane from a raw buffer straight into LDS (lane i lands at lds_addr + 16*i).  Written as
+// inline assembly on purpose: the compiler makes every LDS read that follows an LDS-direct load it
+// knows about wait for vmcnt(0), which exposes the whole latency of every tile load when only one or
+// two wavefronts share a SIMD.  Loads issued here are invisible to it; the kernel orders them itself
+// (explicit s_waitcnt vmcnt before the barrier that publishes a tile).  rsrc, lds_addr and soff
+// must be wave-uniform.
+__device__ __forceinline__ void lds_dma_b128(const u32x4& rsrc, uint32_t lds_addr, int voff, int soff) {
+	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
+}
+__device__ __forceinline__ u32x4 raw_rsrc(const void* base, uint32_t bytes) {
+	const uint64_t a = reinterpret_cast<uint64_t>(base);
+	return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a), (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xFFFFu)),
+				 (uint32_t)__builtin_amdgcn_readfirstlane((int)bytes), 0x00020000u};
+}
+__device__ __forceinline__ uint32_t lds_addr_of(const void* ptr) {
+	return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const void*)ptr);
+}
+
 // DP: head_dim padded to a multiple of 32 (32 or 64).  NW: wavefronts per workgroup.  L2DOM: log2
 // variant (bias from the workspace, or no bias at all).  BIAS_F32: bias stored as fp32 (natural
 // variant only).  SPLIT: for launches too small to fill the chip -- the NW wavefronts of a workgroup
@@ -154,7 +172,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	constexpr int RPI        = 512 / DP;           // tile rows covered by one wave load
 	constexpr int QT         = SPLIT ? 32 : NW * 32;
 	constexpr int LDS_SETS   = SPLIT ? NW : 1;  // private K/V buffer sets
-	static_assert((2 * NI) % NW == 0 || NI % NW == 0, "tile loads must divide evenly over the wavefronts");
+	static_assert(NW <= NI, "every wavefront fetches a whole number of 1 KB pieces of each tile");
 
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 	// [K x3][V x3][mask table: (n_ktiles*64 + 64) dwords][live list]
@@ -299,10 +317,8 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	// One wave load moves 1 KB: lane i -> LDS chunk i of the load's 1 KB window, i.e. tile row
 	// j*RPI + i/CPR, physical chunk i%CPR.  The lane picks the global chunk that belongs there
 	// under the swizzle; lanes of padded head columns (chunk*8 >= D) stay idle.
-	const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-		const_cast<uint16_t*>(static_cast<const uint16_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1]), 0, (int)(((L - 1) * p.k_stride[2] + D) * 2), 0x00020000);
-	const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-		const_cast<uint16_t*>(static_cast<const uint16_t*>(p.v) + b * p.v_stride[0] + h * p.v_stride[1]), 0, (int)(((L - 1) * p.v_stride[2] + D) * 2), 0x00020000);
+	const u32x4 k_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1], (uint32_t)(((L - 1) * p.k_stride[2] + D) * 2));
+	const u32x4 v_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.v) + b * p.v_stride[0] + h * p.v_stride[1], (uint32_t)(((L - 1) * p.v_stride[2] + D) * 2));
 	const int  ld_row  = lane / CPR, ld_pc = lane % CPR;
 	const int  k_chunk = ld_pc ^ k_swizzle<DP>(ld_row);
 	const int  v_chunk = ld_pc ^ v_swizzle<DP>(ld_row);
@@ -311,45 +327,16 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	const bool k_act   = k_chunk * 8 < D, v_act = v_chunk * 8 < D;
 	const int  k_tile_stride = (int)(KT * p.k_stride[2] * 2), v_tile_stride = (int)(KT * p.v_stride[2] * 2);
 	const int  k_ld_stride   = (int)(RPI * p.k_stride[2] * 2), v_ld_stride = (int)(RPI * p.v_stride[2] * 2);
-	auto       load_tile     = [&](int kt, int buf) {
-		if(SPLIT) {
-			// this wavefront fetches whole tiles into its private buffers
+	const uint32_t k_lds_addr = lds_addr_of(k_lds), v_lds_addr = lds_addr_of(v_lds);
+	auto load_tile = [&](int kt, int buf) {
 #pragma unroll
-			for(int j = 0; j < NI; j++) {
-				if(k_act)
-					__builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (__attribute__((address_space(3))) void*)(k_lds + buf * TILE_BYTES + j * 1024), 16, k_voff,
-															 kt * k_tile_stride + j * k_ld_stride, 0, 0);
-				if(v_act)
-					__builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (__attribute__((address_space(3))) void*)(v_lds + buf * TILE_BYTES + j * 1024), 16, v_voff,
-															 kt * v_tile_stride + j * v_ld_stride, 0, 0);
-			}
-		} else if(NW <= NI) {
-#pragma unroll
-			for(int t = 0; t < NI / NW; t++) {
-				const int j = wave + NW * t;
-				if(k_act)
-					__builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (__attribute__((address_space(3))) void*)(k_lds + buf * TILE_BYTES + j * 1024), 16, k_voff,
-															 kt * k_tile_stride + j * k_ld_stride, 0, 0);
-				if(v_act)
-					__builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (__attribute__((address_space(3))) void*)(v_lds + buf * TILE_BYTES + j * 1024), 16, v_voff,
-															 kt * v_tile_stride + j * v_ld_stride, 0, 0);
-			}
-		} else {
-			// more wavefronts than 1 KB pieces per tensor: the first NI wavefronts fetch K, the next NI fetch V
-			if(wave < NI) {
-				if(k_act)
-					__builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (__attribute__((address_space(3))) void*)(k_lds + buf * TILE_BYTES + wave * 1024), 16, k_voff,
-															 kt * k_tile_stride + wave * k_ld_stride, 0, 0);
-			} else if(wave < 2 * NI) {
-				const int j = wave - NI;
-				if(v_act)
-					__builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (__attribute__((address_space(3))) void*)(v_lds + buf * TILE_BYTES + j * 1024), 16, v_voff,
-															 kt * v_tile_stride + j * v_ld_stride, 0, 0);
-			}
+		for(int t = 0; t < (SPLIT ? NI : NI / NW); t++) {
+			const int j = SPLIT ? t : wave + NW * t;  // split: this wavefront fetches whole tiles into its private buffers
+			if(k_act) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + j * 1024, k_voff, kt * k_tile_stride + j * k_ld_stride);
+			if(v_act) lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + j * 1024, v_voff, kt * v_tile_stride + j * v_ld_stride);
 		}
 	};
 
-	// bias fragments of one 64-key tile: [2*sub + c2]; loaded one sub-tile (two fragments) at a time
 	// Natural variant: four fragments in flight, each sub-tile's pair requested two stages before its
 	// use.  Log2 variant (BIAS_LATE): one pair only -- the registers are the scarce resource at four
 	// wavefronts per SIMD -- requested inside the previous stage, right after the matrix
@@ -659,10 +646,10 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			stage(ic<1>{}, buf * TILE_BYTES, mask_rd + kt * mask_stride, buf * TILE_BYTES, ic<0>{}, kt1, ic<0>{});
 			if(!BIAS_LATE) load_bias_frags(kt1, ic<1>{});
 			// Tile it+1 (issued one iteration ago) must have landed, and every wavefront must be done
-			// with tile it-1, whose buffer tile it+2 is about to overwrite.
-			// (vmcnt counts loads in issue order; in the log2 variant exactly four bias-fragment loads were
-			// issued after that tile's LDS-direct loads and may stay in flight)
-			if(L2DOM && has_bias) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+			// with tile it-1, whose buffer tile it+2 is about to overwrite.  Loads complete in issue
+			// order; the only loads this wavefront has issued since that tile are bias fragments: two in
+			// the log2 variant (the pair requested inside the stage above), which may stay in flight.
+			if(L2DOM && has_bias) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
 			else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 			if(!SPLIT) __syncthreads();
 			if(it + 2 < my_n) load_tile(kt2, bufnn);

@@ -134,6 +134,19 @@ def _check_shapes(q, k, v, keep, bias, v_transposed=False):
             raise ValueError(f"mask must be [L] or [B, L] with B={B}, L={L}, got {tuple(keep.shape)}")
 
 
+_exact_bias = False
+
+
+def set_exact_bias(flag: bool) -> bool:
+    """With True, batched bf16 calls read the bias in place and add it exactly instead of going
+    through the kernel's fp16 log2-domain bias workspace (whose rounding error in a logit is at most
+    2^-12 * |bias| * log2 e: irrelevant for pair biases of ordinary size, 2 % of a softmax weight
+    at |bias| = 40).  Slower for B >= 2.  Returns the previous setting."""
+    global _exact_bias
+    prev, _exact_bias = _exact_bias, bool(flag)
+    return prev
+
+
 def _dpa_forward_impl(q, k, v, keep, bias, mma_dtype: int, force_generic: bool) -> torch.Tensor:
     _require_device(q, k, v, keep, bias)
     q, k, v = _inner_contig(q), _inner_contig(k), _inner_contig(v)
@@ -148,7 +161,7 @@ def _dpa_forward_impl(q, k, v, keep, bias, mma_dtype: int, force_generic: bool) 
     p = _fill_params(q, k, v, keep, bias, out, mma_dtype, force_generic)
     lib = _lib.load()
     ws_bytes = lib.af3_dpa_workspace_bytes(ctypes.byref(p))
-    if ws_bytes > 0:
+    if ws_bytes > 0 and not _exact_bias:
         # scratch for the kernel's bias rewrite; torch's caching allocator makes this a pointer bump
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
         p.workspace, p.workspace_bytes = ws.data_ptr(), ws_bytes

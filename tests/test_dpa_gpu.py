@@ -252,6 +252,12 @@ def test_logits_far_above_the_first_tile_move_the_reference(af3, oracle):
     bias[:, 7, :] = -3.0e4
     bias[:, 9, :40] = -1.0e9          # masking expressed through the bias: the first tile of the row is dead
     run_case(af3, oracle, q[:1], k[:1], v[:1], m[:1], bias, expect_kernel="bf16_mfma")
+    # the same large biases with a batch: exact when the caller asks for the in-place bias
+    prev = af3.set_exact_bias(True)
+    try:
+        run_case(af3, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+    finally:
+        af3.set_exact_bias(prev)
 
 
 def test_length_beyond_the_matrix_core_limit_uses_the_fma_kernel(af3):

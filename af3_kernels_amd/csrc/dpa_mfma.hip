@@ -141,10 +141,11 @@ __global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restric
 // inline assembly on purpose: the compiler makes every LDS read that follows an LDS-direct load it
 // knows about wait for vmcnt(0), which exposes the whole latency of every tile load when only one or
 // two wavefronts share a SIMD.  Loads issued here are invisible to it; the kernel orders them itself
-// (explicit s_waitcnt vmcnt before the barrier that publishes a tile).  rsrc, lds_addr and soff
-// must be wave-uniform.
-__device__ __forceinline__ void lds_dma_b128(const u32x4& rsrc, uint32_t lds_addr, int voff, int soff) {
-	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
+// (explicit s_waitcnt vmcnt before the barrier that publishes a tile).  rsrc and lds_addr must be
+// wave-uniform.  The whole byte offset travels in the vector operand, which the hardware range-checks
+// against the buffer size: a lane whose offset is past the end fetches nothing from memory.
+__device__ __forceinline__ void lds_dma_b128(const u32x4& rsrc, uint32_t lds_addr, int voff) {
+	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc) : "memory", "m0");
 }
 __device__ __forceinline__ u32x4 raw_rsrc(const void* base, uint32_t bytes) {
 	const uint64_t a = reinterpret_cast<uint64_t>(base);
@@ -160,10 +161,11 @@ __device__ __forceinline__ uint32_t lds_addr_of(const void* ptr) {
 // variant only).  SPLIT: for launches too small to fill the chip -- the NW wavefronts of a workgroup
 // share ONE block of 32 query rows and split its key tiles round robin (each with private LDS
 // buffers, no barrier in the loop); their partial (O, m, l) are merged through LDS at the end.
-template <int DP, int NW, bool L2DOM, bool BIAS_F32, bool SPLIT>
+template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT>
 // (at least 2 wavefronts per SIMD: keeps the register budget at 256 so that the compiler writes MFMA
-// results to ordinary VGPRs instead of AGPRs, which every softmax operand would have to be copied out of)
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP == 32 ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups) {
+// results to ordinary VGPRs instead of AGPRs, which every softmax operand would have to be copied out of;
+// the key-split variants are limited to fewer than 2 wavefronts per SIMD by their LDS buffers anyway)
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP == 32 && !SPLIT ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups) {
 	constexpr int NC         = DP / 16;            // contraction chunks of QK^T
 	constexpr int NDB        = DP / 32;            // 32-row blocks of O^T
 	constexpr int CPR        = DP / 8;             // 16-byte chunks per K/V row
@@ -171,15 +173,20 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	constexpr int NI         = TILE_BYTES / 1024;  // 1 KB wave loads per tile and tensor
 	constexpr int RPI        = 512 / DP;           // tile rows covered by one wave load
 	constexpr int QT         = SPLIT ? 32 : NW * 32;
-	constexpr int LDS_SETS   = SPLIT ? NW : 1;  // private K/V buffer sets
+	constexpr int  LDS_SETS   = SPLIT ? NW : 1;  // private K/V buffer sets
+	constexpr bool BIAS_F32   = BMODE == 1;      // natural variant, bias stored as fp32, read in place
+	constexpr bool BRING      = BMODE == 2;      // natural variant, bf16 bias streamed through a per-wavefront LDS ring
+	constexpr int  RING_BYTES = BRING ? NW * 3 * 4096 : 0;
+	constexpr int  MASK_BASE  = LDS_SETS * 6 * TILE_BYTES + RING_BYTES;
+	static_assert(!(L2DOM && BMODE != 0), "the log2 variant reads its bias from the workspace");
 	static_assert(NW <= NI, "every wavefront fetches a whole number of 1 KB pieces of each tile");
 
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-	// [K x3][V x3][mask table: (n_ktiles*64 + 64) dwords][live list]
+	// [K x3][V x3][bias ring: 3 x 4 KB per wavefront (BRING)][mask table: (n_ktiles*64 + 64) dwords][live list]
 	const int            tid_pre   = threadIdx.x;
 	unsigned char* const k_lds     = smem + (SPLIT ? __builtin_amdgcn_readfirstlane(tid_pre >> 6) * 6 * TILE_BYTES : 0);
 	unsigned char* const v_lds     = k_lds + 3 * TILE_BYTES;
-	uint32_t* const      mask_tab  = reinterpret_cast<uint32_t*>(smem + LDS_SETS * 6 * TILE_BYTES);
+	uint32_t* const      mask_tab  = reinterpret_cast<uint32_t*>(smem + MASK_BASE);
 	const int            n_ktiles  = (int)((p.L + KT - 1) / KT);
 	int16_t* const       live_list = reinterpret_cast<int16_t*>(mask_tab + n_ktiles * KT + 64);
 	__shared__ int       s_nvalid, s_nlive;
@@ -205,7 +212,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	// ---- zero the K/V buffers: lanes of padded head columns never write them, and whatever a
 	// bounds-checked load leaves behind for rows past L must be finite (0 * stale NaN = NaN) ----
 	if(D != DP || L % KT != 0)
-		for(int i = tid; i < LDS_SETS * 6 * TILE_BYTES / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
+		for(int i = tid; i < (LDS_SETS * 6 * TILE_BYTES + RING_BYTES) / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
 	// ---- key-mask table and list of tiles with at least one live key ----
 	// entry = bf16 additive mask value in the low half (contraction slot 0) and, in the log2
 	// variant, 1.0 in the high half (slot 1, multiplies -m_ref); the last 64 entries are zero
@@ -332,10 +339,34 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 #pragma unroll
 		for(int t = 0; t < (SPLIT ? NI : NI / NW); t++) {
 			const int j = SPLIT ? t : wave + NW * t;  // split: this wavefront fetches whole tiles into its private buffers
-			if(k_act) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + j * 1024, k_voff, kt * k_tile_stride + j * k_ld_stride);
-			if(v_act) lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + j * 1024, v_voff, kt * v_tile_stride + j * v_ld_stride);
+			if(k_act) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + j * 1024, k_voff + (kt * k_tile_stride + j * k_ld_stride));
+			if(v_act) lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + j * 1024, v_voff + (kt * v_tile_stride + j * v_ld_stride));
 		}
 	};
+
+	// ---- bias ring (BRING): the 32 x 64 bias tile of this wavefront's query block, 4 KB, travels
+	// HBM -> LDS by four LDS-direct loads of whole 128-byte row segments (eight lanes per row), two
+	// tiles ahead of its use and without occupying registers.  Slot layout: [row 32][128 B], the
+	// 16-byte chunk c of row r stored at chunk position c ^ (r & 7) so that the fragment reads (one
+	// chunk per lane, 32 rows at once) spread over the banks.  Rows past L lie beyond the buffer's
+	// range; chunks of keys past L (last tile) are sent there too, so padding behind a row's L valid
+	// entries is never read.  Whatever such lanes leave in LDS is finite: the ring starts zeroed.
+	const u32x4    b_rsrc    = raw_rsrc(BRING ? static_cast<const uint16_t*>(p.bias) + h * p.bias_stride[0] : nullptr,
+										BRING ? (uint32_t)(((L - 1) * p.bias_stride[1] + L) * 2) : 0u);
+	unsigned char* const bring = smem + LDS_SETS * 6 * TILE_BYTES + (BRING ? wave * 3 * 4096 : 0);
+	const uint32_t bring_addr = lds_addr_of(bring);
+	const int      b_voff     = (int)((lane >> 3) * p.bias_stride[1] * 2) + (((lane & 7) ^ (lane >> 3)) << 4);
+	const int      b_row0     = (int)((qtile * QT + (SPLIT ? 0 : wave * 32)) * p.bias_stride[1] * 2);
+	const int      b_row8     = (int)(8 * p.bias_stride[1] * 2);
+	const int      b_key      = ((lane & 7) ^ (lane >> 3)) * 8;  // first key of this lane's chunk within a tile
+	auto load_bias_tile = [&](int kt, int slot_i) {
+		if(!BRING) return;
+		const int in_row = kt * KT + b_key < (int)L ? b_voff + kt * (KT * 2) : 0x7FFF0000;
+#pragma unroll
+		for(int j = 0; j < 4; j++) lds_dma_b128(b_rsrc, bring_addr + slot_i * 4096 + j * 1024, in_row + (b_row0 + j * b_row8));
+	};
+	// fragment read: lane (n, half) takes chunk 4*sub + 2*c2 + half of row n
+	const int b_rd = n * 128 + (((n & 7) ^ half) << 4);
 
 	// Natural variant: four fragments in flight, each sub-tile's pair requested two stages before its
 	// use.  Log2 variant (BIAS_LATE): one pair only -- the registers are the scarce resource at four
@@ -345,7 +376,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	u32x4 bfrag[4];
 	auto  load_bias_frags = [&](int kt, auto sub_c) {
 		constexpr int SUB = decltype(sub_c)::value;
-		if(!has_bias) return;
+		if(!has_bias || BRING) return;
 		if(L2DOM) {
 #pragma unroll
 			for(int c2 = 0; c2 < 2; c2++)
@@ -391,7 +422,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		}
 	}
 	// mask table read address: lanes of the upper half-wave always read the zero entries
-	const int mask_rd     = (int)(LDS_SETS * 6 * TILE_BYTES) + (half == 0 ? n * 4 : (n_ktiles * KT + n) * 4);
+	const int mask_rd     = (int)MASK_BASE + (half == 0 ? n * 4 : (n_ktiles * KT + n) * 4);
 	const int mask_stride = half == 0 ? KT * 4 : 0;
 
 	// ---- online-softmax state (per lane: one query row; the two halves hold disjoint keys) ----
@@ -535,8 +566,15 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), s, 0, 0, 0);
 	};
 
-	auto stage = [&](auto subn_c, int k_off, int mask_addr_next, int v_off, auto subc_c, int bias_kt, auto bias_sub_c) {
+	auto read_bias_ring = [&](int slot_off, auto sub_c) {
+		constexpr int SUB = decltype(sub_c)::value;
+#pragma unroll
+		for(int c2 = 0; c2 < 2; c2++) bfrag[2 * SUB + c2] = *reinterpret_cast<const u32x4*>(bring + slot_off + (b_rd ^ ((4 * SUB + 2 * c2) << 4)));
+	};
+	// ring_off (BRING): byte offset of the ring slot that holds the bias tile of sub-tile j+1
+	auto stage = [&](auto subn_c, int k_off, int mask_addr_next, int v_off, auto subc_c, int bias_kt, auto bias_sub_c, int ring_off) {
 		constexpr int SUBN = decltype(subn_c)::value, SUBC = decltype(subc_c)::value, FB = 2 * SUBN;
+		if(BRING) read_bias_ring(ring_off, subn_c);
 		// operands of S^T(j+1) from LDS
 		u32x4 kf[NC];
 #pragma unroll
@@ -623,13 +661,18 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		// ---- prologue: first two tiles, first sub-tile's S^T and its row maximum ----
 		const int kt0 = __builtin_amdgcn_readfirstlane(live_at(0));
 		load_tile(kt0, 0);
-		if(my_n > 1) load_tile(__builtin_amdgcn_readfirstlane(live_at(1)), 1);
+		load_bias_tile(kt0, 0);
+		if(my_n > 1) {
+			load_tile(__builtin_amdgcn_readfirstlane(live_at(1)), 1);
+			load_bias_tile(__builtin_amdgcn_readfirstlane(live_at(1)), 1);
+		}
 #pragma unroll
 		for(int f = 0; f < 4; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
 		load_bias_frags(kt0, ic<0>{});
 		if(!BIAS_LATE) load_bias_frags(kt0, ic<1>{});
 		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 		if(!SPLIT) __syncthreads();
+		if(BRING) read_bias_ring(0, ic<0>{});
 		sc = compute_s_plain(0, 0, mask_rd + kt0 * mask_stride, 0);
 		rereference(sc, nullptr, true);
 		if(BIAS_LATE) load_bias_frags(kt0, ic<1>{});
@@ -643,7 +686,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			const int kt3_v = live_at(it + 3);
 			const int bufn = buf == 2 ? 0 : buf + 1, bufnn = bufn == 2 ? 0 : bufn + 1;
 			// sub-tile (it, 0): next is (it, 1) in the same buffer
-			stage(ic<1>{}, buf * TILE_BYTES, mask_rd + kt * mask_stride, buf * TILE_BYTES, ic<0>{}, kt1, ic<0>{});
+			stage(ic<1>{}, buf * TILE_BYTES, mask_rd + kt * mask_stride, buf * TILE_BYTES, ic<0>{}, kt1, ic<0>{}, buf * 4096);
 			if(!BIAS_LATE) load_bias_frags(kt1, ic<1>{});
 			// Tile it+1 (issued one iteration ago) must have landed, and every wavefront must be done
 			// with tile it-1, whose buffer tile it+2 is about to overwrite.  Loads complete in issue
@@ -652,9 +695,12 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			if(L2DOM && has_bias) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
 			else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 			if(!SPLIT) __syncthreads();
-			if(it + 2 < my_n) load_tile(kt2, bufnn);
+			if(it + 2 < my_n) {
+				load_tile(kt2, bufnn);
+				load_bias_tile(kt2, bufnn);  // (its slot held tile it-1, last read in the stage above)
+			}
 			// sub-tile (it, 1): next is (it+1, 0) in the next buffer (harmless stale data after the last tile)
-			stage(ic<0>{}, bufn * TILE_BYTES, mask_rd + kt1 * mask_stride, buf * TILE_BYTES, ic<1>{}, kt1, ic<1>{});
+			stage(ic<0>{}, bufn * TILE_BYTES, mask_rd + kt1 * mask_stride, buf * TILE_BYTES, ic<1>{}, kt1, ic<1>{}, bufn * 4096);
 			if(!BIAS_LATE) load_bias_frags(kt2, ic<0>{});
 			buf = bufn;
 			kt  = kt1;
@@ -762,7 +808,7 @@ int64_t mfma_bf16_workspace_bytes(const af3_dpa_params& p) {
 	return ws_bytes_needed(p);
 }
 
-template <int DP, int NW, bool L2DOM, bool BIAS_F32, bool SPLIT = false>
+template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT = false>
 static int launch_one(const af3_dpa_params& p, hipStream_t s) {
 	constexpr int QT       = SPLIT ? 32 : NW * 32;
 	const int     n_qtiles = (int)((p.L + QT - 1) / QT);
@@ -770,8 +816,8 @@ static int launch_one(const af3_dpa_params& p, hipStream_t s) {
 	const int64_t n_groups = p.B * p.H;
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
-	const size_t smem = (size_t)(SPLIT ? NW : 1) * 6 * KT * DP * 2 + ((size_t)n_ktiles * KT + 64) * 4 + (size_t)n_ktiles * 2 + 16;
-	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BIAS_F32, SPLIT>;
+	const size_t smem = (size_t)(SPLIT ? NW : 1) * 6 * KT * DP * 2 + (BMODE == 2 ? NW * 3 * 4096 : 0) + ((size_t)n_ktiles * KT + 64) * 4 + (size_t)n_ktiles * 2 + 16;
+	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BMODE, SPLIT>;
 	if(smem > 64 * 1024) {  // beyond the default dynamic-LDS limit: raise it for this kernel (idempotent, host side)
 		if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
 	}
@@ -779,20 +825,20 @@ static int launch_one(const af3_dpa_params& p, hipStream_t s) {
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }
 
-template <int DP, bool L2DOM, bool BIAS_F32>
+template <int DP, bool L2DOM, int BMODE>
 static int launch_nw(const af3_dpa_params& p, hipStream_t s) {
 	// the largest workgroup that still gives the 256 CUs a few workgroups each
 	const int64_t groups = p.B * p.H;
-	if(groups * ((p.L + 127) / 128) >= 768) return launch_one<DP, 4, L2DOM, BIAS_F32>(p, s);
-	if(groups * ((p.L + 63) / 64) >= 768) return launch_one<DP, 2, L2DOM, BIAS_F32>(p, s);
+	if(groups * ((p.L + 127) / 128) >= 768) return launch_one<DP, 4, L2DOM, BMODE>(p, s);
+	if(groups * ((p.L + 63) / 64) >= 768) return launch_one<DP, 2, L2DOM, BMODE>(p, s);
 	// Small launches: one 32-row block per workgroup, its key tiles split over 2 or 4 wavefronts so that
 	// more of the 1024 SIMDs have work.  The private LDS buffers limit a compute unit to one 4-wave or
 	// three 2-wave workgroups, so each split is only taken while the whole grid is resident at once
 	// (measured: beyond that the second round of workgroups costs more than the split gains).
 	const int64_t blocks1 = groups * ((p.L + 31) / 32), ktiles = (p.L + KT - 1) / KT;
-	if(DP == 32 && ktiles >= 4 && blocks1 <= 256) return launch_one<DP, 4, L2DOM, BIAS_F32, true>(p, s);
-	if(ktiles >= 2 && blocks1 <= (L2DOM ? 768 : 512)) return launch_one<DP, 2, L2DOM, BIAS_F32, true>(p, s);
-	return launch_one<DP, 1, L2DOM, BIAS_F32>(p, s);
+	if(DP == 32 && ktiles >= 4 && blocks1 <= 256) return launch_one<DP, 4, L2DOM, BMODE, true>(p, s);
+	if(ktiles >= 2 && blocks1 <= (L2DOM ? 768 : 512)) return launch_one<DP, 2, L2DOM, BMODE, true>(p, s);
+	return launch_one<DP, 1, L2DOM, BMODE>(p, s);
 }
 
 int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s) {
@@ -813,12 +859,16 @@ int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s) {
 		if(hipGetLastError() != hipSuccess) return AF3_ERR_LAUNCH;
 	}
 	const bool l2dom = use_ws || !p.bias;
+	// in-place bf16 bias: through the LDS ring when its rows can be fetched in aligned 16-byte chunks that
+	// never straddle the end of a row's L valid entries, element-wise otherwise
+	const bool ring = !l2dom && !bf32 && ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) && (p.bias_stride[0] % 8 == 0) && (p.bias_stride[1] % 8 == 0) && (p.L % 8 == 0) &&
+					  ((p.L - 1) * p.bias_stride[1] + p.L) * 2 < (int64_t)1 << 31;
 	if(p.D <= 32) {
-		if(l2dom) return launch_nw<32, true, false>(p, s);
-		return bf32 ? launch_nw<32, false, true>(p, s) : launch_nw<32, false, false>(p, s);
+		if(l2dom) return launch_nw<32, true, 0>(p, s);
+		return bf32 ? launch_nw<32, false, 1>(p, s) : ring ? launch_nw<32, false, 2>(p, s) : launch_nw<32, false, 0>(p, s);
 	}
-	if(l2dom) return launch_nw<64, true, false>(p, s);
-	return bf32 ? launch_nw<64, false, true>(p, s) : launch_nw<64, false, false>(p, s);
+	if(l2dom) return launch_nw<64, true, 0>(p, s);
+	return bf32 ? launch_nw<64, false, 1>(p, s) : ring ? launch_nw<64, false, 2>(p, s) : launch_nw<64, false, 0>(p, s);
 }
 
 }  // namespace af3

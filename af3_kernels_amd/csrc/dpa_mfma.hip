@@ -830,14 +830,24 @@ static int launch_nw(const af3_dpa_params& p, hipStream_t s) {
 	// the largest workgroup that still gives the 256 CUs a few workgroups each
 	const int64_t groups = p.B * p.H;
 	if(groups * ((p.L + 127) / 128) >= 768) return launch_one<DP, 4, L2DOM, BMODE>(p, s);
-	if(groups * ((p.L + 63) / 64) >= 768) return launch_one<DP, 2, L2DOM, BMODE>(p, s);
+	if(L2DOM && groups * ((p.L + 63) / 64) >= 768) return launch_one<DP, 2, L2DOM, BMODE>(p, s);
 	// Small launches: one 32-row block per workgroup, its key tiles split over 2 or 4 wavefronts so that
 	// more of the 1024 SIMDs have work.  The private LDS buffers limit a compute unit to one 4-wave or
 	// three 2-wave workgroups, so each split is only taken while the whole grid is resident at once
 	// (measured: beyond that the second round of workgroups costs more than the split gains).
 	const int64_t blocks1 = groups * ((p.L + 31) / 32), ktiles = (p.L + KT - 1) / KT;
+	if(!L2DOM) {
+		// In-place bias (one batch row): every single-wave workgroup would re-read the whole K and V of
+		// its head from L2, which then outweighs the bias stream; from 512 query blocks on, four blocks
+		// share each K/V tile instead (measured, B=1 H=16 D=24: L=1536 25.6 us against 32.7 us with
+		// single-wave workgroups; L=768 14.0 us split in two against 14.3 / 17.8; L=384 8.5 us split in four).
+		if(blocks1 >= 512) return launch_one<DP, 4, L2DOM, BMODE>(p, s);
+		if(DP == 32 && ktiles >= 4 && blocks1 <= 256) return launch_one<DP, 4, L2DOM, BMODE, true>(p, s);
+		if(ktiles >= 2) return launch_one<DP, 2, L2DOM, BMODE, true>(p, s);
+		return launch_one<DP, 1, L2DOM, BMODE>(p, s);
+	}
 	if(DP == 32 && ktiles >= 4 && blocks1 <= 256) return launch_one<DP, 4, L2DOM, BMODE, true>(p, s);
-	if(ktiles >= 2 && blocks1 <= (L2DOM ? 768 : 512)) return launch_one<DP, 2, L2DOM, BMODE, true>(p, s);
+	if(ktiles >= 2 && blocks1 <= 768) return launch_one<DP, 2, L2DOM, BMODE, true>(p, s);
 	return launch_one<DP, 1, L2DOM, BMODE>(p, s);
 }
 

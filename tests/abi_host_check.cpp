@@ -1,0 +1,175 @@
+// Torch-free check of the C ABI (include/af3_dpa.h): a plain HIP host program that allocates device
+// buffers with hipMalloc, calls af3_dpa_forward on a stream of its own the way a C / C++ / cgo / JNI
+// caller would, and compares the result with the CPU oracle's fp64 formula (af3o_dpa_formula).
+//
+//   abi_host_check            run every case on device 0; exit status 0 = all within tolerance
+//   abi_host_check --list     print the cases, touch no GPU
+//
+// Built by tests/Makefile (hipcc, links libaf3_dpa.so and the oracle library); run by tests/test_abi_host.py.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "af3_dpa.h"
+
+extern "C" int      af3o_dpa_formula(const float* q, const float* k, const float* v, const float* bias, const uint8_t* keep, float* out, int64_t B, int64_t H, int64_t L, int64_t D);
+extern "C" uint16_t af3o_f32_to_bf16_bits(float f);
+extern "C" float    af3o_bf16_bits_to_f32(uint16_t h);
+
+namespace {
+
+struct Case {
+	const char* name;
+	int64_t     B, H, L, D;
+	int         dtype;      // AF3_F32 or AF3_BF16
+	bool        workspace;  // hand the library its optional scratch buffer
+	int         drop_tail;  // keys dropped at the end of every row of the last batch entry
+	double      tol;
+};
+
+const Case CASES[] = {
+	{"fp32 2x4x128x32 (fp32-FMA kernel)", 2, 4, 128, 32, AF3_F32, false, 16, 1e-4},
+	{"bf16 3x4x200x32 with workspace", 3, 4, 200, 32, AF3_BF16, true, 20, 2e-2},
+	{"bf16 3x4x200x32 without workspace", 3, 4, 200, 32, AF3_BF16, false, 20, 2e-2},
+	{"bf16 1x16x256x24 in-place bias", 1, 16, 256, 24, AF3_BF16, false, 13, 2e-2},
+	{"bf16 2x2x96x64", 2, 2, 96, 64, AF3_BF16, true, 0, 2e-2},
+};
+
+// splitmix64 -> approximately normal values (sum of 4 uniforms), reproducible without <random>
+struct Rng {
+	uint64_t s;
+	double   u() {
+        uint64_t z = (s += 0x9E3779B97F4A7C15ull);
+        z          = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z          = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return (double)((z ^ (z >> 31)) >> 11) / 9007199254740992.0;
+	}
+	float n() { return (float)((u() + u() + u() + u() - 2.0) * 1.7320508); }
+};
+
+#define HIP_OK(x)                                                                      \
+	do {                                                                               \
+		hipError_t e_ = (x);                                                           \
+		if(e_ != hipSuccess) {                                                         \
+			std::fprintf(stderr, "%s failed: %s\n", #x, hipGetErrorString(e_));        \
+			return 2;                                                                  \
+		}                                                                              \
+	} while(0)
+
+int run(const Case& c, hipStream_t stream) {
+	const int64_t n = c.B * c.H * c.L * c.D, nb = c.H * c.L * c.L;
+	Rng           rng{0x5eed0000ull + (uint64_t)(c.L * 131 + c.D)};
+	std::vector<float> q(n), k(n), v(n), bias(nb), want(n);
+	for(auto* t : {&q, &k, &v}) for(auto& x : *t) x = rng.n();
+	for(auto& x : bias) x = rng.n();
+	std::vector<uint8_t> keep(c.B * c.L, 1);
+	for(int64_t j = c.L - c.drop_tail; j < c.L; j++) keep[(c.B - 1) * c.L + j] = 0;
+	const bool bf = c.dtype == AF3_BF16;
+	if(bf)  // the formula sees exactly what the kernel sees
+		for(auto* t : {&q, &k, &v, &bias}) for(auto& x : *t) x = af3o_bf16_bits_to_f32(af3o_f32_to_bf16_bits(x));
+	if(af3o_dpa_formula(q.data(), k.data(), v.data(), bias.data(), keep.data(), want.data(), c.B, c.H, c.L, c.D) != 0) return 2;
+
+	const size_t         esz = bf ? 2 : 4;
+	std::vector<uint8_t> hq(n * esz), hk(n * esz), hv(n * esz), hb(nb * esz), ho(n * esz);
+	auto                 pack = [&](const std::vector<float>& src, std::vector<uint8_t>& dst) {
+        for(size_t i = 0; i < src.size(); i++) {
+            if(bf) {
+                const uint16_t h = af3o_f32_to_bf16_bits(src[i]);
+                std::memcpy(&dst[2 * i], &h, 2);
+            } else {
+                std::memcpy(&dst[4 * i], &src[i], 4);
+            }
+        }
+	};
+	pack(q, hq), pack(k, hk), pack(v, hv), pack(bias, hb);
+
+	void *dq, *dk, *dv, *db, *dm, *dout, *dws = nullptr;
+	HIP_OK(hipMalloc(&dq, hq.size()));
+	HIP_OK(hipMalloc(&dk, hk.size()));
+	HIP_OK(hipMalloc(&dv, hv.size()));
+	HIP_OK(hipMalloc(&db, hb.size()));
+	HIP_OK(hipMalloc(&dm, keep.size()));
+	HIP_OK(hipMalloc(&dout, ho.size()));
+	HIP_OK(hipMemcpy(dq, hq.data(), hq.size(), hipMemcpyHostToDevice));
+	HIP_OK(hipMemcpy(dk, hk.data(), hk.size(), hipMemcpyHostToDevice));
+	HIP_OK(hipMemcpy(dv, hv.data(), hv.size(), hipMemcpyHostToDevice));
+	HIP_OK(hipMemcpy(db, hb.data(), hb.size(), hipMemcpyHostToDevice));
+	HIP_OK(hipMemcpy(dm, keep.data(), keep.size(), hipMemcpyHostToDevice));
+
+	af3_dpa_params p;
+	std::memset(&p, 0, sizeof p);
+	p.q = dq, p.k = dk, p.v = dv, p.bias = db, p.key_mask = static_cast<const uint8_t*>(dm), p.out = dout;
+	p.B = c.B, p.H = c.H, p.L = c.L, p.D = c.D;
+	const int64_t st[3] = {c.H * c.L * c.D, c.L * c.D, c.D};
+	for(int i = 0; i < 3; i++) p.q_stride[i] = p.k_stride[i] = p.v_stride[i] = p.out_stride[i] = st[i];
+	p.bias_stride[0] = c.L * c.L, p.bias_stride[1] = c.L;
+	p.key_mask_stride_b = c.L;
+	p.io_dtype = p.bias_dtype = p.out_dtype = p.mma_dtype = c.dtype;
+	p.softmax_scale = 1.0f / std::sqrt((float)c.D);
+	p.q_descale = p.k_descale = p.v_descale = 1.0f;
+	const int64_t ws = af3_dpa_workspace_bytes(&p);
+	if(c.workspace && ws > 0) {
+		HIP_OK(hipMalloc(&dws, (size_t)ws));
+		p.workspace = dws, p.workspace_bytes = ws;
+	}
+	const int kernel = af3_dpa_select_kernel(&p);
+	const int rc     = af3_dpa_forward(&p, stream);
+	if(rc != AF3_OK) {
+		std::fprintf(stderr, "af3_dpa_forward: %s\n", af3_status_string(rc));
+		return 1;
+	}
+	HIP_OK(hipStreamSynchronize(stream));
+	HIP_OK(hipMemcpy(ho.data(), dout, ho.size(), hipMemcpyDeviceToHost));
+	double err = 0.0;
+	bool   finite = true;
+	for(int64_t i = 0; i < n; i++) {
+		float g;
+		if(bf) {
+			uint16_t h;
+			std::memcpy(&h, &ho[2 * i], 2);
+			g = af3o_bf16_bits_to_f32(h);
+		} else {
+			std::memcpy(&g, &ho[4 * i], 4);
+		}
+		finite = finite && std::isfinite(g);
+		err    = std::fmax(err, std::fabs((double)g - (double)want[i]));
+	}
+	for(void* ptr : {dq, dk, dv, db, dm, dout, dws})
+		if(ptr) HIP_OK(hipFree(ptr));
+	const bool ok = finite && err <= c.tol;
+	std::printf("%-40s kernel=%d workspace=%lld B  max_abs_err=%.3e (tol %.0e)  %s\n", c.name, kernel, (long long)(dws ? ws : 0), err, c.tol, ok ? "ok" : "FAIL");
+	std::fflush(stdout);
+	return ok ? 0 : 1;
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+	if(argc > 1 && std::strcmp(argv[1], "--list") == 0) {
+		std::printf("abi version %d\n", af3_abi_version());
+		for(const Case& c : CASES) std::printf("%s\n", c.name);
+		return 0;
+	}
+	HIP_OK(hipSetDevice(0));
+	hipStream_t stream;
+	HIP_OK(hipStreamCreate(&stream));
+	int bad = 0;
+	for(const Case& c : CASES) {
+		const int r = run(c, stream);
+		if(r == 2) return 2;
+		bad += r;
+	}
+	// error behaviour: a malformed call is refused with a status code, nothing is launched
+	af3_dpa_params p;
+	std::memset(&p, 0, sizeof p);
+	const int rc = af3_dpa_forward(&p, stream);
+	std::printf("empty params -> %d (%s)\n", rc, af3_status_string(rc));
+	if(rc >= 0) bad++;
+	HIP_OK(hipStreamDestroy(stream));
+	return bad ? 1 : 0;
+}

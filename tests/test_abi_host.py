@@ -1,0 +1,32 @@
+"""The C ABI without torch: tests/abi_host_check.cpp (plain HIP host code, hipMalloc'd buffers, its
+own stream) is built by tests/Makefile ahead of time and run here as a child process."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "_build", "abi_host_check")
+
+
+def _need_binary():
+    if not os.path.exists(BIN):
+        pytest.fail(f"{BIN} is missing: run `python -c 'import __graft_entry__ as g; g.build()'` (or make -C tests) first")
+
+
+def test_host_program_links_the_library_and_lists_its_cases():
+    _need_binary()
+    r = subprocess.run([BIN, "--list"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, r.stderr
+    lines = r.stdout.strip().splitlines()
+    assert lines[0] == "abi version 1" and len(lines) >= 5
+
+
+@pytest.mark.gpu
+def test_c_callers_get_the_formula_through_the_abi_alone():
+    _need_binary()
+    print("running", BIN, flush=True)
+    r = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
+    print(r.stdout, r.stderr, flush=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count(" ok") >= 5 and "FAIL" not in r.stdout

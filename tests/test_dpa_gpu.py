@@ -442,3 +442,32 @@ def test_cfg5_fp8_full_size(af3, oracle):
         want = oracle.dpa_formula(f32np(q[b:b + 1]), f32np(k[b:b + 1]), f32np(v[b:b + 1]), mask.numpy(), f32np(bias))
         err = np.abs(f32np(out[b:b + 1]) - want).max()
         assert err <= case.tol, (b, err)
+
+
+# ---- HIP graph capture ------------------------------------------------------------------------
+
+def test_calls_can_be_captured_in_a_hip_graph_and_replayed(af3):
+    """The entry points only enqueue kernels on the given stream (no allocation, no synchronisation,
+    no memset nodes), so a call can be recorded into a HIP graph.  Every replay, with eager work and
+    synchronisations in between and fresh inputs copied into the captured buffers, must reproduce
+    the eager result bit for bit."""
+    B, H, L, D = 3, 4, 200, 32
+    q, k, v, m, bias = dev(*rand_inputs(B, H, L, D, torch.bfloat16, seed=21, mask="random"))
+    sq, sk, sv = q.clone(), k.clone(), v.clone()
+    af3.dot_product_attention_cpp(sq, sk, sv, m, bias)          # warm-up outside the capture (library load)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            out = af3.dot_product_attention_cpp(sq, sk, sv, m, bias)
+    torch.cuda.synchronize()
+    for rep in range(4):
+        g = torch.Generator().manual_seed(100 + rep)
+        nq, nk, nv = [torch.randn(B, H, L, D, generator=g).to(torch.bfloat16).cuda() for _ in range(3)]
+        sq.copy_(nq), sk.copy_(nk), sv.copy_(nv)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = af3.dot_product_attention_cpp(nq, nk, nv, m, bias)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager call"

@@ -170,9 +170,9 @@ __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2
 	// K: lane i of load j -> tile row j*(1024/DP) + i/(DP/16), 16-byte chunk i%(DP/16)
 	// V^T: lane i of load j -> row d = j*16 + i/4, 16-byte chunk i%4 of the 64-key row
 	const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-		const_cast<uint8_t*>(static_cast<const uint8_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1]), 0, (int)((L - 1) * p.k_stride[2] + (D + 15) / 16 * 16), 0x00020000);  // rows are fetched in 16-byte chunks
+		const_cast<uint8_t*>(static_cast<const uint8_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1]), 0, (int)((L - 1) * p.k_stride[2] + D), 0x00020000);  // exact end of the slab: rows are fetched in 16-byte chunks, range-checked per dword, so the tail of the last chunk reads as zero
 	const __amdgpu_buffer_rsrc_t klo_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-		const_cast<uint8_t*>(static_cast<const uint8_t*>(COMP ? p.k_lo : p.k) + b * p.k_stride[0] + h * p.k_stride[1]), 0, (int)((L - 1) * p.k_stride[2] + (D + 15) / 16 * 16), 0x00020000);
+		const_cast<uint8_t*>(static_cast<const uint8_t*>(COMP ? p.k_lo : p.k) + b * p.k_stride[0] + h * p.k_stride[1]), 0, (int)((L - 1) * p.k_stride[2] + D), 0x00020000);
 	const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
 		const_cast<uint8_t*>(static_cast<const uint8_t*>(p.v) + b * p.v_stride[0] + h * p.v_stride[1]), 0, (int)((D - 1) * p.v_stride[2] + p.v_stride[2]), 0x00020000);
 	constexpr int KCPR = DP / 16;       // 16-byte chunks per K row

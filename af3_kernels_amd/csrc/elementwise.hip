@@ -158,16 +158,17 @@ __global__ void __launch_bounds__(EW_THREADS) quantize_e4m3_kernel(const void* _
 			if(dst_lo) *reinterpret_cast<uint32_t*>(dst_lo + r * dst_row_stride + c) = residual(f0, f1, f2, f3, w);
 		}
 	} else {
-		// one thread = 4 consecutive rows of one column, written as 4 consecutive bytes of dst[matrix][col][row..row+3]
-		// (rows past the end of a matrix quantise to zero)
-		const int64_t rq = (rows_per_matrix + 3) >> 2, n_mat = rows / rows_per_matrix, total = n_mat * rq * cols;
+		// one thread = 4 consecutive rows of one column, written as 4 consecutive bytes of dst[matrix][col][row..row+3];
+		// rows past the end of a matrix quantise to zero, and the whole padded length of every output row
+		// (dst_row_stride, a multiple of 4) is written, so the destination needs no clearing beforehand
+		const int64_t rq = dst_row_stride >> 2, n_mat = rows / rows_per_matrix, total = n_mat * rq * cols;
 		for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += stride) {
 			const int64_t c   = i % cols;
 			const int64_t r4  = (i / cols) % rq;
 			const int64_t mat = i / (cols * rq);
 			const int64_t r   = mat * rows_per_matrix + (r4 << 2);
 			const int64_t left = rows_per_matrix - (r4 << 2);
-			const float   f0 = ld(r, c), f1 = left > 1 ? ld(r + 1, c) : 0.f, f2 = left > 2 ? ld(r + 2, c) : 0.f, f3 = left > 3 ? ld(r + 3, c) : 0.f;
+			const float   f0 = left > 0 ? ld(r, c) : 0.f, f1 = left > 1 ? ld(r + 1, c) : 0.f, f2 = left > 2 ? ld(r + 2, c) : 0.f, f3 = left > 3 ? ld(r + 3, c) : 0.f;
 			uint32_t      w   = 0;
 			w = __builtin_amdgcn_cvt_pk_fp8_f32(f0, f1, w, false);
 			w = __builtin_amdgcn_cvt_pk_fp8_f32(f2, f3, w, true);

@@ -280,12 +280,14 @@ def convert(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 
 
 def quantize_fp8_e4m3(x: torch.Tensor, pre_scale: float = 1.0, transpose_last2: bool = False, descale_out: Optional[torch.Tensor] = None,
-                      with_residual: bool = False):
+                      with_residual: bool = False, amax_buf: Optional[torch.Tensor] = None):
     """Per-tensor scaled quantisation to OCP e4m3: returns (fp8 tensor, descale) where descale is
     a 1-element device float and real ~= fp8 * descale.  The scale is the largest power of two
     that keeps amax * pre_scale <= 448.  With transpose_last2 the last two axes are swapped in
-    the output and the new innermost axis is padded to a multiple of 16 bytes.  With with_residual a third
-    value is returned: e4m3(x * pre_scale * scale - fp8), the rounding error at the same scale."""
+    the output and the new innermost axis is padded (with zeros) to a multiple of 16 bytes.  With
+    with_residual a third value is returned: e4m3(x * pre_scale * scale - fp8), the rounding error
+    at the same scale.  amax_buf: optional 1-element device float that already holds 0 (saves the
+    fill a fresh one needs)."""
     _require_device(x)
     if x.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("quantize_fp8_e4m3 takes float32 or bfloat16")
@@ -293,7 +295,7 @@ def quantize_fp8_e4m3(x: torch.Tensor, pre_scale: float = 1.0, transpose_last2: 
     rows_per_matrix, cols = x.shape[-2], x.shape[-1]
     rows = x.numel() // cols
     lib = _lib.load()
-    amax = torch.zeros(1, dtype=torch.float32, device=x.device)
+    amax = amax_buf if amax_buf is not None else torch.zeros(1, dtype=torch.float32, device=x.device)
     if descale_out is None:
         descale_out = torch.empty(1, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
@@ -301,19 +303,17 @@ def quantize_fp8_e4m3(x: torch.Tensor, pre_scale: float = 1.0, transpose_last2: 
         _lib.check(lib.af3_amax(x.data_ptr(), _DTYPE_CODE[x.dtype], x.numel(), amax.data_ptr(), st), "af3_amax")
         if transpose_last2:
             lpad = (rows_per_matrix + 15) // 16 * 16
-            full = torch.zeros(x.shape[:-2] + (cols, lpad), dtype=torch.float8_e4m3fn, device=x.device)
+            # (the quantiser writes the padding itself: nothing to clear)
+            full = torch.empty(x.shape[:-2] + (cols, lpad), dtype=torch.float8_e4m3fn, device=x.device)
             out = full[..., :rows_per_matrix]
-            full_lo = torch.zeros_like(full) if with_residual else None
+            full_lo = torch.empty_like(full) if with_residual else None
             lo = full_lo[..., :rows_per_matrix] if with_residual else None
             _lib.check(lib.af3_quantize_fp8_e4m3(x.data_ptr(), _DTYPE_CODE[x.dtype], full.data_ptr(), rows, cols, cols, 1, rows_per_matrix, lpad,
                                                  pre_scale, amax.data_ptr(), descale_out.data_ptr(), full_lo.data_ptr() if with_residual else None, st),
                        "af3_quantize_fp8_e4m3")
         else:
-            # 16 bytes of slack behind the last row: the fp8 attention kernel fetches rows in 16-byte chunks
-            flat = torch.zeros(x.numel() + 16, dtype=torch.uint8, device=x.device)
-            out = flat[:x.numel()].view(torch.float8_e4m3fn).view(x.shape)
-            flat_lo = torch.zeros_like(flat) if with_residual else None
-            lo = flat_lo[:x.numel()].view(torch.float8_e4m3fn).view(x.shape) if with_residual else None
+            out = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+            lo = torch.empty_like(out) if with_residual else None
             _lib.check(lib.af3_quantize_fp8_e4m3(x.data_ptr(), _DTYPE_CODE[x.dtype], out.data_ptr(), rows, cols, cols, 0, 0, cols,
                                                  pre_scale, amax.data_ptr(), descale_out.data_ptr(), lo.data_ptr() if with_residual else None, st),
                        "af3_quantize_fp8_e4m3")
@@ -330,10 +330,11 @@ def dot_product_attention_fp8(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     No reference counterpart (the reference has no fp8 path)."""
     _require_device(q, k, v, mask, bias)
     B, H, L, D = q.shape
-    descales = torch.empty(3, dtype=torch.float32, device=q.device)
-    q8, _, q_lo = quantize_fp8_e4m3(q, pre_scale=float(D) ** -0.5, descale_out=descales[0:1], with_residual=True)
-    k8, _, k_lo = quantize_fp8_e4m3(k, descale_out=descales[1:2], with_residual=True)
-    v8t, _ = quantize_fp8_e4m3(v, transpose_last2=True, descale_out=descales[2:3])
+    scratch = torch.zeros(6, dtype=torch.float32, device=q.device)   # three amax accumulators (start at 0), three descales
+    descales = scratch[3:6]
+    q8, _, q_lo = quantize_fp8_e4m3(q, pre_scale=float(D) ** -0.5, descale_out=descales[0:1], with_residual=True, amax_buf=scratch[0:1])
+    k8, _, k_lo = quantize_fp8_e4m3(k, descale_out=descales[1:2], with_residual=True, amax_buf=scratch[1:2])
+    v8t, _ = quantize_fp8_e4m3(v, transpose_last2=True, descale_out=descales[2:3], amax_buf=scratch[2:3])
     keep = _lift_mask(mask, L) if mask is not None else None
     bias = _inner_contig(bias.to(torch.bfloat16)) if bias is not None else None
     _check_shapes(q8, k8, v8t, keep, bias, v_transposed=True)

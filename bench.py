@@ -102,7 +102,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (every (batch, head, query-tile) task is "
-              "independent; see DESIGN.md for how it would shard). Run with --gpus 1.", file=sys.stderr)
+              "independent, so a node would shard the batch axis). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import torch

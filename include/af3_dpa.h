@@ -60,8 +60,9 @@ typedef enum af3_dtype {
  *                  are e4m3 bytes [B,H,L,D] and v is e4m3 bytes laid out TRANSPOSED as
  *                  [B, H, D, L] -- v_stride then holds strides for B, H and D, innermost (L) 1 --
  *                  as written by af3_quantize_fp8_e4m3 with transpose_last2 = 1).  K rows are
- *                  fetched in 16-byte chunks: when D % 16 != 0 the k allocation must extend at
- *                  least 8 readable bytes past its last row.
+ *                  fetched in 16-byte chunks through a range-checked buffer that ends at the last
+ *                  valid byte of each (batch, head) slab: nothing behind it is read, so the
+ *                  allocation needs no slack.
  *   bias_dtype   : AF3_F32 or AF3_BF16.          out_dtype : AF3_F32 or AF3_BF16.
  *   mma_dtype    : arithmetic of the two products: AF3_F32 (fp32 FMA), AF3_BF16 (bf16 MFMA,
  *                  fp32 accumulate) or AF3_FP8_E4M3 (e4m3 MFMA, fp32 accumulate).
@@ -159,7 +160,8 @@ int af3_amax(const void* src, int32_t src_dtype, int64_t n, float* amax_out, voi
  * 1/scale to *descale_out (device float).  src is viewed as [rows, cols] row-major with
  * row stride src_row_stride; with transpose_last2 != 0, every consecutive block of
  * `rows_per_matrix` rows is written transposed: dst[matrix][col][row], row stride
- * dst_row_stride (>= rows_per_matrix), so V [B*H*L, D] becomes [B*H, D, L].
+ * dst_row_stride (>= rows_per_matrix, a multiple of 4), so V [B*H*L, D] becomes [B*H, D, L];
+ * the padding bytes [rows_per_matrix, dst_row_stride) of every output row are written as zero.
  * dst_residual (optional, same layout as dst): e4m3(src * pre_scale * scale - dst), the rounding
  * error of dst at the same scale, for the compensated product of af3_dpa_forward.
  * No reference counterpart (see af3_amax).

@@ -471,3 +471,38 @@ def test_calls_can_be_captured_in_a_hip_graph_and_replayed(af3):
         eager = af3.dot_product_attention_cpp(nq, nk, nv, m, bias)
         torch.cuda.synchronize()
         assert torch.equal(out, eager), f"replay {rep} differs from the eager call"
+
+
+def test_fp8_k_rows_are_not_read_past_their_allocation(af3, oracle):
+    """head_dim 24: K rows are fetched in 16-byte chunks, so the last chunk of the last row would reach
+    8 bytes past the tensor.  The kernel's buffer ends at the last valid byte and must return zeros
+    beyond it: k and its residual are placed directly in front of e4m3 NaN bytes (0x7F), which would
+    poison the result if they were read."""
+    import ctypes
+    from af3_kernels_amd import ops
+    B, H, L, D = 2, 3, 200, 24
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=77, mask="random")
+    dq, dk, dv, dm, db = dev(q, k, v, m, bias)
+    want = af3.dot_product_attention_fp8(dq, dk, dv, dm, db)
+    scratch = torch.zeros(6, dtype=torch.float32, device="cuda")
+    q8, _, q_lo = af3.quantize_fp8_e4m3(dq, pre_scale=D ** -0.5, descale_out=scratch[3:4], with_residual=True, amax_buf=scratch[0:1])
+    k8, _, k_lo = af3.quantize_fp8_e4m3(dk, descale_out=scratch[4:5], with_residual=True, amax_buf=scratch[1:2])
+    v8t, _ = af3.quantize_fp8_e4m3(dv, transpose_last2=True, descale_out=scratch[5:6], amax_buf=scratch[2:3])
+
+    def poisoned(t):
+        arena = torch.full((t.numel() + 64,), 0x7F, dtype=torch.uint8, device="cuda")
+        arena[:t.numel()] = t.contiguous().view(torch.uint8).reshape(-1)
+        return arena, arena[:t.numel()].view(torch.float8_e4m3fn).view(t.shape)
+
+    a1, k8p = poisoned(k8)
+    a2, klop = poisoned(k_lo)
+    out = torch.empty_like(dq)
+    keep = ops._lift_mask(dm, L)
+    p = ops._fill_params(q8, k8p, v8t, keep, db, out, ops.AF3_FP8_E4M3, False, descales=scratch[3:6], softmax_scale=1.0)
+    p.q_lo, p.k_lo = q_lo.data_ptr(), klop.data_ptr()
+    print("fp8 forward on k tensors followed by NaN bytes", flush=True)
+    rc = af3._lib.load().af3_dpa_forward(ctypes.byref(p), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0
+    assert torch.isfinite(out).all()
+    assert torch.equal(out, want)

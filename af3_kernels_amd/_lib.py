@@ -30,6 +30,8 @@ class DpaParams(ctypes.Structure):
     ]
 
 
+QKV_SCRATCH_FLOATS = 768   # AF3_QKV_SCRATCH_FLOATS
+
 # name -> (restype, argtypes); every symbol include/af3_dpa.h declares
 SYMBOLS = {
     "af3_dpa_forward": (ctypes.c_int, [ctypes.POINTER(DpaParams), vp]),
@@ -38,6 +40,7 @@ SYMBOLS = {
     "af3_convert": (ctypes.c_int, [vp, i32, vp, i32, i64, vp]),
     "af3_amax": (ctypes.c_int, [vp, i32, i64, vp, vp]),
     "af3_quantize_fp8_e4m3": (ctypes.c_int, [vp, i32, vp, i64, i64, i64, i32, i64, i64, f32, vp, vp, vp, vp]),
+    "af3_quantize_qkv_fp8_e4m3": (ctypes.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, f32, vp, vp, vp, i64, vp, vp, vp, vp, vp]),
     "af3_pad_nd": (ctypes.c_int, [vp, vp, i32, ctypes.POINTER(i64), ctypes.POINTER(i64), ctypes.POINTER(i64), i32, ctypes.c_uint32, vp]),
     "af3_vnni_repack_bf16": (ctypes.c_int, [vp, vp, i64, i64, i64, vp]),
     "af3_status_string": (ctypes.c_char_p, [ctypes.c_int]),

@@ -144,8 +144,11 @@ __global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restric
 // (explicit s_waitcnt vmcnt before the barrier that publishes a tile).  rsrc and lds_addr must be
 // wave-uniform.  The whole byte offset travels in the vector operand, which the hardware range-checks
 // against the buffer size: a lane whose offset is past the end fetches nothing from memory.
+// M0 (the LDS base of the load) is written behind the compiler's back: nothing else in this file
+// makes it use M0 -- no LDS-direct builtins, no indirect register indexing -- and gfx950's LDS
+// instructions do not read it.
 __device__ __forceinline__ void lds_dma_b128(const u32x4& rsrc, uint32_t lds_addr, int voff) {
-	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc) : "memory", "m0");
+	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
 }
 __device__ __forceinline__ u32x4 raw_rsrc(const void* base, uint32_t bytes) {
 	const uint64_t a = reinterpret_cast<uint64_t>(base);

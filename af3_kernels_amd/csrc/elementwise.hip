@@ -83,8 +83,9 @@ __global__ void __launch_bounds__(EW_THREADS) cvt_e4m3_kernel(const uint8_t* __r
 // ---- per-tensor amax -------------------------------------------------------------------------
 // 16-byte loads, wave then workgroup reduction, one atomic per workgroup (a few hundred atomics on
 // the one result word instead of one per wavefront).
+// maximum of |src[i]| over this workgroup's grid-stride share; valid in thread 0
 template <bool SRC_BF16>
-__global__ void __launch_bounds__(EW_THREADS) amax_kernel(const void* __restrict__ src, int64_t n, float* amax_out) {
+__device__ __forceinline__ float block_amax(const void* __restrict__ src, int64_t n) {
 	__shared__ float part[EW_THREADS / 64];
 	const int64_t stride = (int64_t)gridDim.x * EW_THREADS, tid0 = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x;
 	constexpr int PER  = SRC_BF16 ? 8 : 4;  // elements per 16-byte load
@@ -106,11 +107,30 @@ __global__ void __launch_bounds__(EW_THREADS) amax_kernel(const void* __restrict
 	for(int o = 32; o > 0; o >>= 1) a = fmaxf(a, __shfl_xor(a, o));
 	if((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = a;
 	__syncthreads();
-	if(threadIdx.x == 0) {
+	if(threadIdx.x == 0)
 		for(int w = 1; w < EW_THREADS / 64; w++) a = fmaxf(a, part[w]);
-		// non-negative floats order like their bit patterns
-		atomicMax(reinterpret_cast<unsigned int*>(amax_out), __float_as_uint(a));
-	}
+	return a;
+}
+
+template <bool SRC_BF16>
+__global__ void __launch_bounds__(EW_THREADS) amax_kernel(const void* __restrict__ src, int64_t n, float* amax_out) {
+	const float a = block_amax<SRC_BF16>(src, n);
+	// non-negative floats order like their bit patterns
+	if(threadIdx.x == 0) atomicMax(reinterpret_cast<unsigned int*>(amax_out), __float_as_uint(a));
+}
+
+// Three tensors in one launch (blockIdx.y), every workgroup storing its partial maximum: no atomics,
+// nothing to clear beforehand.  partials: [3][AMAX3_BLOCKS].
+constexpr int AMAX3_BLOCKS = 256;
+struct Amax3Args {
+	const void* src[3];
+	int64_t     n[3];
+};
+template <bool SRC_BF16>
+__global__ void __launch_bounds__(EW_THREADS) amax3_kernel(Amax3Args a, float* __restrict__ partials) {
+	const int   t = blockIdx.y;
+	const float m = block_amax<SRC_BF16>(a.src[t], a.n[t]);
+	if(threadIdx.x == 0) partials[t * AMAX3_BLOCKS + blockIdx.x] = m;
 }
 
 // scale = 2^floor(log2(448 / (amax*pre_scale))); the power of two keeps every descale product exact.
@@ -125,11 +145,9 @@ __device__ __forceinline__ float fp8_pow2_scale(float amax, float pre_scale) {
 }
 
 template <bool SRC_BF16>
-__global__ void __launch_bounds__(EW_THREADS) quantize_e4m3_kernel(const void* __restrict__ src, uint8_t* __restrict__ dst, int64_t rows, int64_t cols,
-																	 int64_t src_row_stride, int transpose, int64_t rows_per_matrix, int64_t dst_row_stride,
-																	 float pre_scale, const float* amax, float* descale_out, uint8_t* __restrict__ dst_lo) {
-	const float scale = fp8_pow2_scale(*amax, pre_scale);
-	if(blockIdx.x == 0 && threadIdx.x == 0 && descale_out) *descale_out = 1.f / scale;
+__device__ __forceinline__ void quantize_e4m3_body(const void* __restrict__ src, uint8_t* __restrict__ dst, int64_t rows, int64_t cols, int64_t src_row_stride,
+													 int transpose, int64_t rows_per_matrix, int64_t dst_row_stride, float pre_scale, float scale,
+													 uint8_t* __restrict__ dst_lo) {
 	const float   mul    = pre_scale * scale;
 	const int64_t stride = (int64_t)gridDim.x * EW_THREADS;
 	auto          ld     = [&](int64_t r, int64_t c) -> float {
@@ -176,6 +194,45 @@ __global__ void __launch_bounds__(EW_THREADS) quantize_e4m3_kernel(const void* _
 			if(dst_lo) *reinterpret_cast<uint32_t*>(dst_lo + (mat * cols + c) * dst_row_stride + (r4 << 2)) = residual(f0, f1, f2, f3, w);
 		}
 	}
+}
+
+template <bool SRC_BF16>
+__global__ void __launch_bounds__(EW_THREADS) quantize_e4m3_kernel(const void* __restrict__ src, uint8_t* __restrict__ dst, int64_t rows, int64_t cols,
+																	 int64_t src_row_stride, int transpose, int64_t rows_per_matrix, int64_t dst_row_stride,
+																	 float pre_scale, const float* amax, float* descale_out, uint8_t* __restrict__ dst_lo) {
+	const float scale = fp8_pow2_scale(*amax, pre_scale);
+	if(blockIdx.x == 0 && threadIdx.x == 0 && descale_out) *descale_out = 1.f / scale;
+	quantize_e4m3_body<SRC_BF16>(src, dst, rows, cols, src_row_stride, transpose, rows_per_matrix, dst_row_stride, pre_scale, scale, dst_lo);
+}
+
+// q, k and v of one attention call in one launch (blockIdx.y): q and k as they are (plus residuals),
+// v transposed; each workgroup first folds its tensor's partial maxima from amax3_kernel.
+struct Quant3Args {
+	const void* src[3];
+	uint8_t*    dst[3];
+	uint8_t*    dst_lo[3];
+	int64_t     rows, cols, rows_per_matrix, v_row_stride;
+	float       pre_scale[3];
+};
+template <bool SRC_BF16>
+__global__ void __launch_bounds__(EW_THREADS) quantize3_kernel(Quant3Args a, const float* __restrict__ partials, float* __restrict__ descales) {
+	__shared__ float red[EW_THREADS / 64];
+	__shared__ float s_amax;
+	const int t = blockIdx.y;
+	static_assert(AMAX3_BLOCKS == EW_THREADS, "one partial per thread");
+	float m = partials[t * AMAX3_BLOCKS + threadIdx.x];
+	for(int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+	if((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+	__syncthreads();
+	if(threadIdx.x == 0) {
+		for(int w = 1; w < EW_THREADS / 64; w++) m = fmaxf(m, red[w]);
+		s_amax = m;
+	}
+	__syncthreads();
+	const float scale = fp8_pow2_scale(s_amax, a.pre_scale[t]);
+	if(blockIdx.x == 0 && threadIdx.x == 0) descales[t] = 1.f / scale;
+	const bool tr = t == 2;
+	quantize_e4m3_body<SRC_BF16>(a.src[t], a.dst[t], a.rows, a.cols, a.cols, tr ? 1 : 0, a.rows_per_matrix, tr ? a.v_row_stride : a.cols, a.pre_scale[t], scale, a.dst_lo[t]);
 }
 
 // ---- pad / repack ----------------------------------------------------------------------------
@@ -269,6 +326,37 @@ extern "C" int af3_quantize_fp8_e4m3(const void* src, int32_t sd, void* dst, int
 						   rows_per_matrix, dst_row_stride, pre_scale, amax, descale_out, static_cast<uint8_t*>(dst_residual));
 	else
 		return AF3_ERR_BAD_DTYPE;
+	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+extern "C" int af3_quantize_qkv_fp8_e4m3(const void* q, const void* k, const void* v, int32_t sd, int64_t B, int64_t H, int64_t L, int64_t D, float q_pre_scale, void* q8,
+										void* k8, void* v8t, int64_t v8t_row_stride, void* q_lo, void* k_lo, float* descales, float* scratch, void* stream) {
+	if(B <= 0 || H <= 0 || L <= 0 || D <= 0) return AF3_ERR_BAD_SHAPE;
+	if(!q || !k || !v || !q8 || !k8 || !v8t || !descales || !scratch) return AF3_ERR_NULL_POINTER;
+	if(D % 4 != 0) return AF3_ERR_BAD_ARGUMENT;
+	if(v8t_row_stride < (L + 3) / 4 * 4 || v8t_row_stride % 4 != 0) return AF3_ERR_BAD_STRIDE;
+	if(sd != AF3_F32 && sd != AF3_BF16) return AF3_ERR_BAD_DTYPE;
+	for(const void* ptr : {(const void*)q8, (const void*)k8, (const void*)v8t, (const void*)q_lo, (const void*)k_lo})
+		if(reinterpret_cast<uintptr_t>(ptr) & 3) return AF3_ERR_BAD_ARGUMENT;
+	hipStream_t   s = static_cast<hipStream_t>(stream);
+	const int64_t n = B * H * L * D;
+	Amax3Args     aa;
+	aa.src[0] = q, aa.src[1] = k, aa.src[2] = v;
+	aa.n[0] = aa.n[1] = aa.n[2] = n;
+	Quant3Args qa;
+	qa.src[0] = q, qa.src[1] = k, qa.src[2] = v;
+	qa.dst[0] = static_cast<uint8_t*>(q8), qa.dst[1] = static_cast<uint8_t*>(k8), qa.dst[2] = static_cast<uint8_t*>(v8t);
+	qa.dst_lo[0] = static_cast<uint8_t*>(q_lo), qa.dst_lo[1] = static_cast<uint8_t*>(k_lo), qa.dst_lo[2] = nullptr;
+	qa.rows = B * H * L, qa.cols = D, qa.rows_per_matrix = L, qa.v_row_stride = v8t_row_stride;
+	qa.pre_scale[0] = q_pre_scale, qa.pre_scale[1] = qa.pre_scale[2] = 1.f;
+	const dim3 ga(AMAX3_BLOCKS, 3), gq(ew_blocks(n / 4, 2048), 3);
+	if(sd == AF3_F32) {
+		hipLaunchKernelGGL(amax3_kernel<false>, ga, dim3(EW_THREADS), 0, s, aa, scratch);
+		hipLaunchKernelGGL(quantize3_kernel<false>, gq, dim3(EW_THREADS), 0, s, qa, scratch, descales);
+	} else {
+		hipLaunchKernelGGL(amax3_kernel<true>, ga, dim3(EW_THREADS), 0, s, aa, scratch);
+		hipLaunchKernelGGL(quantize3_kernel<true>, gq, dim3(EW_THREADS), 0, s, qa, scratch, descales);
+	}
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }
 

@@ -330,11 +330,28 @@ def dot_product_attention_fp8(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     No reference counterpart (the reference has no fp8 path)."""
     _require_device(q, k, v, mask, bias)
     B, H, L, D = q.shape
-    scratch = torch.zeros(6, dtype=torch.float32, device=q.device)   # three amax accumulators (start at 0), three descales
-    descales = scratch[3:6]
-    q8, _, q_lo = quantize_fp8_e4m3(q, pre_scale=float(D) ** -0.5, descale_out=descales[0:1], with_residual=True, amax_buf=scratch[0:1])
-    k8, _, k_lo = quantize_fp8_e4m3(k, descale_out=descales[1:2], with_residual=True, amax_buf=scratch[1:2])
-    v8t, _ = quantize_fp8_e4m3(v, transpose_last2=True, descale_out=descales[2:3], amax_buf=scratch[2:3])
+    if q.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("dot_product_attention_fp8 takes float32 or bfloat16 inputs")
+    if tuple(k.shape) != (B, H, L, D) or tuple(v.shape) != (B, H, L, D):
+        raise ValueError(f"k and v must have q's shape {tuple(q.shape)}, got {tuple(k.shape)} and {tuple(v.shape)}")
+    if D % 4 != 0:
+        raise ValueError("the fp8 path needs head_dim % 4 == 0")
+    q, k, v = q.contiguous(), k.to(q.dtype).contiguous(), v.to(q.dtype).contiguous()
+    # one launch for the three amax reductions, one for the three quantisations (q with D^-1/2 folded in and
+    # k with residuals, v transposed and padded to 16 keys)
+    lpad = (L + 15) // 16 * 16
+    f8 = torch.float8_e4m3fn
+    q8, k8 = torch.empty(q.shape, dtype=f8, device=q.device), torch.empty(q.shape, dtype=f8, device=q.device)
+    q_lo, k_lo = (torch.empty_like(q8), torch.empty_like(k8)) if compensated else (None, None)
+    v8t_full = torch.empty((B, H, D, lpad), dtype=f8, device=q.device)
+    v8t = v8t_full[..., :L]
+    scratch = torch.empty(3 + _lib.QKV_SCRATCH_FLOATS, dtype=torch.float32, device=q.device)
+    descales = scratch[0:3]
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.load().af3_quantize_qkv_fp8_e4m3(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), _DTYPE_CODE[q.dtype], B, H, L, D, float(D) ** -0.5, q8.data_ptr(), k8.data_ptr(), v8t_full.data_ptr(), lpad,
+            q_lo.data_ptr() if compensated else None, k_lo.data_ptr() if compensated else None, descales.data_ptr(), scratch[3:].data_ptr(),
+            _stream_ptr(q.device)), "af3_quantize_qkv_fp8_e4m3")
     keep = _lift_mask(mask, L) if mask is not None else None
     bias = _inner_contig(bias.to(torch.bfloat16)) if bias is not None else None
     _check_shapes(q8, k8, v8t, keep, bias, v_transposed=True)

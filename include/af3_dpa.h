@@ -171,6 +171,21 @@ int af3_quantize_fp8_e4m3(const void* src, int32_t src_dtype, void* dst, int64_t
 						  float* descale_out, void* dst_residual, void* hip_stream);
 
 /*
+ * The whole per-tensor fp8 preparation of one attention call in two launches: amax of q, k and v,
+ * then q8 = e4m3(q * q_pre_scale * sq), k8 = e4m3(k * sk) (both [B,H,L,D], with their residuals
+ * q_lo, k_lo when those pointers are non-NULL) and v8t = e4m3(v * sv) transposed to
+ * [B,H,D,v8t_row_stride] (padding written as zero), scales as in af3_quantize_fp8_e4m3.
+ * q, k, v: contiguous [B,H,L,D] of src_dtype (AF3_F32 or AF3_BF16), D % 4 == 0.
+ * descales: 3 device floats, written {1/sq, 1/sk, 1/sv} (pass them as device_descales).
+ * scratch: AF3_QKV_SCRATCH_FLOATS device floats, overwritten; it need not be cleared.
+ * No reference counterpart (see af3_amax).
+ */
+#define AF3_QKV_SCRATCH_FLOATS 768
+int af3_quantize_qkv_fp8_e4m3(const void* q, const void* k, const void* v, int32_t src_dtype, int64_t B, int64_t H, int64_t L, int64_t D,
+							  float q_pre_scale, void* q8, void* k8, void* v8t, int64_t v8t_row_stride, void* q_lo, void* k_lo,
+							  float* descales, float* scratch, void* hip_stream);
+
+/*
  * N-dimensional pad (ndim <= AF3_PAD_MAX_DIMS): copy src (shape src_shape, element strides
  * src_strides) into the low corner of a contiguous dst of shape dst_shape (>= src_shape in
  * every axis) and fill the rest with the 32-bit pattern `fill_bits` truncated to elem_size

@@ -128,6 +128,15 @@ def test_elementwise_entry_points_validate_on_the_host():
     assert lib.af3_pad_nd(0x1000, 0x2000, 2, arr(4, 4), arr(4, 1), arr(2, 8), 4, 0, None) == -3   # shrinking
     assert lib.af3_pad_nd(0x1000, 0x2000, 9, arr(4, 4), arr(4, 1), arr(4, 8), 4, 0, None) == -3
     assert lib.af3_quantize_fp8_e4m3(0x1000, 1, 0x2000, 8, 6, 6, 0, 0, 6, 1.0, 0x3000, None, None, None) == -7    # cols % 4
+    qkv = lib.af3_quantize_qkv_fp8_e4m3
+    good = dict(q=0x1000, k=0x2000, v=0x3000, sd=1, B=1, H=2, L=10, D=8, pre=1.0, q8=0x4000, k8=0x5000, v8t=0x6000, vs=16, qlo=None, klo=None, ds=0x7000, sc=0x8000)
+    call = lambda **kw: qkv(*[{**good, **kw}[n] for n in ("q", "k", "v", "sd", "B", "H", "L", "D", "pre", "q8", "k8", "v8t", "vs", "qlo", "klo", "ds", "sc")], None)
+    assert call(D=6) == -7            # head_dim % 4
+    assert call(vs=8) == -4           # transposed rows shorter than L
+    assert call(vs=14) == -4          # not a multiple of 4
+    assert call(sd=2) == -2           # fp8 source
+    assert call(sc=None) == -1
+    assert call(L=0) == -3
 
 
 def test_wrapper_rejects_cpu_tensors_and_bad_shapes():

@@ -20,7 +20,28 @@ KERNEL_NAMES = {0: "fp32_fma", 1: "bf16_mfma", 2: "fp8_mfma"}
 
 
 def _stream_ptr(device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """Raw handle of torch's current stream on `device` (the short route: building a torch.cuda.Stream object
+    per call costs several microseconds, which a small attention call notices)."""
+    return torch._C._cuda_getCurrentRawStream(device.index if device.index is not None else torch.cuda.current_device())
+
+
+class _on_device:
+    """`with torch.cuda.device(d)` that does nothing when d is already the current device."""
+    __slots__ = ("idx", "prev")
+
+    def __init__(self, device):
+        self.idx = device.index
+
+    def __enter__(self):
+        self.prev = None
+        if self.idx is not None and self.idx != torch.cuda.current_device():
+            self.prev = torch.cuda.current_device()
+            torch.cuda.set_device(self.idx)
+
+    def __exit__(self, *exc):
+        if self.prev is not None:
+            torch.cuda.set_device(self.prev)
+        return False
 
 
 def _require_device(*tensors):
@@ -165,7 +186,7 @@ def _dpa_forward_impl(q, k, v, keep, bias, mma_dtype: int, force_generic: bool) 
         # scratch for the kernel's bias rewrite; torch's caching allocator makes this a pointer bump
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
         p.workspace, p.workspace_bytes = ws.data_ptr(), ws_bytes
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         if _timers.enabled:
             s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             s.record()
@@ -251,7 +272,9 @@ def dot_product_attention_cpp(
     dtype = q.dtype
     keep = _lift_mask(mask, q.shape[2]) if mask is not None else None
     bias = bias.to(dtype) if bias is not None else None
-    return _dpa_forward_op(q, k.to(dtype), v.to(dtype), keep, bias, code, False)
+    # (straight into the implementation: the registered op torch.ops.af3_kernels.dpa_forward is the same function
+    # behind torch's dispatcher, whose per-call cost is comparable to a small attention kernel)
+    return _dpa_forward_impl(q, k.to(dtype), v.to(dtype), keep, bias, code, False)
 
 
 def selected_kernel(q, k, v, mask, bias, force_generic=False) -> str:
@@ -273,7 +296,7 @@ def convert(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     _require_device(x)
     x = x.contiguous()
     out = torch.empty(x.shape, dtype=dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         _lib.check(_lib.load().af3_convert(x.data_ptr(), _DTYPE_CODE[x.dtype], out.data_ptr(), _DTYPE_CODE[dtype], x.numel(),
                                            _stream_ptr(x.device)), "af3_convert")
     return out
@@ -298,7 +321,7 @@ def quantize_fp8_e4m3(x: torch.Tensor, pre_scale: float = 1.0, transpose_last2: 
     amax = amax_buf if amax_buf is not None else torch.zeros(1, dtype=torch.float32, device=x.device)
     if descale_out is None:
         descale_out = torch.empty(1, dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = _stream_ptr(x.device)
         _lib.check(lib.af3_amax(x.data_ptr(), _DTYPE_CODE[x.dtype], x.numel(), amax.data_ptr(), st), "af3_amax")
         if transpose_last2:
@@ -347,7 +370,7 @@ def dot_product_attention_fp8(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     v8t = v8t_full[..., :L]
     scratch = torch.empty(3 + _lib.QKV_SCRATCH_FLOATS, dtype=torch.float32, device=q.device)
     descales = scratch[0:3]
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         _lib.check(_lib.load().af3_quantize_qkv_fp8_e4m3(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), _DTYPE_CODE[q.dtype], B, H, L, D, float(D) ** -0.5, q8.data_ptr(), k8.data_ptr(), v8t_full.data_ptr(), lpad,
             q_lo.data_ptr() if compensated else None, k_lo.data_ptr() if compensated else None, descales.data_ptr(), scratch[3:].data_ptr(),
@@ -359,7 +382,7 @@ def dot_product_attention_fp8(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     p = _fill_params(q8, k8, v8t, keep, bias, out, AF3_FP8_E4M3, False, descales=descales, softmax_scale=1.0)
     if compensated:
         p.q_lo, p.k_lo = q_lo.data_ptr(), k_lo.data_ptr()
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         _lib.check(_lib.load().af3_dpa_forward(ctypes.byref(p), _stream_ptr(q.device)), "af3_dpa_forward(fp8)")
     return out
 
@@ -384,7 +407,7 @@ def pad_and_align_tensor(x: torch.Tensor, shape, need_init: bool = True, init: f
     fill_bits = int(fill.item()) & 0xFFFFFFFF
     n = x.dim()
     arr = ctypes.c_int64 * n
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         _lib.check(_lib.load().af3_pad_nd(x.data_ptr(), out.data_ptr(), n, arr(*x.shape), arr(*x.stride()), arr(*shape), x.element_size(),
                                           fill_bits, _stream_ptr(x.device)), "af3_pad_nd")
     return out
@@ -405,6 +428,6 @@ def vnni_repack_tensor(x: torch.Tensor, type: int = 2, BLK_SZ: int = 0) -> torch
         raise ValueError("only XFORM_N2V (type=2) is implemented")
     M, N = x.shape
     out = torch.empty_like(x)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         _lib.check(_lib.load().af3_vnni_repack_bf16(x.data_ptr(), out.data_ptr(), M, N, BLK_SZ, _stream_ptr(x.device)), "af3_vnni_repack_bf16")
     return out

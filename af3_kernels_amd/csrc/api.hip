@@ -42,10 +42,11 @@ int validate(const af3_dpa_params* p) {
 	return AF3_OK;
 }
 
-// 0 generic, 1 bf16 MFMA, 2 fp8 MFMA, or a negative status
+// 0 fp32 vector-FMA, 1 bf16 MFMA, 2 fp8 MFMA, 3 fp32 MFMA, or a negative status
 int select_kernel(const af3_dpa_params& p) {
 	if(p.io_dtype == AF3_FP8_E4M3) return mfma_fp8_eligible(p) ? 2 : AF3_ERR_BAD_ARGUMENT;
-	if(p.force_generic || p.mma_dtype == AF3_F32) return 0;
+	if(p.force_generic) return 0;
+	if(p.mma_dtype == AF3_F32) return mfma_f32_eligible(p) ? 3 : 0;
 	return mfma_bf16_eligible(p) ? 1 : 0;
 }
 
@@ -71,6 +72,7 @@ extern "C" int af3_dpa_forward(const af3_dpa_params* params, void* hip_stream) {
 		case 0: return launch_dpa_generic(*params, s);
 		case 1: return launch_dpa_mfma_bf16(*params, s);
 		case 2: return launch_dpa_mfma_fp8(*params, s);
+		case 3: return launch_dpa_mfma_f32(*params, s);
 		default: return AF3_ERR_BAD_ARGUMENT;
 	}
 }

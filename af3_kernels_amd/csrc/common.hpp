@@ -47,5 +47,7 @@ int launch_dpa_mfma_fp8(const af3_dpa_params& p, hipStream_t s);
 bool mfma_bf16_eligible(const af3_dpa_params& p);
 int64_t mfma_bf16_workspace_bytes(const af3_dpa_params& p);
 bool mfma_fp8_eligible(const af3_dpa_params& p);
+int launch_dpa_mfma_f32(const af3_dpa_params& p, hipStream_t s);
+bool mfma_f32_eligible(const af3_dpa_params& p);
 
 }  // namespace af3

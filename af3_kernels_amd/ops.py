@@ -16,7 +16,7 @@ from ._lib import AF3_BF16, AF3_F32, AF3_FP8_E4M3, DpaParams
 _DTYPE_CODE = {torch.float32: AF3_F32, torch.bfloat16: AF3_BF16}
 if hasattr(torch, "float8_e4m3fn"):
     _DTYPE_CODE[torch.float8_e4m3fn] = AF3_FP8_E4M3
-KERNEL_NAMES = {0: "fp32_fma", 1: "bf16_mfma", 2: "fp8_mfma"}
+KERNEL_NAMES = {0: "fp32_fma", 1: "bf16_mfma", 2: "fp8_mfma", 3: "fp32_mfma"}
 
 
 def _stream_ptr(device) -> int:

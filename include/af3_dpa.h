@@ -133,8 +133,9 @@ int af3_dpa_forward(const af3_dpa_params* params, void* hip_stream);
  * no bias, or a kernel that does not take one); negative = af3_status error.  Host only. */
 int64_t af3_dpa_workspace_bytes(const af3_dpa_params* params);
 
-/* Which kernel af3_dpa_forward would run for these arguments: 0 = fp32-FMA kernel,
- * 1 = bf16 MFMA kernel, 2 = fp8 MFMA kernel; negative = af3_status error.  Host only. */
+/* Which kernel af3_dpa_forward would run for these arguments: 0 = fp32 vector-FMA kernel,
+ * 1 = bf16 MFMA kernel, 2 = fp8 MFMA kernel, 3 = fp32 MFMA kernel; negative = af3_status error.
+ * Host only. */
 int af3_dpa_select_kernel(const af3_dpa_params* params);
 
 /*

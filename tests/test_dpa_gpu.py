@@ -92,8 +92,8 @@ def test_golden_vectors(af3, path, dtype):
 def test_cfg1_fp32_plumbing_case(af3, oracle):
     from af3_kernels_amd.synthetic import CASES, make_inputs
     q, k, v, mask, bias = make_inputs(CASES["cfg1"])
-    err = run_case(af3, oracle, q, k, v, mask, bias, expect_kernel="fp32_fma")
-    assert err < 1e-5   # fp32 FMA with an fp32 softmax sits far inside the 1e-4 budget
+    err = run_case(af3, oracle, q, k, v, mask, bias, expect_kernel="fp32_mfma")
+    assert err < 1e-5   # fp32 matrix cores with an fp32 softmax sit far inside the 1e-4 budget
 
 
 # ---- bf16 matrix-core kernel ----------------------------------------------------------------
@@ -209,13 +209,47 @@ def test_strided_inputs_and_prepadded_bias(af3, oracle):
     assert np.abs(f32np(out) - want).max() <= 2e-2
 
 
-def test_fp32_fma_kernel_shapes(af3, oracle):
-    for (B, H, L, D, mask) in [(1, 2, 700, 40, "random"), (2, 3, 37, 20, "tail"), (1, 1, 5, 3, "none"), (1, 2, 130, 128, "random")]:
-        q, k, v, m, bias = rand_inputs(B, H, L, D, torch.float32, seed=L, mask=mask)
-        run_case(af3, oracle, q, k, v, m, bias, expect_kernel="fp32_fma")
-    # bf16 storage whose head_dim is not a multiple of 8 also takes this kernel
+@pytest.mark.parametrize("B,H,L,D,mask,kernel", [
+    (1, 2, 700, 40, "random", "fp32_mfma"),     # head_dim 40: padded to 64 columns
+    (2, 3, 37, 20, "tail", "fp32_mfma"),        # odd length, head_dim 20
+    (3, 4, 384, 32, "random", "fp32_mfma"),
+    (2, 2, 161, 64, "tail", "fp32_mfma"),
+    (1, 1, 1, 4, "none", "fp32_mfma"),          # a single key
+    (1, 1, 5, 3, "none", "fp32_fma"),           # head_dim 3: rows are not 16-byte multiples -> vector-FMA kernel
+    (1, 2, 130, 128, "random", "fp32_fma"),     # head_dim beyond the matrix-core kernel
+])
+def test_fp32_kernels_match_formula(af3, oracle, B, H, L, D, mask, kernel):
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.float32, seed=L, mask=mask)
+    err = run_case(af3, oracle, q, k, v, m, bias, expect_kernel=kernel)
+    assert err <= 2e-5
+
+
+def test_fp32_kernels_agree_and_cover_bf16_storage(af3, oracle):
+    # the two fp32 kernels on the same problem (the lean op's last argument forces the vector-FMA kernel)
+    q, k, v, m, bias = dev(*rand_inputs(2, 4, 300, 32, torch.float32, seed=31, mask="random"))
+    m[1] = False                                    # a batch row without any live key: mean of V in both
+    a = af3.dot_product_attention_cpp(q, k, v, m, bias)
+    b = torch.ops.af3_kernels.dpa_forward(q, k, v, m.view(torch.uint8), bias, 0, True)
+    torch.cuda.synchronize()
+    assert (a - b).abs().max().item() <= 1e-5
+    assert (a[1] - v[1].mean(dim=1, keepdim=True)).abs().max().item() <= 1e-5
+    # bf16 storage whose head_dim is not a multiple of 8 takes the vector-FMA kernel
     q, k, v, m, bias = rand_inputs(2, 2, 90, 20, torch.bfloat16, seed=11, mask="random")
     run_case(af3, oracle, q, k, v, m, bias, expect_kernel="fp32_fma")
+
+
+def test_fp32_mfma_strided_inputs_and_large_logits(af3, oracle):
+    B, H, L, D = 2, 2, 200, 32
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.float32, seed=41, mask="tail")
+    bias = bias + torch.linspace(-50.0, 70.0, L)[None, None, :]      # the running maximum moves along the row
+    big = torch.zeros(B, H, L + 8, D + 32)
+    big[:, :, :L, :D] = q
+    qv = big.cuda()[:, :, :L, :D]                                     # rows with a larger pitch
+    kv = k.cuda().transpose(0, 1).contiguous().transpose(0, 1)        # permuted batch/head strides
+    assert af3.selected_kernel(qv, kv, v.cuda(), m.cuda(), bias.cuda()) == "fp32_mfma"
+    out = af3.dot_product_attention_cpp(qv, kv, v.cuda(), m.cuda(), bias.cuda())
+    want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), f32np(bias))
+    assert np.abs(f32np(out) - want).max() <= 1e-4
 
 
 def test_fp32_bias_and_other_dtypes_are_cast_like_the_reference(af3, oracle):

@@ -46,6 +46,8 @@ CASES = {
     "cfg4": Case("cfg4", 768, 4, 768, 32, "bf16", "bf16", "bernoulli:0.92", 2, 2e-2),
     # diffusion transformer token attention, fp8 MMA with bf16 I/O
     "cfg5": Case("cfg5", 5, 16, 1536, 24, "bf16", "fp8", "tail:154", 1, 6e-2),
+    # not one of the named configurations: a triangle-attention slab in float32, sized to measure the fp32 matrix-core kernel
+    "fp32_n768": Case("fp32_n768", 64, 4, 768, 32, "fp32", "fp32", "bernoulli:0.92", 2, 1e-4),
 }
 
 

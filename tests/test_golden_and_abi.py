@@ -111,7 +111,9 @@ def test_kernel_selection_is_host_only_and_follows_alignment():
     s96 = (ctypes.c_int64 * 3)(4 * 64 * 96, 64 * 96, 96)
     assert sel(ctypes.byref(_params(D=96, q_stride=s96, k_stride=s96, v_stride=s96, out_stride=s96))) == 0   # head_dim > 64
     assert sel(ctypes.byref(_params(D=96))) == -4                         # rows of 96 with stride 32 overlap
-    assert sel(ctypes.byref(_params(io_dtype=0, mma_dtype=0, out_dtype=0))) == 0
+    assert sel(ctypes.byref(_params(io_dtype=0, mma_dtype=0, out_dtype=0, bias_dtype=0))) == 3   # fp32 storage -> fp32 MFMA
+    assert sel(ctypes.byref(_params(io_dtype=0, mma_dtype=0, out_dtype=0, bias_dtype=0, k=0x2004))) == 0   # rows not 16-byte aligned
+    assert sel(ctypes.byref(_params(io_dtype=0, mma_dtype=0, out_dtype=0, bias_dtype=0, force_generic=1))) == 0
     assert sel(ctypes.byref(_params(L=-1))) == -3
 
 

@@ -53,7 +53,6 @@ namespace af3 {
 constexpr int   KT         = 64;       // keys per tile
 constexpr int   MAX_L_MFMA = 8192;     // mask table (4 B/key) and tile list live in LDS
 constexpr float REF_SLACK  = 12.f;     // log2 units: a moved reference sits this close to the row maximum
-constexpr bool  ROWSUM_MFMA = true;  // row sums of P on the matrix pipe instead of 16 vector adds per sub-tile
 constexpr float PSUM_LIMIT = 0x1p30f;  // per-lane row-sum bound that triggers the rare path
 
 typedef __attribute__((ext_vector_type(2))) __bf16   bf16x2;
@@ -92,10 +91,6 @@ __device__ __forceinline__ float half_swap_max(float x) {
 	// lower half of the other, so (x, x) yields {low|low} and {high|high}.
 	auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
 	return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float half_swap_sum(float x) {
-	auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-	return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 // ---- bias prepass (log2 variant) ---------------------------------------------------------------
@@ -431,8 +426,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	// ---- online-softmax state (per lane: one query row; the two halves hold disjoint keys) ----
 	float  m_ref = 0.f;  // reference maximum: log2 units and bf16-exact (log2 variant), natural units (natural variant)
 	float  mc    = 0.f;  // natural variant: m_ref * log2 e
-	float  l_run = 0.f;
-	f32x4  lacc  = {0.f, 0.f, 0.f, 0.f};  // ROWSUM_MFMA: [0] = this lane's row sum (complete, same in both halves)
+	f32x4  lacc  = {0.f, 0.f, 0.f, 0.f};  // [0] = this lane's row sum (complete: the same value in both half-waves)
 	f32x16 oacc[NDB];
 #pragma unroll
 	for(int db = 0; db < NDB; db++)
@@ -475,7 +469,6 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			m_ref = m_new;
 			mc    = m_new * LOG2E;
 		}
-		l_run *= alpha;
 		lacc[0] *= alpha;
 #pragma unroll
 		for(int db = 0; db < NDB; db++)
@@ -483,10 +476,10 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			for(int i = 0; i < 16; i++) oacc[db][i] *= alpha;
 	};
 
-	// p = exp2(s - reference) for logits [I0, I0+N) of a sub-tile, packed to bf16 pairs, and this
-	// lane's part of the row sum.  (Plain fp32 adds: on gfx950 v_dot2c_f32_bf16 on the packed pairs
-	// would halve the instruction count but does not execute concurrently with MFMA, adds do.)
-	auto exp_part = [&](const f32x16& s, u32x4 (&pf)[2], float& psum, auto i0_c, auto n_c) {
+	// p = exp2(s - reference) for logits [I0, I0+N) of a sub-tile, packed to bf16 pairs.  (The row sum is
+	// taken from the packed pairs on the matrix pipe, rowsum_mfma below: 16 vector adds per sub-tile
+	// cost more, and v_dot2c_f32_bf16 on the pairs does not execute concurrently with MFMA.)
+	auto exp_part = [&](const f32x16& s, u32x4 (&pf)[2], auto i0_c, auto n_c) {
 		constexpr int I0 = decltype(i0_c)::value, N = decltype(n_c)::value;
 #pragma unroll
 		for(int i = I0; i < I0 + N; i += 2) {
@@ -498,7 +491,6 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 				p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], LOG2E, -mc));
 				p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], LOG2E, -mc));
 			}
-			if(!ROWSUM_MFMA) psum += p0 + p1;
 			pf[i >> 3][(i & 7) >> 1] = pack_bf16x2(p0, p1);
 		}
 	};
@@ -593,26 +585,25 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 #define AF3_CHUNK_END() __builtin_amdgcn_sched_barrier(0)
 		AF3_CHUNK_END();
 		// O^T += V^T . P^T of the previous sub-tile, exp2 of this one
-		float psum = 0.f;
 #pragma unroll
 		for(int db = 0; db < NDB; db++)
 			oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[0][db]), __builtin_bit_cast(bf16x8, pprev[0]), oacc[db], 0, 0, 0);
-		exp_part(sc, pcur, psum, ic<0>{}, ic<2>{});
+		exp_part(sc, pcur, ic<0>{}, ic<2>{});
 		AF3_CHUNK_END();
 #pragma unroll
 		for(int db = 0; db < NDB; db++)
 			oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[1][db]), __builtin_bit_cast(bf16x8, pprev[1]), oacc[db], 0, 0, 0);
-		exp_part(sc, pcur, psum, ic<2>{}, ic<2>{});
+		exp_part(sc, pcur, ic<2>{}, ic<2>{});
 		AF3_CHUNK_END();
 		// S^T of the next sub-tile
 		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[0]), qf[0], sn, 0, 0, 0);
 		// V^T fragments of this sub-tile for the next stage's PV product: issued as soon as the two PV
 		// MFMAs above have consumed the previous fragments, a whole stage before their use
 		read_vfrags(v_off, SUBC);
-		exp_part(sc, pcur, psum, ic<4>{}, ic<2>{});
+		exp_part(sc, pcur, ic<4>{}, ic<2>{});
 		AF3_CHUNK_END();
 		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[1]), qf[1], sn, 0, 0, 0);
-		exp_part(sc, pcur, psum, ic<6>{}, ic<2>{});
+		exp_part(sc, pcur, ic<6>{}, ic<2>{});
 		AF3_CHUNK_END();
 #pragma unroll
 		for(int c = 2; c < NC; c++) sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[c]), qf[c], sn, 0, 0, 0);
@@ -620,35 +611,26 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 		// whole stage stays one basic block)
 		sn = bias_mfma(sn, FB);
 		const float l_before = lacc[0];
-		if(ROWSUM_MFMA) rowsum_mfma(pcur[0]);
-		exp_part(sc, pcur, psum, ic<8>{}, ic<2>{});
+		rowsum_mfma(pcur[0]);
+		exp_part(sc, pcur, ic<8>{}, ic<2>{});
 		AF3_CHUNK_END();
 		sn = bias_mfma(sn, FB + 1);
-		exp_part(sc, pcur, psum, ic<10>{}, ic<2>{});
+		exp_part(sc, pcur, ic<10>{}, ic<2>{});
 		AF3_CHUNK_END();
 		if(BIAS_LATE) load_bias_frags(bias_kt, bias_sub_c);  // pair of the sub-tile after the next one
 		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), sn, 0, 0, 0);
-		exp_part(sc, pcur, psum, ic<12>{}, ic<4>{});
+		exp_part(sc, pcur, ic<12>{}, ic<4>{});
 		AF3_CHUNK_END();
 #undef AF3_CHUNK_END
-		if(ROWSUM_MFMA) {
+		rowsum_mfma(pcur[1]);
+		// The running sum stays below L * 2^REF_SLACK <= 2^25 while every probability respects the
+		// reference, so this also catches a single probability near or beyond the limit (inf, NaN).
+		if(__ballot(!(lacc[0] < PSUM_LIMIT))) {  // rare
+			lacc[0] = l_before;
+			rereference(sc, &sn, false);
+			exp_part(sc, pcur, ic<0>{}, ic<16>{});
+			rowsum_mfma(pcur[0]);
 			rowsum_mfma(pcur[1]);
-			// The running sum stays below L * 2^REF_SLACK <= 2^25 while every probability respects the
-			// reference, so this also catches a single probability near or beyond the limit (inf, NaN).
-			if(__ballot(!(lacc[0] < PSUM_LIMIT))) {  // rare
-				lacc[0] = l_before;
-				rereference(sc, &sn, false);
-				exp_part(sc, pcur, psum, ic<0>{}, ic<16>{});
-				rowsum_mfma(pcur[0]);
-				rowsum_mfma(pcur[1]);
-			}
-		} else {
-			if(__ballot(!(psum < PSUM_LIMIT))) {  // a logit far above the reference (or inf / NaN): rare
-				rereference(sc, &sn, false);
-				psum = 0.f;
-				exp_part(sc, pcur, psum, ic<0>{}, ic<16>{});
-			}
-			l_run += psum;
 		}
 		sc       = sn;
 		pprev[0] = pcur[0];
@@ -730,7 +712,6 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 #pragma unroll
 		for(int w = 1; w < NW; w++) mstar = fmaxf(mstar, mred[w * 32 + n]);
 		const float scale_w = my_n > 0 ? __builtin_amdgcn_exp2f((m_ref - mstar) * (L2DOM ? 1.f : LOG2E)) : 0.f;
-		l_run *= scale_w;
 		lacc[0] *= scale_w;
 #pragma unroll
 		for(int db = 0; db < NDB; db++)
@@ -742,7 +723,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			for(int db = 0; db < NDB; db++)
 #pragma unroll
 				for(int i = 0; i < 16; i++) mine[(db * 16 + i) * 64] = oacc[db][i];
-			mine[16 * NDB * 64] = ROWSUM_MFMA ? lacc[0] : l_run;
+			mine[16 * NDB * 64] = lacc[0];
 		}
 		__syncthreads();
 		if(wave > 0) return;
@@ -753,13 +734,12 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			for(int db = 0; db < NDB; db++)
 #pragma unroll
 				for(int i = 0; i < 16; i++) oacc[db][i] += theirs[(db * 16 + i) * 64];
-			l_run += theirs[16 * NDB * 64];
 			lacc[0] += theirs[16 * NDB * 64];
 		}
 	}
 
 	// ---- epilogue: O^T register i of block db is head column 32*db + 8*(i/4) + 4*half + i%4 ----
-	const float l_tot = ROWSUM_MFMA ? lacc[0] : half_swap_sum(l_run);
+	const float l_tot = lacc[0];
 	const float inv   = 1.f / l_tot;
 	if(row_ok) {
 		const int64_t ooff = b * p.out_stride[0] + h * p.out_stride[1] + qrow * p.out_stride[2];

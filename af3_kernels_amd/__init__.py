@@ -3,12 +3,14 @@
 Public names, argument order and defaults follow the reference's Python module
 (src/af3_kernels/__init__.py:31-52, :108-135): `dot_product_attention_cpp`,
 `pad_and_align_tensor`, `vnni_repack_tensor`, `reset_debug_timers`, `print_debug_timers`,
-`print_debug_thread_imbalance`.  Behind them a torch custom op hands raw device pointers to
+`print_debug_thread_imbalance`, and the two fused callers of the attention core, `_attention_cpp` (:55-80)
+and `self_attention_cpp` (:83-105), with `GridSelfAttentionCpp` (src/af3_kernels/Attention.py:23-82).  Behind them a torch custom op hands raw device pointers to
 libaf3_dpa.so (hand-written HIP for gfx950) through the C ABI of include/af3_dpa.h.
 
 Inputs must live on a ROCm device; there is no CPU path and no PyTorch fallback.
 """
 from . import _lib
+from .fused import GridSelfAttentionCpp, _attention_cpp, self_attention_cpp  # noqa: F401
 from .ops import (  # noqa: F401
     convert,
     dot_product_attention_cpp,
@@ -26,5 +28,5 @@ from .ops import (  # noqa: F401
 __all__ = [
     "dot_product_attention_cpp", "dot_product_attention_fp8", "pad_and_align_tensor", "vnni_repack_tensor",
     "reset_debug_timers", "print_debug_timers", "print_debug_thread_imbalance", "convert", "quantize_fp8_e4m3",
-    "selected_kernel", "set_exact_bias",
+    "selected_kernel", "set_exact_bias", "_attention_cpp", "self_attention_cpp", "GridSelfAttentionCpp",
 ]

@@ -9,7 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libaf3_dpa.so")
 
 AF3_F32, AF3_BF16, AF3_FP8_E4M3 = 0, 1, 2
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 i64, i32, f32, vp = ctypes.c_int64, ctypes.c_int32, ctypes.c_float, ctypes.c_void_p
 
@@ -27,6 +27,7 @@ class DpaParams(ctypes.Structure):
         ("device_descales", vp),
         ("workspace", vp), ("workspace_bytes", i64),
         ("q_lo", vp), ("k_lo", vp),
+        ("gate", vp), ("gate_stride", i64 * 3),
     ]
 
 

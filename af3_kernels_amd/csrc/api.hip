@@ -23,6 +23,12 @@ int validate(const af3_dpa_params* p) {
 	}
 	if(p->bias && (p->bias_stride[0] < 0 || p->bias_stride[1] < p->L)) return AF3_ERR_BAD_STRIDE;
 	if(p->key_mask && p->key_mask_stride_b != 0 && p->key_mask_stride_b < p->L) return AF3_ERR_BAD_STRIDE;
+	if(p->gate) {
+		if(p->io_dtype == AF3_FP8_E4M3) return AF3_ERR_BAD_DTYPE;
+		for(int i = 0; i < 3; i++)
+			if(p->gate_stride[i] < 0) return AF3_ERR_BAD_STRIDE;
+		if(p->gate_stride[2] < p->D) return AF3_ERR_BAD_STRIDE;
+	}
 	if(p->out_dtype != AF3_F32 && p->out_dtype != AF3_BF16) return AF3_ERR_BAD_DTYPE;
 	if(p->bias && p->bias_dtype != AF3_F32 && p->bias_dtype != AF3_BF16) return AF3_ERR_BAD_DTYPE;
 	if(!(p->softmax_scale > 0.f) || !(p->softmax_scale < INFINITY)) return AF3_ERR_BAD_ARGUMENT;
@@ -92,4 +98,4 @@ extern "C" const char* af3_status_string(int status) {
 	}
 }
 
-extern "C" int af3_abi_version(void) { return 1; }
+extern "C" int af3_abi_version(void) { return 2; }

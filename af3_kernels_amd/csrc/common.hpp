@@ -40,6 +40,9 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 	return __builtin_bit_cast(uint32_t, p);
 }
 
+// sigmoid for the optional output gate (reference: tpp::SigmoidFwdTPP, src/csrc/xsmm_functors.h:2694-2731)
+__device__ __forceinline__ float sigmoidf_fast(float x) { return 1.f / (1.f + __builtin_amdgcn_exp2f(-x * LOG2E)); }
+
 // Launchers implemented in the .hip files; all validated by api.hip before the call.
 int launch_dpa_generic(const af3_dpa_params& p, hipStream_t s);
 int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s);

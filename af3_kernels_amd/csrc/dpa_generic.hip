@@ -94,7 +94,8 @@ __global__ void __launch_bounds__(GEN_WAVES * 64) dpa_generic_kernel(af3_dpa_par
 	for(int t = 0; t < 2; t++) {
 		const int d = lane + 64 * t;
 		if(d >= D) break;
-		const float o = (t == 0 ? acc0 : acc1) * inv;
+		float o = (t == 0 ? acc0 : acc1) * inv;
+		if(p.gate) o *= sigmoidf_fast(load_as_f32(p.gate, b * p.gate_stride[0] + h * p.gate_stride[1] + row * p.gate_stride[2] + d, p.io_dtype));
 		if(p.out_dtype == AF3_F32) static_cast<float*>(p.out)[ooff + d] = o;
 		else static_cast<uint16_t*>(p.out)[ooff + d] = (uint16_t)f32_to_bf16_bits(o);
 	}

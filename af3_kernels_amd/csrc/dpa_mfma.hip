@@ -749,8 +749,13 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 			for(int g4 = 0; g4 < 4; g4++) {
 				const int d0 = 32 * db + 8 * g4 + 4 * half;
 				if(d0 >= D) continue;
-				const float o0 = oacc[db][4 * g4] * inv, o1 = oacc[db][4 * g4 + 1] * inv;
-				const float o2 = oacc[db][4 * g4 + 2] * inv, o3 = oacc[db][4 * g4 + 3] * inv;
+				float o0 = oacc[db][4 * g4] * inv, o1 = oacc[db][4 * g4 + 1] * inv;
+				float o2 = oacc[db][4 * g4 + 2] * inv, o3 = oacc[db][4 * g4 + 3] * inv;
+				if(p.gate) {  // out *= sigmoid(gate): four consecutive head columns = one 8-byte load
+					const u32x2 gw = *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(p.gate) + b * p.gate_stride[0] + h * p.gate_stride[1] + qrow * p.gate_stride[2] + d0);
+					o0 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] & 0xffffu)), o1 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] >> 16));
+					o2 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] & 0xffffu)), o3 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] >> 16));
+				}
 				if(p.out_dtype == AF3_BF16) {
 					u32x2 w = {pack_bf16x2(o0, o1), pack_bf16x2(o2, o3)};
 					*reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.out) + ooff + d0) = w;
@@ -772,6 +777,7 @@ bool mfma_bf16_eligible(const af3_dpa_params& p) {
 		if(p.q_stride[i] % 8 || p.k_stride[i] % 8 || p.v_stride[i] % 8) return false;
 	// buffer addressing of one (batch, head) slab uses 32-bit byte offsets
 	if(p.L * p.k_stride[2] * 2 >= 0x7fffffffLL || p.L * p.v_stride[2] * 2 >= 0x7fffffffLL) return false;
+	if(p.gate && ((reinterpret_cast<uintptr_t>(p.gate) & 7) || p.gate_stride[0] % 4 || p.gate_stride[1] % 4 || p.gate_stride[2] % 4)) return false;
 	if(p.out_dtype == AF3_BF16) {
 		if((reinterpret_cast<uintptr_t>(p.out) & 7) || p.out_stride[0] % 4 || p.out_stride[1] % 4 || p.out_stride[2] % 4) return false;
 	} else {

@@ -239,7 +239,11 @@ __global__ void __launch_bounds__(F32_NW * 64) dpa_mfma_f32_kernel(af3_dpa_param
 			for(int r4 = 0; r4 < 4; r4++) {
 				const int d0 = 32 * db + 8 * r4 + 4 * half;
 				if(d0 < D) {
-					const float4 w = {oacc[db][4 * r4] * inv, oacc[db][4 * r4 + 1] * inv, oacc[db][4 * r4 + 2] * inv, oacc[db][4 * r4 + 3] * inv};
+					float4 w = {oacc[db][4 * r4] * inv, oacc[db][4 * r4 + 1] * inv, oacc[db][4 * r4 + 2] * inv, oacc[db][4 * r4 + 3] * inv};
+					if(p.gate) {  // out *= sigmoid(gate)
+						const float4 g = *reinterpret_cast<const float4*>(static_cast<const float*>(p.gate) + b * p.gate_stride[0] + h * p.gate_stride[1] + qrow * p.gate_stride[2] + d0);
+						w.x *= sigmoidf_fast(g.x), w.y *= sigmoidf_fast(g.y), w.z *= sigmoidf_fast(g.z), w.w *= sigmoidf_fast(g.w);
+					}
 					*reinterpret_cast<float4*>(op + d0) = w;
 				}
 			}
@@ -266,6 +270,7 @@ bool mfma_f32_eligible(const af3_dpa_params& p) {
 	if(p.io_dtype != AF3_F32 || p.mma_dtype != AF3_F32 || p.out_dtype != AF3_F32) return false;
 	if(p.bias && p.bias_dtype != AF3_F32) return false;
 	if(p.D > 64 || p.D % 4 != 0 || p.L > F32_MAX_L) return false;
+	if(p.gate && ((reinterpret_cast<uintptr_t>(p.gate) & 15) || p.gate_stride[0] % 4 || p.gate_stride[1] % 4 || p.gate_stride[2] % 4)) return false;
 	const void* ptrs[4] = {p.q, p.k, p.v, p.out};
 	for(const void* ptr : ptrs)
 		if(reinterpret_cast<uintptr_t>(ptr) & 15) return false;

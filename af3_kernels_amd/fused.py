@@ -1,0 +1,186 @@
+"""The two fused callers of the attention core, with the reference's names and argument lists:
+
+    _attention_cpp      src/af3_kernels/__init__.py:55-80    -> _attention_impl      (dot_product_attention.cpp:200-378)
+    self_attention_cpp  src/af3_kernels/__init__.py:83-105   -> self_attention_impl  (dot_product_attention.cpp:380-543)
+
+and the module that wraps the first one, GridSelfAttentionCpp (src/af3_kernels/Attention.py:23-82).
+
+On the GPU the op is three launches instead of the reference's per-(row, head) loop nest:
+  1. ONE library GEMM for the four projections (q | k | v | gate): x [rows, C] . W [C, 4C]
+     (hipBLASLt through torch.matmul: a plain GEMM is library territory);
+  2. the attention kernel, reading q, k, v as strided views of that GEMM's output (no
+     "b n (h d) -> b h n d" copies), adding bias and mask, and applying sigmoid(gate) in its
+     epilogue while writing straight into the "b n (h d)" layout;
+  3. the output projection GEMM (grid attention only).
+Weights arrive in the layout the reference's callers produce with vnni_repack_tensor(W.T, 2, C/head)
+and are unpacked once per weight set into the fused [C, 4C] matrix (cached).
+"""
+from typing import Optional
+
+import torch
+
+from . import ops
+
+_W_CACHE = {}
+_W_CACHE_MAX = 64
+
+
+def _unpack_panels(w: torch.Tensor, head: int) -> torch.Tensor:
+    """Inverse of vnni_repack_tensor(W_t, 2, K) (src/csrc/tools.cpp:151-176) for W_t = weight^T [C, C]:
+    the packed tensor holds, per head j, the [C, K] column panel of W_t as [C/2][K][2] (bf16 pairs of
+    consecutive input rows).  float32 weights have a pair size of 1, i.e. panels stored as [C][K]."""
+    C = w.shape[0]
+    K = C // head
+    if w.dtype == torch.bfloat16:
+        return w.reshape(head, C // 2, K, 2).permute(1, 3, 0, 2).reshape(C, C)
+    return w.reshape(head, C, K).permute(1, 0, 2).reshape(C, C)
+
+
+def _fused_weight(ws, head: int, dtype: torch.dtype) -> torch.Tensor:
+    """[C, 4C] = (q | k | v | gate) projection matrices side by side, unpacked from the panel layout."""
+    key = tuple((w.data_ptr(), w._version, tuple(w.shape), w.dtype) for w in ws) + (head, dtype)
+    hit = _W_CACHE.get(key)
+    if hit is None:
+        if len(_W_CACHE) >= _W_CACHE_MAX:
+            _W_CACHE.clear()
+        hit = torch.cat([_unpack_panels(w, head).to(dtype) for w in ws], dim=1).contiguous()
+        _W_CACHE[key] = hit
+    return hit
+
+
+def _check_weights(C: int, head: int, ws):
+    if C % head != 0:
+        raise ValueError(f"channel count {C} is not divisible by head={head}")
+    for w in ws:
+        if w.dim() != 2 or w.shape[0] != C or w.shape[1] != C:
+            raise ValueError(f"projection weights must be [{C}, {C}], got {tuple(w.shape)}")
+        if not w.is_contiguous():
+            raise ValueError("projection weights must be contiguous (they carry a packed layout)")
+
+
+def _attention_cpp(
+    pair: torch.Tensor,
+    mask: torch.Tensor,
+    bias: torch.Tensor,
+    q_proj: torch.Tensor,
+    k_proj: torch.Tensor,
+    v_proj: torch.Tensor,
+    gating_query: torch.Tensor,
+    out_proj: torch.Tensor,
+    head: int,
+    use_flash_attention: bool = False,  # unused, as in the reference
+    BLK_SZ: int = 128,                   # CPU tile size in the reference; no meaning here
+    FLASH_SZ: int = 1024,                # unused, as in the reference
+) -> torch.Tensor:
+    """Grid / triangle self-attention on already normalised pair rows:
+        q, k, v, g = pair . Wq, Wk, Wv, Wg  (per head);  out = (softmax(q k^T K^-1/2 + bias, mask) v * sigmoid(g)) . Wout
+    pair [B, N, C]; mask [B, N] or [N] (truthy = attend); bias [head, N, N]; q_proj, k_proj, v_proj,
+    gating_query: weight^T packed with vnni_repack_tensor(., 2, C/head); out_proj: weight^T [C, C].
+    Returns [B, N, C] in pair's dtype (bfloat16 or float32)."""
+    ops._require_device(pair, mask, bias, q_proj, k_proj, v_proj, gating_query, out_proj)
+    if pair.dim() != 3:
+        raise ValueError(f"pair must be [B, N, C], got {tuple(pair.shape)}")
+    B, N, C = pair.shape
+    _check_weights(C, head, (q_proj, k_proj, v_proj, gating_query, out_proj))
+    dtype = pair.dtype
+    code = ops._DTYPE_CODE.get(dtype)
+    if code not in (ops.AF3_F32, ops.AF3_BF16):
+        raise ValueError(f"unsupported dtype {dtype}: float32 or bfloat16")
+    K = C // head
+    W = _fused_weight((q_proj, k_proj, v_proj, gating_query), head, dtype)
+    y = torch.matmul(pair.reshape(B * N, C), W).view(B, N, 4, head, K)     # q | k | v | gate, each "(h d)"
+    q, k, v, g = (y[:, :, i].permute(0, 2, 1, 3) for i in range(4))        # [B, head, N, K] views, no copies
+    gated = torch.empty(B, N, C, dtype=dtype, device=pair.device)
+    keep = ops._lift_mask(mask, N) if mask is not None else None
+    ops._dpa_forward_impl(q, k, v, keep, bias.to(dtype) if bias is not None else None, code, False, gate=g,
+                          out=gated.view(B, N, head, K).permute(0, 2, 1, 3))
+    return torch.matmul(gated.view(B * N, C), out_proj.to(dtype)).view(B, N, C)
+
+
+def self_attention_cpp(
+    pair: torch.Tensor,
+    mask: torch.Tensor,
+    bias: torch.Tensor,
+    q_proj: torch.Tensor,
+    q_bias: torch.Tensor,
+    k_proj: torch.Tensor,
+    v_proj: torch.Tensor,
+    gating_query: torch.Tensor,
+    head: int,
+    use_flash_attention: bool = False,  # unused, as in the reference
+    BLK_SZ: int = 128,
+    FLASH_SZ: int = 1024,                # unused, as in the reference
+) -> torch.Tensor:
+    """Diffusion-transformer self-attention on one token sequence:
+        q = x . Wq + q_bias;  k, v, g = x . Wk, Wv, Wg;  out = softmax(q k^T K^-1/2 + bias, mask) v * sigmoid(g)
+    pair (x) [N, C]; mask [N]; bias [head, N, N]; q_bias [C] (or [head, C/head]); weights as in
+    _attention_cpp.  Returns [N, C]."""
+    ops._require_device(pair, mask, bias, q_proj, q_bias, k_proj, v_proj, gating_query)
+    if pair.dim() != 2:
+        raise ValueError(f"pair must be [N, C], got {tuple(pair.shape)}")
+    N, C = pair.shape
+    _check_weights(C, head, (q_proj, k_proj, v_proj, gating_query))
+    dtype = pair.dtype
+    code = ops._DTYPE_CODE.get(dtype)
+    if code not in (ops.AF3_F32, ops.AF3_BF16):
+        raise ValueError(f"unsupported dtype {dtype}: float32 or bfloat16")
+    K = C // head
+    W = _fused_weight((q_proj, k_proj, v_proj, gating_query), head, dtype)
+    if q_bias is not None:
+        # the q bias rides the GEMM's epilogue: [q_bias | 0 | 0 | 0] added to every output row
+        row = torch.zeros(4 * C, dtype=dtype, device=pair.device)
+        row[:C] = q_bias.reshape(C).to(dtype)
+        y = torch.addmm(row, pair, W)
+    else:
+        y = torch.matmul(pair, W)
+    y = y.view(1, N, 4, head, K)
+    q, k, v, g = (y[:, :, i].permute(0, 2, 1, 3) for i in range(4))
+    out = torch.empty(N, C, dtype=dtype, device=pair.device)
+    keep = ops._lift_mask(mask, N) if mask is not None else None
+    ops._dpa_forward_impl(q, k, v, keep, bias.to(dtype) if bias is not None else None, code, False, gate=g,
+                          out=out.view(1, N, head, K).permute(0, 2, 1, 3))
+    return out
+
+
+class GridSelfAttentionCpp(torch.nn.Module):
+    """Same constructor, parameters and forward as the reference module (src/af3_kernels/Attention.py:23-82):
+    LayerNorm and the pair-bias projection stay torch ops, the rest is _attention_cpp."""
+
+    def __init__(self, c_pair: int = 128, num_head: int = 4, transpose: bool = False):
+        super().__init__()
+        self.c_pair = c_pair
+        self.num_head = num_head
+        self.qkv_dim = self.c_pair // self.num_head
+        self.transpose = transpose
+        self.act_norm = torch.nn.LayerNorm(self.c_pair)
+        self.pair_bias_projection = torch.nn.Linear(self.c_pair, self.num_head, bias=False)
+        self.q_projection = torch.nn.Linear(self.c_pair, self.c_pair, bias=False)
+        self.k_projection = torch.nn.Linear(self.c_pair, self.c_pair, bias=False)
+        self.v_projection = torch.nn.Linear(self.c_pair, self.c_pair, bias=False)
+        self.gating_query = torch.nn.Linear(self.c_pair, self.c_pair, bias=False)
+        self.output_projection = torch.nn.Linear(self.c_pair, self.c_pair, bias=False)
+        self.first_run = True
+        self.q_proj = self.k_proj = self.v_proj = self.gq = self.out_proj = None
+
+    def _pack(self, linear: torch.nn.Linear) -> torch.Tensor:
+        w_t = linear.weight.T.contiguous()
+        if w_t.dtype == torch.bfloat16:
+            return ops.vnni_repack_tensor(w_t, 2, self.qkv_dim)
+        # float32: one [C, K] panel per head (pair size 1), the layout _attention_impl<float> indexes
+        return w_t.view(self.c_pair, self.num_head, self.qkv_dim).permute(1, 0, 2).contiguous().view(self.c_pair, self.c_pair)
+
+    def _packed_weights(self):
+        """Packed once, on the first forward, like the reference (weights are frozen for inference)."""
+        if self.first_run:
+            self.q_proj, self.k_proj, self.v_proj, self.gq = (
+                self._pack(m) for m in (self.q_projection, self.k_projection, self.v_projection, self.gating_query))
+            self.out_proj = self.output_projection.weight.T.contiguous()
+            self.first_run = False
+        return self.q_proj, self.k_proj, self.v_proj, self.gq, self.out_proj
+
+    def forward(self, pair: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
+        normed = self.act_norm(pair)
+        bias = self.pair_bias_projection(normed).permute(2, 0, 1)          # [head, N, N]
+        rows = normed.transpose(0, 1) if self.transpose else normed         # attend along columns when transposed
+        out = _attention_cpp(rows, mask, bias, *self._packed_weights(), self.num_head, False, 128 if pair.shape[1] > 256 else 64, 0)
+        return out.transpose(0, 1) if self.transpose else out

@@ -113,7 +113,7 @@ def print_debug_thread_imbalance():
 # ------------------------------------------------------------------------------------------
 # attention
 # ------------------------------------------------------------------------------------------
-def _fill_params(q, k, v, keep, bias, out, mma_dtype, force_generic, descales=None, softmax_scale=None, v_transposed=False) -> DpaParams:
+def _fill_params(q, k, v, keep, bias, out, mma_dtype, force_generic, descales=None, softmax_scale=None, v_transposed=False, gate=None) -> DpaParams:
     B, H, L, D = q.shape
     p = DpaParams()
     p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
@@ -137,6 +137,9 @@ def _fill_params(q, k, v, keep, bias, out, mma_dtype, force_generic, descales=No
     p.force_generic = int(bool(force_generic))
     if descales is not None:
         p.device_descales = descales.data_ptr()
+    if gate is not None:
+        p.gate = gate.data_ptr()
+        p.gate_stride = (ctypes.c_int64 * 3)(*gate.stride()[:3])
     return p
 
 
@@ -168,18 +171,25 @@ def set_exact_bias(flag: bool) -> bool:
     return prev
 
 
-def _dpa_forward_impl(q, k, v, keep, bias, mma_dtype: int, force_generic: bool) -> torch.Tensor:
-    _require_device(q, k, v, keep, bias)
+def _dpa_forward_impl(q, k, v, keep, bias, mma_dtype: int, force_generic: bool, gate=None, out=None) -> torch.Tensor:
+    """gate: optional [B,H,L,D] pre-activation values, the result is multiplied by sigmoid(gate) in the
+    kernel's epilogue; out: optional preallocated (possibly strided, innermost stride 1) result view."""
+    _require_device(q, k, v, keep, bias, gate, out)
     q, k, v = _inner_contig(q), _inner_contig(k), _inner_contig(v)
+    if gate is not None and (gate.stride(-1) != 1 or tuple(gate.shape) != tuple(q.shape) or gate.dtype != q.dtype):
+        raise ValueError("gate must have q's shape and dtype with a unit innermost stride")
+    if out is not None and (out.stride(-1) != 1 or tuple(out.shape) != tuple(q.shape)):
+        raise ValueError("out must have q's shape with a unit innermost stride")
     if bias is not None:
         bias = _inner_contig(bias)
     if keep is not None:
         keep = _inner_contig(keep)
     _check_shapes(q, k, v, keep, bias)
-    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     if q.numel() == 0:
         return out
-    p = _fill_params(q, k, v, keep, bias, out, mma_dtype, force_generic)
+    p = _fill_params(q, k, v, keep, bias, out, mma_dtype, force_generic, gate=gate)
     lib = _lib.load()
     ws_bytes = lib.af3_dpa_workspace_bytes(ctypes.byref(p))
     if ws_bytes > 0 and not _exact_bias:

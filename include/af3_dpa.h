@@ -115,6 +115,14 @@ typedef struct af3_dpa_params {
 	 * that recover about six mantissa bits for q and k. */
 	const void*    q_lo;
 	const void*    k_lo;
+	/* Optional output gate (ABI version 2): out = sigmoid(gate) * (softmax(...) . v), the
+	 * "weighted_avg *= sigmoid(gating_query(pair))" step of the reference's fused grid attention
+	 * (src/csrc/dot_product_attention.cpp:335-349), applied in the kernel's epilogue so the
+	 * un-gated result never goes to memory.  gate: [B, H, L, D] pre-activation values of io_dtype
+	 * with element strides for B, H and L (innermost 1), 8-byte aligned rows.  NULL: no gate.
+	 * Not available for fp8 inputs. */
+	const void*    gate;
+	int64_t        gate_stride[3];
 } af3_dpa_params;
 
 /*

@@ -491,3 +491,193 @@ int af3o_dpa_formula(const float* q, const float* k, const float* v, const float
 	}
 	return fail ? -1 : 0;
 }
+
+/* ---- the two fused callers of the core ("next" rows) ------------------------------------ */
+
+/* SigmoidFwdTPP::ref, xsmm_functors.h:2717-2723: out = 1 / (1 + exp(-in)), stored as T. */
+void af3o_sigmoid(const float* in, float* out, int64_t n, int dtype) {
+	for(int64_t i = 0; i < n; i++) {
+		out[i] = round_T((float)(1. / (1. + exp(-(double)in[i]))), dtype);
+	}
+}
+
+/* MulTPP::ref, xsmm_functors.h:1269-1275: out = in0 * in1, stored as T. */
+void af3o_mul(const float* in0, const float* in1, float* out, int64_t n, int dtype) {
+	for(int64_t i = 0; i < n; i++) {
+		out[i] = round_T(in0[i] * in1[i], dtype);
+	}
+}
+
+/*
+ * Restatement of the two fused attention drivers:
+ *   _attention_impl<T>      src/csrc/dot_product_attention.cpp:200-378  (wo != NULL, qbias == NULL)
+ *   self_attention_impl<T>  src/csrc/dot_product_attention.cpp:380-543  (B == 1, wo == NULL, qbias optional)
+ *
+ *   x     : [B, L, C] input rows (the normalised pair rows / the single representation)
+ *   keep  : [B, L] bytes, non-zero = attend
+ *   bias  : [H, L, L]
+ *   wq, wk, wv, wg : [C, C] = weight^T, natural row-major layout; head j uses columns j*K .. j*K+K-1,
+ *           i.e. the [C, K] panel the reference addresses as q_a[j] (:241-244, :418-423) after its
+ *           VNNI repack of the same matrix (the repack itself is af3o_vnni_repack)
+ *   wo    : [C, C] = output_projection.weight^T or NULL
+ *   qbias : [C] or NULL (added to q before the scaling, :490-492)
+ *   out   : [B, L, C]
+ *
+ * Per (row i, head j), with every stored intermediate rounded to T as the reference stores a T:
+ *   :290-303 / :461-476  k, v = x_i . Wk_j, x_i . Wv_j over the whole padded row
+ *   :306-310 / :471-476  q = x_tile . Wq_j          (:490-492 q += q_bias)
+ *   :311-314 / :493-496  q *= K^-1/2
+ *   :315-319 / :497-501  logits = q . k^T
+ *   :320-326 / :502-507  logits += bias ; logits += mask * -1e9
+ *   :331-333 / :508-510  softmax over the padded row
+ *   :334-338 / :511-515  weighted = P . v
+ *   :339-349 / :516-527  gate = sigmoid(x_tile . Wg_j) ; out_a = weighted * gate
+ *   :356-372             out = out_a . Wo   (_attention only)
+ * M = ceil(L/BLK)*BLK; padded input rows are zero, padded mask entries dropped, padded bias 0.
+ * Returns 0, or -1 on allocation failure.
+ */
+int af3o_fused_attention_reference(const float* x, const uint8_t* keep, const float* bias, const float* wq, const float* wk, const float* wv, const float* wg,
+								   const float* wo, const float* qbias, float* out, int64_t B, int64_t L, int64_t C, int64_t H, int dtype, int64_t BLK) {
+	const int64_t K = C / H, M = (L + BLK - 1) / BLK * BLK, Mb = M / BLK;
+	float*        xp = (float*)calloc((size_t)(B * M * C), sizeof(float));
+	float*        bp = (float*)calloc((size_t)(H * M * M), sizeof(float));
+	float*        mp = (float*)malloc(sizeof(float) * (size_t)(B * M));
+	float*        oa = (float*)calloc((size_t)(B * M * C), sizeof(float));
+	if(!xp || !bp || !mp || !oa) {
+		free(xp), free(bp), free(mp), free(oa);
+		return -1;
+	}
+	for(int64_t i = 0; i < B; i++) af3o_pad_2d(x + i * L * C, xp + i * M * C, L, C, M, C, 0.0f);
+	for(int64_t h = 0; h < H; h++) af3o_pad_2d(bias + h * L * L, bp + h * M * M, L, L, M, M, 0.0f);
+	for(int64_t i = 0; i < B; i++) {
+		for(int64_t c = 0; c < M; c++) mp[i * M + c] = (c < L && keep[i * L + c]) ? 0.0f : 1.0f;
+		af3o_scale(mp + i * M, mp + i * M, M, -1e9f, dtype);
+	}
+	const float scaling = 1.0f / sqrtf((float)K);
+	int         fail    = 0;
+#pragma omp parallel for schedule(dynamic)
+	for(int64_t t = 0; t < B * H; t++) {
+		const int64_t i = t / H, j = t % H;
+		float*        tk = (float*)malloc(sizeof(float) * (size_t)(M * K));
+		float*        tv = (float*)malloc(sizeof(float) * (size_t)(M * K));
+		float*        tq = (float*)malloc(sizeof(float) * (size_t)(BLK * K));
+		float*        to = (float*)malloc(sizeof(float) * (size_t)(BLK * (M > K ? M : K)));
+		if(!tk || !tv || !tq || !to) {
+			free(tk), free(tv), free(tq), free(to);
+			fail = 1;
+			continue;
+		}
+		const float* xi = xp + i * M * C;
+		af3o_brgemm(xi, wk + j * K, tk, (int)M, (int)K, (int)C, (int)C, (int)C, (int)K, 0, dtype);
+		af3o_brgemm(xi, wv + j * K, tv, (int)M, (int)K, (int)C, (int)C, (int)C, (int)K, 0, dtype);
+		for(int64_t kb = 0; kb < Mb; kb++) {
+			const float* xt = xi + kb * BLK * C;
+			af3o_brgemm(xt, wq + j * K, tq, (int)BLK, (int)K, (int)C, (int)C, (int)C, (int)K, 0, dtype);
+			if(qbias) af3o_add_bias(qbias + j * K, tq, (int)BLK, (int)K, (int)K, dtype);
+			af3o_scale(tq, tq, BLK * K, scaling, dtype);
+			af3o_brgemm(tq, tk, to, (int)BLK, (int)M, (int)K, (int)K, (int)K, (int)M, 1, dtype);
+			af3o_add(bp + (j * M + kb * BLK) * M, to, to, 1, (int)(BLK * M), 0, 0, 0, dtype);
+			af3o_add_bias(mp + i * M, to, (int)BLK, (int)M, (int)M, dtype);
+			af3o_softmax_fwd(to, to, (int)BLK, (int)M, (int)M, dtype);
+			af3o_brgemm(to, tv, tq, (int)BLK, (int)K, (int)M, (int)M, (int)K, (int)K, 0, dtype);
+			af3o_brgemm(xt, wg + j * K, to, (int)BLK, (int)K, (int)C, (int)C, (int)C, (int)K, 0, dtype);
+			af3o_sigmoid(to, to, BLK * K, dtype);
+			for(int64_t r = 0; r < BLK; r++) af3o_mul(to + r * K, tq + r * K, oa + (i * M + kb * BLK + r) * C + j * K, K, dtype);
+		}
+		free(tk), free(tv), free(tq), free(to);
+	}
+	if(!fail) {
+		for(int64_t i = 0; i < B; i++) {
+			if(wo) {
+				float* row = (float*)malloc(sizeof(float) * (size_t)(M * C));
+				if(!row) {
+					fail = 1;
+					break;
+				}
+				af3o_brgemm(oa + i * M * C, wo, row, (int)M, (int)C, (int)C, (int)C, (int)C, (int)C, 0, dtype);
+				memcpy(out + i * L * C, row, sizeof(float) * (size_t)(L * C)); /* narrow(1, 0, Mp) */
+				free(row);
+			} else {
+				memcpy(out + i * L * C, oa + i * M * C, sizeof(float) * (size_t)(L * C));
+			}
+		}
+	}
+	free(xp), free(bp), free(mp), free(oa);
+	return fail ? -1 : 0;
+}
+
+/*
+ * Ground truth of the two fused callers in double precision: the torch modules of the reference's
+ * own harnesses (examples/grid_self_attention.py:46-94 without the LayerNorm / bias projection that
+ * precede the op, examples/self_attention.py:64-96), evaluated on the given fp32 values and rounded
+ * once to fp32.  Same arguments as af3o_fused_attention_reference.
+ */
+int af3o_fused_attention_formula(const float* x, const uint8_t* keep, const float* bias, const float* wq, const float* wk, const float* wv, const float* wg,
+								 const float* wo, const float* qbias, float* out, int64_t B, int64_t L, int64_t C, int64_t H) {
+	const int64_t K = C / H;
+	double*       ga = (double*)malloc(sizeof(double) * (size_t)(B * L * C)); /* gated weighted average */
+	if(!ga) return -1;
+	int fail = 0;
+#pragma omp parallel for schedule(dynamic)
+	for(int64_t t = 0; t < B * H; t++) {
+		const int64_t i = t / H, j = t % H;
+		double*       q = (double*)malloc(sizeof(double) * (size_t)(L * K) * 4);
+		double*       w = (double*)malloc(sizeof(double) * (size_t)L);
+		if(!q || !w) {
+			free(q), free(w);
+			fail = 1;
+			continue;
+		}
+		double *k = q + L * K, *v = k + L * K, *g = v + L * K;
+		for(int64_t r = 0; r < L; r++) {
+			for(int64_t d = 0; d < K; d++) {
+				double sq = qbias ? (double)qbias[j * K + d] : 0.0, sk = 0.0, sv = 0.0, sg = 0.0;
+				for(int64_t c = 0; c < C; c++) {
+					const double xv = (double)x[(i * L + r) * C + c];
+					sq += xv * (double)wq[c * C + j * K + d];
+					sk += xv * (double)wk[c * C + j * K + d];
+					sv += xv * (double)wv[c * C + j * K + d];
+					sg += xv * (double)wg[c * C + j * K + d];
+				}
+				q[r * K + d] = sq / sqrt((double)K), k[r * K + d] = sk, v[r * K + d] = sv, g[r * K + d] = 1.0 / (1.0 + exp(-sg));
+			}
+		}
+		for(int64_t r = 0; r < L; r++) {
+			double mx = -INFINITY, sum = 0.0;
+			for(int64_t c = 0; c < L; c++) {
+				double sdot = 0.0;
+				for(int64_t d = 0; d < K; d++) sdot += q[r * K + d] * k[c * K + d];
+				sdot += (double)bias[(j * L + r) * L + c];
+				if(!keep[i * L + c]) sdot = -1e9;
+				w[c] = sdot;
+				if(sdot > mx) mx = sdot;
+			}
+			for(int64_t c = 0; c < L; c++) {
+				w[c] = exp(w[c] - mx);
+				sum += w[c];
+			}
+			for(int64_t d = 0; d < K; d++) {
+				double acc = 0.0;
+				for(int64_t c = 0; c < L; c++) acc += w[c] * v[c * K + d];
+				ga[(i * L + r) * C + j * K + d] = acc / sum * g[r * K + d];
+			}
+		}
+		free(q), free(w);
+	}
+	if(!fail) {
+#pragma omp parallel for schedule(static)
+		for(int64_t r = 0; r < B * L; r++) {
+			for(int64_t o = 0; o < C; o++) {
+				if(wo) {
+					double acc = 0.0;
+					for(int64_t c = 0; c < C; c++) acc += ga[r * C + c] * (double)wo[c * C + o];
+					out[r * C + o] = (float)acc;
+				} else {
+					out[r * C + o] = (float)ga[r * C + o];
+				}
+			}
+		}
+	}
+	free(ga);
+	return fail ? -1 : 0;
+}

@@ -55,6 +55,10 @@ def lib():
         L.af3o_pad_2d.argtypes = [fp, fp, i64, i64, i64, i64, ctypes.c_float]
         L.af3o_softmax_fwd.argtypes = [fp, fp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         L.af3o_brgemm.argtypes = [fp, fp, fp] + [ctypes.c_int] * 8
+        L.af3o_fused_attention_reference.argtypes = [fp, u8, fp, fp, fp, fp, fp, fp, fp, fp, i64, i64, i64, i64, ctypes.c_int, i64]
+        L.af3o_fused_attention_reference.restype = ctypes.c_int
+        L.af3o_fused_attention_formula.argtypes = [fp, u8, fp, fp, fp, fp, fp, fp, fp, fp, i64, i64, i64, i64]
+        L.af3o_fused_attention_formula.restype = ctypes.c_int
         _lib = L
     return _lib
 
@@ -98,6 +102,38 @@ def dpa_formula(q, k, v, mask, bias):
     if rc != 0:
         raise MemoryError("af3o_dpa_formula failed")
     return out
+
+
+def _fused(fn, x, mask, bias, wq, wk, wv, wg, wo, qbias, head, extra):
+    x = np.asarray(x, dtype=np.float32)
+    squeeze = x.ndim == 2                      # the diffusion op has no batch axis: [N, C]
+    if squeeze:
+        x = x[None]
+    B, L, C = x.shape
+    x, xp = _f(x); bias, bp = _f(bias)
+    ws = [_f(w) for w in (wq, wk, wv, wg)]
+    null = ctypes.POINTER(ctypes.c_float)()
+    wo_a, wo_p = _f(wo) if wo is not None else (None, null)
+    qb_a, qb_p = _f(qbias) if qbias is not None else (None, null)
+    m, mp = _keep(mask, B, L)
+    out = np.empty((B, L, C), np.float32)
+    rc = fn(xp, mp, bp, ws[0][1], ws[1][1], ws[2][1], ws[3][1], wo_p, qb_p, out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), B, L, C, head, *extra)
+    if rc != 0:
+        raise MemoryError("fused attention oracle failed")
+    return out[0] if squeeze else out
+
+
+def fused_attention_reference(x, mask, bias, wq, wk, wv, wg, wo=None, qbias=None, head=4, dtype=BF16, BLK_SZ=128):
+    """Restatement of _attention_impl<T> (wo given; dot_product_attention.cpp:200-378) and of
+    self_attention_impl<T> (x [N, C], qbias; :380-543) with the reference's roundings to T.
+    Weights are weight^T in natural [C_in, C_out] layout; head j uses output columns j*K .. j*K+K-1."""
+    return _fused(lib().af3o_fused_attention_reference, x, mask, bias, wq, wk, wv, wg, wo, qbias, head, (dtype, BLK_SZ))
+
+
+def fused_attention_formula(x, mask, bias, wq, wk, wv, wg, wo=None, qbias=None, head=4):
+    """The torch modules of examples/grid_self_attention.py:46-94 (after LayerNorm and bias projection)
+    and examples/self_attention.py:64-96 in double precision."""
+    return _fused(lib().af3o_fused_attention_formula, x, mask, bias, wq, wk, wv, wg, wo, qbias, head, ())
 
 
 def f32_to_bf16_bits(x):

@@ -1,0 +1,213 @@
+"""GPU parity tests for the two fused callers of the attention core, _attention_cpp (grid / triangle
+self-attention) and self_attention_cpp (diffusion transformer), and for the GridSelfAttentionCpp module,
+against the CPU oracle's fp64 formula on the same seeded inputs.
+
+Tolerances, max-abs against the formula evaluated on the inputs the device saw, relative to max(1, |out|max):
+2e-4 for float32 and 3e-2 for bfloat16 (the op rounds q, k, v, the gate and the gated result to bfloat16 like the
+reference does, so its budget is wider than the bare attention core's 2e-2), plus a summed relative error
+<= 1e-2 for bfloat16; the bf16 result must also be no worse than twice the error of the reference's own
+arithmetic restated on the CPU (oracle.fused_attention_reference).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def af3():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import af3_kernels_amd
+    af3_kernels_amd._lib.load()   # raises if libaf3_dpa.so is missing: no fallback
+    return af3_kernels_amd
+
+
+def f32np(t):
+    return t.detach().float().cpu().numpy()
+
+
+def pack(af3, w_t, head):
+    """weight^T [C, C] -> the layout the reference's callers hand over: vnni_repack_tensor(W.T, 2, C/head) for
+    bfloat16, one [C, C/head] panel per head for float32."""
+    C = w_t.shape[0]
+    if w_t.dtype == torch.bfloat16:
+        return af3.vnni_repack_tensor(w_t.contiguous(), 2, C // head)
+    return w_t.view(C, head, C // head).permute(1, 0, 2).contiguous().view(C, C)
+
+
+def make(B, N, C, head, dtype, seed, with_out, with_qbias, mask_p=0.85, mask_rank=2, bias_scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    shape = (B, N, C) if B is not None else (N, C)
+    x = torch.randn(*shape, generator=g).to(dtype)
+    ws = [(torch.randn(C, C, generator=g) / C ** 0.5).to(dtype) for _ in range(5)]
+    bias = (bias_scale * torch.randn(head, N, N, generator=g)).to(dtype)
+    mshape = (N,) if (B is None or mask_rank == 1) else (B, N)
+    mask = torch.rand(*mshape, generator=g) < mask_p
+    mask[..., 0] = True
+    qb = torch.randn(C, generator=g).to(dtype) if with_qbias else None
+    return x, mask, bias, ws[0], ws[1], ws[2], ws[3], (ws[4] if with_out else None), qb
+
+
+def check(got, want, ref, dtype):
+    got = f32np(got)
+    assert np.isfinite(got).all()
+    scale = max(1.0, float(np.abs(want).max()))
+    err = float(np.abs(got - want).max())
+    if dtype == torch.float32:
+        assert err <= 2e-4 * scale, f"max abs err {err}"
+        return
+    assert err <= 3e-2 * scale, f"max abs err {err} (scale {scale})"
+    rel = float(np.abs(got - want).sum() / np.abs(want).sum())
+    assert rel <= 1e-2, f"summed relative error {rel}"
+    if ref is not None:
+        ref_err = float(np.abs(ref - want).max())
+        assert err <= 2.0 * ref_err + 4e-3 * scale, f"device error {err} vs the reference arithmetic's {ref_err}"
+
+
+GRID_CASES = [
+    # B, N, C, head, dtype
+    (4, 72, 128, 4, torch.bfloat16),     # the module's shape family: c_pair 128, 4 heads of 32
+    (9, 200, 128, 4, torch.bfloat16),
+    (3, 37, 128, 4, torch.bfloat16),     # odd row count: the reference pads to BLK_SZ, the kernel masks its tail tile
+    (2, 96, 64, 2, torch.bfloat16),
+    (1, 130, 96, 4, torch.bfloat16),     # 24 channels per head
+    (2, 64, 128, 4, torch.float32),
+    (3, 45, 64, 4, torch.float32),       # 16 channels per head
+]
+
+
+@pytest.mark.parametrize("B,N,C,head,dtype", GRID_CASES)
+def test_attention_cpp_matches_formula(af3, oracle, B, N, C, head, dtype):
+    x, mask, bias, wq, wk, wv, wg, wo, _ = make(B, N, C, head, dtype, seed=B * 1000 + N, with_out=True, with_qbias=False)
+    print(f"_attention_cpp B,N,C,head={B, N, C, head} {dtype}", flush=True)
+    d = lambda t: t.cuda()
+    out = af3._attention_cpp(d(x), d(mask), d(bias), pack(af3, d(wq), head), pack(af3, d(wk), head), pack(af3, d(wv), head),
+                             pack(af3, d(wg), head), d(wo), head, False, 128 if N > 256 else 64, 0)
+    torch.cuda.synchronize()
+    assert out.shape == x.shape and out.dtype == dtype and out.is_cuda
+    args = [f32np(t) if t is not None and t.dtype != torch.bool else (t.numpy() if t is not None else None) for t in (x, mask, bias, wq, wk, wv, wg, wo)]
+    want = oracle.fused_attention_formula(*args, None, head=head)
+    ref = oracle.fused_attention_reference(*args, None, head=head, dtype=oracle.BF16, BLK_SZ=64) if dtype == torch.bfloat16 else None
+    check(out, want, ref, dtype)
+
+
+SELF_CASES = [
+    # N, C, head, dtype
+    (64, 768, 16, torch.bfloat16),       # the diffusion transformer's shape: 16 heads of 48 channels
+    (200, 768, 16, torch.bfloat16),
+    (77, 256, 8, torch.bfloat16),
+    (150, 128, 4, torch.float32),
+]
+
+
+@pytest.mark.parametrize("N,C,head,dtype", SELF_CASES)
+def test_self_attention_cpp_matches_formula(af3, oracle, N, C, head, dtype):
+    x, mask, bias, wq, wk, wv, wg, _, qb = make(None, N, C, head, dtype, seed=N + C, with_out=False, with_qbias=True)
+    print(f"self_attention_cpp N,C,head={N, C, head} {dtype}", flush=True)
+    d = lambda t: t.cuda()
+    out = af3.self_attention_cpp(d(x), d(mask), d(bias), pack(af3, d(wq), head), d(qb), pack(af3, d(wk), head), pack(af3, d(wv), head),
+                                 pack(af3, d(wg), head), head, False, 64, 0)
+    torch.cuda.synchronize()
+    assert out.shape == x.shape and out.dtype == dtype
+    args = [f32np(x), mask.numpy(), f32np(bias), f32np(wq), f32np(wk), f32np(wv), f32np(wg), None, f32np(qb)]
+    want = oracle.fused_attention_formula(*args, head=head)
+    ref = oracle.fused_attention_reference(*args, head=head, dtype=oracle.BF16, BLK_SZ=64) if dtype == torch.bfloat16 else None
+    check(out, want, ref, dtype)
+
+
+def test_attention_cpp_mask_ranks_and_weight_cache(af3, oracle):
+    """A 1-D mask is broadcast over the batch; a fully masked row set still yields finite values; changing a weight
+    in place is seen by the next call (the fused weight matrix is cached per weight version)."""
+    B, N, C, head = 3, 48, 128, 4
+    x, mask, bias, wq, wk, wv, wg, wo, _ = make(B, N, C, head, torch.bfloat16, 11, True, False, mask_rank=1)
+    d = lambda t: t.cuda()
+    packed = [pack(af3, d(w), head) for w in (wq, wk, wv, wg)]
+    run = lambda m: af3._attention_cpp(d(x), d(m), d(bias), *packed, d(wo), head)
+    a = run(mask)
+    b = run(mask[None].expand(B, N).contiguous())
+    assert torch.equal(a, b)
+    want = oracle.fused_attention_formula(f32np(x), mask.numpy(), f32np(bias), f32np(wq), f32np(wk), f32np(wv), f32np(wg), f32np(wo), None, head=head)
+    check(a, want, None, torch.bfloat16)
+    none = torch.zeros(N, dtype=torch.bool)
+    assert torch.isfinite(run(none)).all()
+    packed[2].mul_(2.0)                      # doubling the value projection doubles the result before the gate and out-proj
+    c = run(mask)
+    assert np.abs(f32np(c) - 2.0 * f32np(a)).max() <= 3e-2 * max(1.0, 2.0 * float(np.abs(want).max()))
+
+
+def test_attention_cpp_rejects_malformed_calls(af3):
+    C, head = 64, 4
+    x = torch.randn(2, 16, C, device="cuda", dtype=torch.bfloat16)
+    w = torch.randn(C, C, device="cuda", dtype=torch.bfloat16)
+    mask, bias = torch.ones(2, 16, dtype=torch.bool, device="cuda"), torch.zeros(head, 16, 16, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        af3._attention_cpp(x, mask, bias, w, w, w, w, w, 5)                    # channels not divisible by the head count
+    with pytest.raises(ValueError):
+        af3._attention_cpp(x, mask, bias, w[:, :32], w, w, w, w, head)         # wrong weight shape
+    with pytest.raises(ValueError):
+        af3._attention_cpp(x[0], mask, bias, w, w, w, w, w, head)              # pair without a batch axis
+    with pytest.raises(RuntimeError):
+        af3._attention_cpp(x.cpu(), mask, bias, w, w, w, w, w, head)           # no CPU path
+    with pytest.raises(ValueError):
+        af3.self_attention_cpp(x, mask[0], bias, w, None, w, w, w, head)       # the diffusion op takes [N, C]
+
+
+@pytest.mark.parametrize("transpose", [False, True])
+def test_grid_self_attention_module_matches_torch_module_math(af3, oracle, transpose):
+    """The module against the same layers evaluated with the oracle: LayerNorm and the bias projection are torch
+    ops on both sides (computed once on the device and shared), the attention block is the oracle's formula."""
+    N, C, head = 56, 128, 4
+    torch.manual_seed(3)
+    mod = af3.GridSelfAttentionCpp(C, head, transpose=transpose).cuda().to(torch.bfloat16).eval()
+    with torch.no_grad():
+        for lin in (mod.q_projection, mod.k_projection, mod.v_projection, mod.gating_query, mod.output_projection, mod.pair_bias_projection):
+            lin.weight.normal_(0.0, C ** -0.5)
+        pair = torch.randn(N, N, C, device="cuda").to(torch.bfloat16)
+        mask = torch.rand(N, N, device="cuda") < 0.9
+        mask[:, 0] = True
+        out = mod(pair, mask)
+        torch.cuda.synchronize()
+        assert out.shape == pair.shape and out.dtype == torch.bfloat16
+        normed = mod.act_norm(pair)
+        bias = mod.pair_bias_projection(normed).permute(2, 0, 1)
+        rows = normed.transpose(0, 1) if transpose else normed
+        wt = lambda lin: f32np(lin.weight.T)
+        want = oracle.fused_attention_formula(f32np(rows), mask.cpu().numpy(), f32np(bias), wt(mod.q_projection), wt(mod.k_projection),
+                                              wt(mod.v_projection), wt(mod.gating_query), wt(mod.output_projection), None, head=head)
+        if transpose:
+            want = want.transpose(1, 0, 2)
+    check(out, want, None, torch.bfloat16)
+    # second call reuses the packed weights
+    assert mod.first_run is False and mod.q_proj is not None
+    with torch.no_grad():
+        assert torch.equal(mod(pair, mask), out)
+
+
+@pytest.mark.parametrize("dtype,force_generic,D", [(torch.bfloat16, False, 32), (torch.bfloat16, False, 64), (torch.float32, False, 32),
+                                                   (torch.float32, True, 32), (torch.bfloat16, True, 24), (torch.float32, True, 7)])
+def test_output_gate_in_every_kernel(af3, oracle, dtype, force_generic, D):
+    """out = attention * sigmoid(gate), with strided q/k/v/gate views of one buffer and a strided output view, in
+    the bf16 MFMA, fp32 MFMA and generic kernels."""
+    from af3_kernels_amd import ops
+    B, H, L = 3, 4, 150
+    g = torch.Generator().manual_seed(D)
+    y = torch.randn(B, L, 4, H, D, generator=g).to(dtype)
+    bias = torch.randn(H, L, L, generator=g).to(dtype)
+    mask = torch.rand(B, L, generator=g) < 0.8
+    mask[:, 0] = True
+    dy = y.cuda()
+    q, k, v, gate = (dy[:, :, i].permute(0, 2, 1, 3) for i in range(4))
+    out = torch.zeros(B, L, H * D, dtype=dtype, device="cuda")
+    code = ops._DTYPE_CODE[dtype]
+    print(f"gate {dtype} generic={force_generic} D={D}", flush=True)
+    ops._dpa_forward_impl(q, k, v, ops._lift_mask(mask.cuda(), L), bias.cuda(), code, force_generic, gate=gate, out=out.view(B, L, H, D).permute(0, 2, 1, 3))
+    torch.cuda.synchronize()
+    hq, hk, hv, hg = (f32np(y[:, :, i].permute(0, 2, 1, 3)) for i in range(4))
+    want = oracle.dpa_formula(hq, hk, hv, mask.numpy(), f32np(bias)) / (1.0 + np.exp(-hg.astype(np.float64)))
+    got = f32np(out.view(B, L, H, D).permute(0, 2, 1, 3))
+    err = float(np.abs(got - want).max())
+    assert err <= (1e-4 if dtype == torch.float32 else 2e-2), f"max abs err {err}"
+    # the same call without a gate is the bare attention
+    plain = ops._dpa_forward_impl(q, k, v, ops._lift_mask(mask.cuda(), L), bias.cuda(), code, force_generic)
+    assert float(np.abs(f32np(plain) - oracle.dpa_formula(hq, hk, hv, mask.numpy(), f32np(bias))).max()) <= (1e-4 if dtype == torch.float32 else 2e-2)

@@ -60,8 +60,8 @@ def test_library_exports_every_declared_symbol():
 def test_params_struct_matches_header_layout():
     from af3_kernels_amd._lib import DpaParams
     # 6 pointers, 4 dims, 4*3 + 2 + 1 strides (int64), 4 int32, 4 floats, 2 int32, 2 pointers, 1 int64, 2 pointers
-    assert ctypes.sizeof(DpaParams) == 6 * 8 + 4 * 8 + 15 * 8 + 4 * 4 + 4 * 4 + 2 * 4 + 8 + 8 + 8 + 8 + 8
-    assert DpaParams.k_lo.offset == ctypes.sizeof(DpaParams) - 8
+    assert ctypes.sizeof(DpaParams) == 6 * 8 + 4 * 8 + 15 * 8 + 4 * 4 + 4 * 4 + 2 * 4 + 8 + 8 + 8 + 8 + 8 + 8 + 3 * 8
+    assert DpaParams.gate.offset == ctypes.sizeof(DpaParams) - 32 and DpaParams.k_lo.offset == DpaParams.gate.offset - 8
 
 
 def _params(**kw):

@@ -221,3 +221,97 @@ def test_pad_2d(oracle):
     want = np.ones((4, 5), np.float32)
     want[:2, :3] = x
     assert np.array_equal(got, want)
+
+
+# ------------------------------------------------------------------------------------------
+# fused callers: grid self-attention (_attention_impl) and diffusion self-attention (self_attention_impl)
+# ------------------------------------------------------------------------------------------
+def fused_case(rng, B, L, C, head, with_out=True, with_qbias=False, mask_p=0.8):
+    x = rng.standard_normal((B, L, C)).astype(np.float32)
+    ws = [(rng.standard_normal((C, C)) / np.sqrt(C)).astype(np.float32) for _ in range(5)]
+    bias = rng.standard_normal((head, L, L)).astype(np.float32)
+    mask = rng.random((B, L)) < mask_p
+    mask[:, 0] = True
+    qb = rng.standard_normal(C).astype(np.float32) if with_qbias else None
+    return x, mask, bias, ws[0], ws[1], ws[2], ws[3], (ws[4] if with_out else None), qb
+
+
+def torch_fused(x, mask, bias, wq, wk, wv, wg, wo, qb, head):
+    """The op spelled with torch library routines in float64 (weights are weight^T: y = x @ w)."""
+    t = lambda a: torch.from_numpy(np.asarray(a)).double()
+    x_, B, L, C = t(x), *x.shape
+    split = lambda y: y.reshape(B, L, head, C // head).permute(0, 2, 1, 3)
+    q = x_ @ t(wq)
+    if qb is not None:
+        q = q + t(qb)
+    add = t(bias)[None] + torch.where(torch.from_numpy(mask), 0.0, -1e9).double()[:, None, None, :]
+    o = torch.nn.functional.scaled_dot_product_attention(split(q), split(x_ @ t(wk)), split(x_ @ t(wv)), attn_mask=add)
+    o = o.permute(0, 2, 1, 3).reshape(B, L, C) * torch.sigmoid(x_ @ t(wg))
+    return (o @ t(wo) if wo is not None else o).numpy()
+
+
+@pytest.mark.parametrize("B,L,C,head,with_out,with_qbias", [(2, 40, 32, 4, True, False), (1, 33, 48, 3, False, True), (3, 17, 16, 2, True, True)])
+def test_fused_formula_matches_torch_library_ops(oracle, B, L, C, head, with_out, with_qbias):
+    case = fused_case(np.random.default_rng(B * 100 + L), B, L, C, head, with_out, with_qbias)
+    got = oracle.fused_attention_formula(*case, head=head)
+    want = torch_fused(*case, head)
+    assert np.abs(got - want).max() <= 2e-6 * max(1.0, np.abs(want).max())
+
+
+def test_fused_formula_without_batch_axis_is_the_b1_case(oracle):
+    x, mask, bias, wq, wk, wv, wg, _, qb = fused_case(np.random.default_rng(5), 1, 24, 32, 4, False, True)
+    a = oracle.fused_attention_formula(x[0], mask[0], bias, wq, wk, wv, wg, None, qb, head=4)
+    b = oracle.fused_attention_formula(x, mask, bias, wq, wk, wv, wg, None, qb, head=4)
+    assert a.shape == (24, 32) and np.array_equal(a, b[0])
+
+
+def test_fused_formula_special_cases(oracle):
+    """Zero gate weights halve the ungated result (sigmoid(0) = 1/2); an identity output projection is a no-op;
+    with a zero q projection the q bias alone drives the logits; heads do not mix before the output projection."""
+    rng = np.random.default_rng(6)
+    B, L, C, head = 2, 20, 32, 4
+    K = C // head
+    x, mask, bias, wq, wk, wv, wg, wo, _ = fused_case(rng, B, L, C, head)
+    eye, zero = np.eye(C, dtype=np.float32), np.zeros((C, C), np.float32)
+    base = oracle.fused_attention_formula(x, mask, bias, wq, wk, wv, zero, None, None, head=head)
+    # ungated attention from the core formula, heads split by hand
+    split = lambda y: y.reshape(B, L, head, K).transpose(0, 2, 1, 3)
+    core = oracle.dpa_formula(split(x @ wq), split(x @ wk), split(x @ wv), mask, bias).transpose(0, 2, 1, 3).reshape(B, L, C)
+    assert np.abs(base - 0.5 * core).max() <= 2e-5
+    assert np.abs(oracle.fused_attention_formula(x, mask, bias, wq, wk, wv, zero, eye, None, head=head) - base).max() <= 1e-6
+    assert np.abs(oracle.fused_attention_formula(x, mask, bias, wq, wk, wv, zero, wo, None, head=head) - base @ wo).max() <= 2e-5
+    # q = q_bias for every row: logits = q_bias . k_j / sqrt(K) + bias
+    qb = rng.standard_normal(C).astype(np.float32)
+    got = oracle.fused_attention_formula(x, mask, bias, zero, wk, wv, zero, None, qb, head=head)
+    qconst = np.broadcast_to(qb, (B, L, C)).copy()
+    want = 0.5 * oracle.dpa_formula(split(qconst), split(x @ wk), split(x @ wv), mask, bias).transpose(0, 2, 1, 3).reshape(B, L, C)
+    assert np.abs(got - want).max() <= 2e-5
+    # changing head 1's value columns changes only head 1's output columns
+    wv2 = wv.copy()
+    wv2[:, K:2 * K] *= 2.0
+    a = oracle.fused_attention_formula(x, mask, bias, wq, wk, wv, wg, None, None, head=head)
+    b = oracle.fused_attention_formula(x, mask, bias, wq, wk, wv2, wg, None, None, head=head)
+    assert np.abs(b[..., K:2 * K] - 2.0 * a[..., K:2 * K]).max() <= 2e-5
+    assert np.array_equal(np.delete(a, np.s_[K:2 * K], axis=-1), np.delete(b, np.s_[K:2 * K], axis=-1))
+
+
+@pytest.mark.parametrize("L,BLK", [(64, 64), (100, 64), (200, 128), (37, 128)])
+def test_fused_reference_restatement_fp32_equals_formula(oracle, L, BLK):
+    """The tiled loop nest with padding to a multiple of BLK_SZ computes the same function as the formula."""
+    for with_out, with_qbias, B in ((True, False, 2), (False, True, 1)):
+        case = fused_case(np.random.default_rng(L + BLK), B, L, 32, 4, with_out, with_qbias)
+        got = oracle.fused_attention_reference(*case, head=4, dtype=oracle.F32, BLK_SZ=BLK)
+        want = oracle.fused_attention_formula(*case, head=4)
+        assert np.abs(got - want).max() <= 2e-5
+
+
+def test_fused_reference_restatement_bf16_within_tolerance(oracle):
+    """With every intermediate rounded to bf16 as the reference does, the result stays within the bf16 budget of the
+    exact formula on bf16-representable inputs (the reference's own harness accepts mean relative error 5e-2)."""
+    case = list(fused_case(np.random.default_rng(77), 2, 96, 64, 4))
+    for i in (0, 2, 3, 4, 5, 6, 7):
+        case[i] = oracle.round_bf16(case[i])
+    got = oracle.fused_attention_reference(*case, head=4, dtype=oracle.BF16, BLK_SZ=64)
+    want = oracle.fused_attention_formula(*case, head=4)
+    assert np.abs(got - want).max() <= 3e-2 * max(1.0, np.abs(want).max())
+    assert np.abs(got - want).sum() / np.abs(want).sum() <= 2e-2

@@ -6,15 +6,16 @@
 and the module that wraps the first one, GridSelfAttentionCpp (src/af3_kernels/Attention.py:23-82).
 
 On the GPU the op is three launches instead of the reference's per-(row, head) loop nest:
-  1. ONE library GEMM for the four projections (q | k | v | gate): x [rows, C] . W [C, 4C]
-     (hipBLASLt through torch.matmul: a plain GEMM is library territory);
+  1. ONE library GEMM for the four projections: x [rows, C] . W [C, 4C], output columns ordered
+     (head, [k, v, q, gate], channel)  (hipBLASLt through torch: a plain GEMM is library territory);
   2. the attention kernel, reading q, k, v as strided views of that GEMM's output (no
      "b n (h d) -> b h n d" copies), adding bias and mask, and applying sigmoid(gate) in its
      epilogue while writing straight into the "b n (h d)" layout;
   3. the output projection GEMM (grid attention only).
 Weights arrive in the layout the reference's callers produce with vnni_repack_tensor(W.T, 2, C/head)
-and are unpacked once per weight set into the fused [C, 4C] matrix (cached).
+and are unpacked once per weight set into the fused matrix (cached per live weight tensor and version).
 """
+import weakref
 from typing import Optional
 
 import torch
@@ -36,16 +37,45 @@ def _unpack_panels(w: torch.Tensor, head: int) -> torch.Tensor:
     return w.reshape(head, C, K).permute(1, 0, 2).reshape(C, C)
 
 
-def _fused_weight(ws, head: int, dtype: torch.dtype) -> torch.Tensor:
-    """[C, 4C] = (q | k | v | gate) projection matrices side by side, unpacked from the panel layout."""
-    key = tuple((w.data_ptr(), w._version, tuple(w.shape), w.dtype) for w in ws) + (head, dtype)
+def _cached(sources, extra, make):
+    """make()'s result, remembered for as long as the source tensors are the same live objects at the same
+    version (an in-place update bumps the version; a freed tensor's address or id may be reused by another
+    tensor, which the weak references tell apart)."""
+    key = tuple(id(t) for t in sources) + extra
     hit = _W_CACHE.get(key)
-    if hit is None:
-        if len(_W_CACHE) >= _W_CACHE_MAX:
-            _W_CACHE.clear()
-        hit = torch.cat([_unpack_panels(w, head).to(dtype) for w in ws], dim=1).contiguous()
-        _W_CACHE[key] = hit
-    return hit
+    if hit is not None:
+        refs, versions, value = hit
+        if all(r() is t for r, t in zip(refs, sources)) and versions == tuple(t._version for t in sources):
+            return value
+    if len(_W_CACHE) >= _W_CACHE_MAX:
+        _W_CACHE.clear()
+    value = make()
+    _W_CACHE[key] = (tuple(weakref.ref(t) for t in sources), tuple(t._version for t in sources), value)
+    return value
+
+
+def _fused_weight(ws, head: int, dtype: torch.dtype) -> torch.Tensor:
+    """The four projection matrices (q, k, v, gate: weight^T in panel layout) as ONE [4C, C] matrix for a single
+    GEMM, rows (= output columns) ordered (head, [k, v, q, gate], channel): the 4K values of one token and
+    head are contiguous, K and V side by side, so that every 128-byte line the attention kernel fetches
+    for a key is used whole by the workgroups of that head."""
+    def make():
+        C = ws[0].shape[0]
+        K = C // head
+        q, k, v, g = (_unpack_panels(w, head).to(dtype).view(C, head, K) for w in ws)
+        return torch.stack((k, v, q, g), dim=2).reshape(C, 4 * C).t().contiguous()
+    return _cached(tuple(ws), (head, dtype), make)
+
+
+def _q_bias_row(q_bias: torch.Tensor, head: int, dtype: torch.dtype) -> torch.Tensor:
+    """[4C] row added by the projection GEMM's epilogue: q_bias in the q columns, zero elsewhere."""
+    def make():
+        C = q_bias.numel()
+        K = C // head
+        row = torch.zeros(head, 4, K, dtype=dtype, device=q_bias.device)
+        row[:, 2] = q_bias.reshape(head, K).to(dtype)
+        return row.view(4 * C)
+    return _cached((q_bias,), (head, dtype, "q_bias"), make)
 
 
 def _check_weights(C: int, head: int, ws):
@@ -56,6 +86,26 @@ def _check_weights(C: int, head: int, ws):
             raise ValueError(f"projection weights must be [{C}, {C}], got {tuple(w.shape)}")
         if not w.is_contiguous():
             raise ValueError("projection weights must be contiguous (they carry a packed layout)")
+
+
+def _project(rows: torch.Tensor, ws, q_bias: Optional[torch.Tensor], head: int) -> torch.Tensor:
+    """Stage 1: [rows, C] . [C, 4C] -> per token and head (k | v | q | gate).  The q bias of the diffusion op
+    rides the GEMM's epilogue."""
+    W = _fused_weight(ws, head, rows.dtype)
+    return torch.nn.functional.linear(rows, W, None if q_bias is None else _q_bias_row(q_bias, head, rows.dtype))
+
+
+def _attend(y: torch.Tensor, B: int, N: int, head: int, mask, bias) -> torch.Tensor:
+    """Stage 2: the attention kernel on strided [B, head, N, K] views of stage 1's output (no "b n (h d) -> b h n d"
+    copies); sigmoid(gate) is applied in its epilogue and the result lands in "b n (h d)" order.  Returns [B, N, C]."""
+    C = y.shape[1] // 4
+    K = C // head
+    k, v, q, g = (y.view(B, N, head, 4, K)[:, :, :, i].permute(0, 2, 1, 3) for i in range(4))
+    out = torch.empty(B, N, C, dtype=y.dtype, device=y.device)
+    keep = ops._lift_mask(mask, N) if mask is not None else None
+    ops._dpa_forward_impl(q, k, v, keep, bias.to(y.dtype) if bias is not None else None, ops._DTYPE_CODE[y.dtype], False, gate=g,
+                          out=out.view(B, N, head, K).permute(0, 2, 1, 3))
+    return out
 
 
 def _attention_cpp(
@@ -86,14 +136,8 @@ def _attention_cpp(
     code = ops._DTYPE_CODE.get(dtype)
     if code not in (ops.AF3_F32, ops.AF3_BF16):
         raise ValueError(f"unsupported dtype {dtype}: float32 or bfloat16")
-    K = C // head
-    W = _fused_weight((q_proj, k_proj, v_proj, gating_query), head, dtype)
-    y = torch.matmul(pair.reshape(B * N, C), W).view(B, N, 4, head, K)     # q | k | v | gate, each "(h d)"
-    q, k, v, g = (y[:, :, i].permute(0, 2, 1, 3) for i in range(4))        # [B, head, N, K] views, no copies
-    gated = torch.empty(B, N, C, dtype=dtype, device=pair.device)
-    keep = ops._lift_mask(mask, N) if mask is not None else None
-    ops._dpa_forward_impl(q, k, v, keep, bias.to(dtype) if bias is not None else None, code, False, gate=g,
-                          out=gated.view(B, N, head, K).permute(0, 2, 1, 3))
+    y = _project(pair.reshape(B * N, C), (q_proj, k_proj, v_proj, gating_query), None, head)
+    gated = _attend(y, B, N, head, mask, bias)
     return torch.matmul(gated.view(B * N, C), out_proj.to(dtype)).view(B, N, C)
 
 
@@ -124,22 +168,8 @@ def self_attention_cpp(
     code = ops._DTYPE_CODE.get(dtype)
     if code not in (ops.AF3_F32, ops.AF3_BF16):
         raise ValueError(f"unsupported dtype {dtype}: float32 or bfloat16")
-    K = C // head
-    W = _fused_weight((q_proj, k_proj, v_proj, gating_query), head, dtype)
-    if q_bias is not None:
-        # the q bias rides the GEMM's epilogue: [q_bias | 0 | 0 | 0] added to every output row
-        row = torch.zeros(4 * C, dtype=dtype, device=pair.device)
-        row[:C] = q_bias.reshape(C).to(dtype)
-        y = torch.addmm(row, pair, W)
-    else:
-        y = torch.matmul(pair, W)
-    y = y.view(1, N, 4, head, K)
-    q, k, v, g = (y[:, :, i].permute(0, 2, 1, 3) for i in range(4))
-    out = torch.empty(N, C, dtype=dtype, device=pair.device)
-    keep = ops._lift_mask(mask, N) if mask is not None else None
-    ops._dpa_forward_impl(q, k, v, keep, bias.to(dtype) if bias is not None else None, code, False, gate=g,
-                          out=out.view(1, N, head, K).permute(0, 2, 1, 3))
-    return out
+    y = _project(pair, (q_proj, k_proj, v_proj, gating_query), q_bias, head)
+    return _attend(y, 1, N, head, mask, bias).view(N, C)
 
 
 class GridSelfAttentionCpp(torch.nn.Module):

@@ -9,7 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libaf3_dpa.so")
 
 AF3_F32, AF3_BF16, AF3_FP8_E4M3 = 0, 1, 2
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 i64, i32, f32, vp = ctypes.c_int64, ctypes.c_int32, ctypes.c_float, ctypes.c_void_p
 
@@ -31,6 +31,19 @@ class DpaParams(ctypes.Structure):
     ]
 
 
+class GridAttentionParams(ctypes.Structure):
+    """Mirror of struct af3_grid_attention_params."""
+    _fields_ = [
+        ("pair", vp), ("pair_stride", i64 * 2),
+        ("q_proj", vp), ("k_proj", vp), ("v_proj", vp), ("gating_query", vp),
+        ("bias", vp), ("bias_stride", i64 * 2), ("bias_dtype", i32), ("dtype", i32),
+        ("key_mask", vp), ("key_mask_stride_b", i64),
+        ("out", vp), ("out_stride", i64 * 2),
+        ("B", i64), ("N", i64), ("C", i64), ("head", i64),
+        ("workspace", vp), ("workspace_bytes", i64),
+    ]
+
+
 QKV_SCRATCH_FLOATS = 768   # AF3_QKV_SCRATCH_FLOATS
 
 # name -> (restype, argtypes); every symbol include/af3_dpa.h declares
@@ -38,6 +51,9 @@ SYMBOLS = {
     "af3_dpa_forward": (ctypes.c_int, [ctypes.POINTER(DpaParams), vp]),
     "af3_dpa_select_kernel": (ctypes.c_int, [ctypes.POINTER(DpaParams)]),
     "af3_dpa_workspace_bytes": (ctypes.c_int64, [ctypes.POINTER(DpaParams)]),
+    "af3_grid_attention_forward": (ctypes.c_int, [ctypes.POINTER(GridAttentionParams), vp]),
+    "af3_grid_attention_workspace_bytes": (ctypes.c_int64, [ctypes.POINTER(GridAttentionParams)]),
+    "af3_grid_attention_supported": (ctypes.c_int, [ctypes.POINTER(GridAttentionParams)]),
     "af3_convert": (ctypes.c_int, [vp, i32, vp, i32, i64, vp]),
     "af3_amax": (ctypes.c_int, [vp, i32, i64, vp, vp]),
     "af3_quantize_fp8_e4m3": (ctypes.c_int, [vp, i32, vp, i64, i64, i64, i32, i64, i64, f32, vp, vp, vp, vp]),

@@ -83,6 +83,29 @@ extern "C" int af3_dpa_forward(const af3_dpa_params* params, void* hip_stream) {
 	}
 }
 
+static int validate_grid(const af3_grid_attention_params* g) {
+	if(!g || !g->pair || !g->out || !g->q_proj || !g->k_proj || !g->v_proj || !g->gating_query) return AF3_ERR_NULL_POINTER;
+	if(g->B <= 0 || g->N <= 0 || g->C <= 0 || g->head <= 0 || g->C % g->head != 0 || g->B > 0x3fffffff) return AF3_ERR_BAD_SHAPE;
+	if(g->pair_stride[0] < 0 || g->pair_stride[1] < g->C || g->out_stride[0] < 0 || g->out_stride[1] < g->C) return AF3_ERR_BAD_STRIDE;
+	if(g->bias && (g->bias_stride[0] < 0 || g->bias_stride[1] < g->N)) return AF3_ERR_BAD_STRIDE;
+	if(g->key_mask && g->key_mask_stride_b != 0 && g->key_mask_stride_b < g->N) return AF3_ERR_BAD_STRIDE;
+	return AF3_OK;
+}
+
+extern "C" int af3_grid_attention_supported(const af3_grid_attention_params* g) { return validate_grid(g) == AF3_OK && grid_fused_eligible(*g) ? 1 : 0; }
+
+extern "C" int64_t af3_grid_attention_workspace_bytes(const af3_grid_attention_params* g) {
+	const int rc = validate_grid(g);
+	return rc != AF3_OK ? rc : grid_fused_workspace_bytes(*g);
+}
+
+extern "C" int af3_grid_attention_forward(const af3_grid_attention_params* g, void* hip_stream) {
+	const int rc = validate_grid(g);
+	if(rc != AF3_OK) return rc;
+	if(!grid_fused_eligible(*g)) return AF3_ERR_BAD_ARGUMENT;
+	return launch_grid_fused(*g, static_cast<hipStream_t>(hip_stream));
+}
+
 extern "C" const char* af3_status_string(int status) {
 	switch(status) {
 		case AF3_OK: return "ok";
@@ -98,4 +121,4 @@ extern "C" const char* af3_status_string(int status) {
 	}
 }
 
-extern "C" int af3_abi_version(void) { return 2; }
+extern "C" int af3_abi_version(void) { return 3; }

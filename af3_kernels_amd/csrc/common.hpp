@@ -43,6 +43,14 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 // sigmoid for the optional output gate (reference: tpp::SigmoidFwdTPP, src/csrc/xsmm_functors.h:2694-2731)
 __device__ __forceinline__ float sigmoidf_fast(float x) { return 1.f / (1.f + __builtin_amdgcn_exp2f(-x * LOG2E)); }
 
+// Extra kernel arguments of the fused grid-attention variant of the bf16 kernel: the input rows and the four
+// per-head projection matrices (weight^T in the reference's panel layout [head][C/2][32][2]).
+struct fused_grid_args {
+	const uint16_t* x;
+	int64_t         x_stride_b, x_stride_n;  // elements
+	const void *    wq, *wk, *wv, *wg;
+};
+
 // Launchers implemented in the .hip files; all validated by api.hip before the call.
 int launch_dpa_generic(const af3_dpa_params& p, hipStream_t s);
 int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s);
@@ -52,5 +60,8 @@ int64_t mfma_bf16_workspace_bytes(const af3_dpa_params& p);
 bool mfma_fp8_eligible(const af3_dpa_params& p);
 int launch_dpa_mfma_f32(const af3_dpa_params& p, hipStream_t s);
 bool mfma_f32_eligible(const af3_dpa_params& p);
+bool grid_fused_eligible(const af3_grid_attention_params& g);
+int64_t grid_fused_workspace_bytes(const af3_grid_attention_params& g);
+int launch_grid_fused(const af3_grid_attention_params& g, hipStream_t s);
 
 }  // namespace af3

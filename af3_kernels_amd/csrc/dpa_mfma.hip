@@ -159,11 +159,16 @@ __device__ __forceinline__ uint32_t lds_addr_of(const void* ptr) {
 // variant only).  SPLIT: for launches too small to fill the chip -- the NW wavefronts of a workgroup
 // share ONE block of 32 query rows and split its key tiles round robin (each with private LDS
 // buffers, no barrier in the loop); their partial (O, m, l) are merged through LDS at the end.
-template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT>
+// FUSED: the grid-attention variant.  One workgroup = one (batch, head); q, k, v and the gate are not
+// read from memory but projected in the kernel from the input rows x[b] (C channels) with the four
+// weight matrices of this head, K and V of ALL keys stay in LDS for the whole workgroup, and each
+// wavefront then walks query blocks qb = wave, wave + NW, ... on its own (no barrier after the
+// projection of K and V).  Requires DP = 32, the log2 variant, no key split.
+template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT, bool FUSED>
 // (at least 2 wavefronts per SIMD: keeps the register budget at 256 so that the compiler writes MFMA
 // results to ordinary VGPRs instead of AGPRs, which every softmax operand would have to be copied out of;
 // the key-split variants are limited to fewer than 2 wavefronts per SIMD by their LDS buffers anyway)
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP == 32 && !SPLIT ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups) {
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FUSED ? (NW + 3) / 4 : DP == 32 && !SPLIT ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups, fused_grid_args fa) {
 	constexpr int NC         = DP / 16;            // contraction chunks of QK^T
 	constexpr int NDB        = DP / 32;            // 32-row blocks of O^T
 	constexpr int CPR        = DP / 8;             // 16-byte chunks per K/V row
@@ -177,15 +182,20 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	constexpr int  RING_BYTES = BRING ? NW * 3 * 4096 : 0;
 	constexpr int  MASK_BASE  = LDS_SETS * 6 * TILE_BYTES + RING_BYTES;
 	static_assert(!(L2DOM && BMODE != 0), "the log2 variant reads its bias from the workspace");
-	static_assert(NW <= NI, "every wavefront fetches a whole number of 1 KB pieces of each tile");
+	static_assert(FUSED || NW <= NI, "every wavefront fetches a whole number of 1 KB pieces of each tile");
+	static_assert(!FUSED || (DP == 32 && L2DOM && !SPLIT && NW % 2 == 0), "the fused variant exists for 32-channel heads in the log2 variant");
 
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 	// [K x3][V x3][bias ring: 3 x 4 KB per wavefront (BRING)][mask table: (n_ktiles*64 + 64) dwords][live list]
 	const int            tid_pre   = threadIdx.x;
-	unsigned char* const k_lds     = smem + (SPLIT ? __builtin_amdgcn_readfirstlane(tid_pre >> 6) * 6 * TILE_BYTES : 0);
-	unsigned char* const v_lds     = k_lds + 3 * TILE_BYTES;
-	uint32_t* const      mask_tab  = reinterpret_cast<uint32_t*>(smem + MASK_BASE);
+	// FUSED: [K of all tiles][V of all tiles][Wq fragments][Wgate fragments][mask table][live list]
 	const int            n_ktiles  = (int)((p.L + KT - 1) / KT);
+	constexpr int        NS        = 8;  // FUSED: contraction steps of a projection (C = 128 input channels, 16 per MFMA)
+	unsigned char* const k_lds     = smem + (SPLIT ? __builtin_amdgcn_readfirstlane(tid_pre >> 6) * 6 * TILE_BYTES : 0);
+	unsigned char* const v_lds     = k_lds + (FUSED ? n_ktiles : 3) * TILE_BYTES;
+	unsigned char* const w_lds     = v_lds + n_ktiles * TILE_BYTES;  // FUSED only
+	const int            mask_base = FUSED ? 2 * n_ktiles * TILE_BYTES + 2 * NS * 1024 : MASK_BASE;
+	uint32_t* const      mask_tab  = reinterpret_cast<uint32_t*>(smem + mask_base);
 	int16_t* const       live_list = reinterpret_cast<int16_t*>(mask_tab + n_ktiles * KT + 64);
 	__shared__ int       s_nvalid, s_nlive;
 
@@ -209,7 +219,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 
 	// ---- zero the K/V buffers: lanes of padded head columns never write them, and whatever a
 	// bounds-checked load leaves behind for rows past L must be finite (0 * stale NaN = NaN) ----
-	if(D != DP || L % KT != 0)
+	if(!FUSED && (D != DP || L % KT != 0))
 		for(int i = tid; i < (LDS_SETS * 6 * TILE_BYTES + RING_BYTES) / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
 	// ---- key-mask table and list of tiles with at least one live key ----
 	// entry = bf16 additive mask value in the low half (contraction slot 0) and, in the log2
@@ -255,515 +265,634 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DP
 	// the mask constant and the weights come out uniform whatever the accumulation order.
 	const bool all_dropped = __builtin_amdgcn_readfirstlane(s_nvalid) == 0;
 
-	// ---- per-lane constants ----
-	const int64_t qrow   = (int64_t)qtile * QT + (SPLIT ? 0 : wave * 32) + n;
-	const bool    row_ok = qrow < L;
-
-	// Q fragments (B operand of S^T = K.Q^T): lane (q = n, g = half) holds q[q][16c + 8g .. +7]
-	// scaled and rounded to bf16 (the reference also rounds the scaled q,
-	// src/csrc/dot_product_attention.cpp:95-98).
+	// ---- FUSED: projections.  out^T[d][token] = sum_c W[c][d] * x[token][c], 32 tokens per matrix instruction chain:
+	//   A operand (weights)    lane (d = lane%32, g = lane/32), step s: W[16s + 8g + 0..7][d]; in the panel layout
+	//                          [C/2][32][2] of one head these are four dwords, 32 dwords apart;
+	//   B operand (rows of x)  lane (token = lane%32, g), step s: x[token][16s + 8g + 0..7], one 16-byte load
+	//                          (range-checked: rows past L read as zero);
+	//   result                 lane = token, register i = output channel 8*(i/4) + 4*g + i%4.
+	[[maybe_unused]] __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(static_cast<uint16_t*>(nullptr), 0, 0, 0x00020000);
+	[[maybe_unused]] int x_row_bytes = 0;
+	auto load_x_frags = [&](int token, u32x4 (&xf)[NS]) {
+#pragma unroll
+		for(int st = 0; st < NS; st++)
+			xf[st] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, token * x_row_bytes + (16 * st + 8 * half) * 2, 0, 0));
+	};
+	// q fragments (B operand of S^T = K.Q^T) and, FUSED, the gate pre-activations of this lane's 16 output channels as
+	// bf16 pairs: per query block; the fused variant prepares them one block ahead
 	const float qmul = all_dropped ? 0.f : (L2DOM ? p.softmax_scale * LOG2E : p.softmax_scale);
 	bf16x8      qf[NC];
-	{
-		const uint16_t* qp = static_cast<const uint16_t*>(p.q) + b * p.q_stride[0] + h * p.q_stride[1] + qrow * p.q_stride[2];
+	[[maybe_unused]] u32x4 gate_pk[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
+	// q and gate rows of a block from its rows of x (src/csrc/dot_product_attention.cpp:301-312, :334-345); q is scaled
+	// in fp32 and rounded once, the gate is rounded to bf16 like the reference's tmp buffer
+	auto project_q_gate = [&](const u32x4 (&xf)[NS]) {
+		f32x16 aq, ag;
+#pragma unroll
+		for(int i = 0; i < 16; i++) aq[i] = 0.f, ag[i] = 0.f;
+#pragma unroll
+		for(int st = 0; st < NS; st++) {
+			const u32x4 wqf = reinterpret_cast<const u32x4*>(w_lds)[st * 64 + lane], wgf = reinterpret_cast<const u32x4*>(w_lds)[(NS + st) * 64 + lane];
+			aq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wqf), __builtin_bit_cast(bf16x8, xf[st]), aq, 0, 0, 0);
+			ag = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wgf), __builtin_bit_cast(bf16x8, xf[st]), ag, 0, 0, 0);
+		}
 #pragma unroll
 		for(int c = 0; c < NC; c++) {
-			const int d0  = 16 * c + 8 * half;
-			u32x4     raw = {0u, 0u, 0u, 0u};
-			if(row_ok && d0 < D) raw = *reinterpret_cast<const u32x4*>(qp + d0);
-			u32x4 sc;
+			u32x4 sc4;
 #pragma unroll
-			for(int j = 0; j < 4; j++) sc[j] = pack_bf16x2(bf16_bits_to_f32(raw[j] & 0xffffu) * qmul, bf16_bits_to_f32(raw[j] >> 16) * qmul);
-			qf[c] = __builtin_bit_cast(bf16x8, sc);
+			for(int j = 0; j < 4; j++) sc4[j] = pack_bf16x2(aq[8 * c + 2 * j] * qmul, aq[8 * c + 2 * j + 1] * qmul);
+			qf[c] = __builtin_bit_cast(bf16x8, sc4);
 		}
-	}
-	// Identity fragments (A operand of the bias MFMA): lane (m = n, g = half), slot j of chunk c2
-	// is 1.0 iff m == 16*c2 + 8*g + j.  bf16 1.0 for the natural variant, fp16 1.0 for the log2 one.
-	u32x4 idf[2];
 #pragma unroll
-	for(int c2 = 0; c2 < 2; c2++) {
-		u32x4     v = {0u, 0u, 0u, 0u};
-		const int j = n - 16 * c2 - 8 * half;
-		if(j >= 0 && j < 8) v[j >> 1] = (L2DOM ? 0x3C00u : 0x3F80u) << ((j & 1) * 16);
-		idf[c2] = v;
-	}
-	// B operand of the mask MFMA: slot 0 = 1.0 (multiplies the key's mask value); log2 variant: slots 1
-	// and 2 = the reference maximum as -(m_hi + m_lo), two bf16 terms (16 significant bits, so that a
-	// reference of large magnitude -- a row whose biases are all hugely negative -- is still subtracted
-	// to within a fraction of a unit), multiplying the 1.0 that every key carries in slots 1 and 2 of A.
-	u32x4 maskB = {0u, 0u, 0u, 0u};
-	if(half == 0) maskB[0] = 0x3F80u;
-	u32x4 maskA = {0u, 0u, 0u, 0u};
-	if(L2DOM && half == 0) maskA[1] = 0x3F80u;  // slot 2; slots 0 and 1 come from the mask table
-
-	const bool has_bias = p.bias != nullptr && !all_dropped;
-	// natural variant: direct bias access through per-lane row pointers
-	const unsigned char* bias_row = nullptr;
-	bool                 bias_vec = false;
-	if(!L2DOM && has_bias) {
-		const int64_t esz = BIAS_F32 ? 4 : 2;
-		bias_row = static_cast<const unsigned char*>(p.bias) + (h * p.bias_stride[0] + (row_ok ? qrow : 0) * p.bias_stride[1]) * esz;
-		bias_vec = !BIAS_F32 && ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) && (p.bias_stride[0] % 8 == 0) && (p.bias_stride[1] % 8 == 0);
-	}
-	// log2 variant: fragment-ordered workspace; the tile base is wave-uniform
-	const u32x4* ws_wave = nullptr;
-	if(L2DOM && has_bias) {
-		const int     n_qblocks = (int)((L + 31) / 32);
-		const int64_t qb        = SPLIT ? (int64_t)qtile : (int64_t)qtile * NW + wave;
-		// query blocks beyond the last one only hold rows >= L; clamp so that loads stay in bounds
-		const int64_t qbc = qb < n_qblocks ? qb : n_qblocks - 1;
-		ws_wave = static_cast<const u32x4*>(p.workspace) + ((h * n_qblocks + qbc) * n_ktiles) * 256;
-	}
-	// (scalar base + per-lane 16-byte offset + scalar tile offset: no 64-bit pointer in vector registers)
-	const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(ws_wave), 0, ws_wave ? n_ktiles * 4096 : 0, 0x00020000);
-	const int                    ws_voff = lane * 16;
-
-	// ---- K/V tile loader: buffer loads that write LDS directly ----
-	// One wave load moves 1 KB: lane i -> LDS chunk i of the load's 1 KB window, i.e. tile row
-	// j*RPI + i/CPR, physical chunk i%CPR.  The lane picks the global chunk that belongs there
-	// under the swizzle; lanes of padded head columns (chunk*8 >= D) stay idle.
-	const u32x4 k_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1], (uint32_t)(((L - 1) * p.k_stride[2] + D) * 2));
-	const u32x4 v_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.v) + b * p.v_stride[0] + h * p.v_stride[1], (uint32_t)(((L - 1) * p.v_stride[2] + D) * 2));
-	const int  ld_row  = lane / CPR, ld_pc = lane % CPR;
-	const int  k_chunk = ld_pc ^ k_swizzle<DP>(ld_row);
-	const int  v_chunk = ld_pc ^ v_swizzle<DP>(ld_row);
-	const int  k_voff  = (int)(ld_row * p.k_stride[2] * 2) + k_chunk * 16;
-	const int  v_voff  = (int)(ld_row * p.v_stride[2] * 2) + v_chunk * 16;
-	const bool k_act   = k_chunk * 8 < D, v_act = v_chunk * 8 < D;
-	const int  k_tile_stride = (int)(KT * p.k_stride[2] * 2), v_tile_stride = (int)(KT * p.v_stride[2] * 2);
-	const int  k_ld_stride   = (int)(RPI * p.k_stride[2] * 2), v_ld_stride = (int)(RPI * p.v_stride[2] * 2);
-	const uint32_t k_lds_addr = lds_addr_of(k_lds), v_lds_addr = lds_addr_of(v_lds);
-	auto load_tile = [&](int kt, int buf) {
-#pragma unroll
-		for(int t = 0; t < (SPLIT ? NI : NI / NW); t++) {
-			const int j = SPLIT ? t : wave + NW * t;  // split: this wavefront fetches whole tiles into its private buffers
-			if(k_act) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + j * 1024, k_voff + (kt * k_tile_stride + j * k_ld_stride));
-			if(v_act) lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + j * 1024, v_voff + (kt * v_tile_stride + j * v_ld_stride));
-		}
+		for(int j = 0; j < 8; j++) gate_pk[j >> 2][j & 3] = pack_bf16x2(ag[2 * j], ag[2 * j + 1]);
 	};
-
-	// ---- bias ring (BRING): the 32 x 64 bias tile of this wavefront's query block, 4 KB, travels
-	// HBM -> LDS by four LDS-direct loads of whole 128-byte row segments (eight lanes per row), two
-	// tiles ahead of its use and without occupying registers.  Slot layout: [row 32][128 B], the
-	// 16-byte chunk c of row r stored at chunk position c ^ (r & 7) so that the fragment reads (one
-	// chunk per lane, 32 rows at once) spread over the banks.  Rows past L lie beyond the buffer's
-	// range; chunks of keys past L (last tile) are sent there too, so padding behind a row's L valid
-	// entries is never read.  Whatever such lanes leave in LDS is finite: the ring starts zeroed.
-	const u32x4    b_rsrc    = raw_rsrc(BRING ? static_cast<const uint16_t*>(p.bias) + h * p.bias_stride[0] : nullptr,
-										BRING ? (uint32_t)(((L - 1) * p.bias_stride[1] + L) * 2) : 0u);
-	unsigned char* const bring = smem + LDS_SETS * 6 * TILE_BYTES + (BRING ? wave * 3 * 4096 : 0);
-	const uint32_t bring_addr = lds_addr_of(bring);
-	const int      b_voff     = (int)((lane >> 3) * p.bias_stride[1] * 2) + (((lane & 7) ^ (lane >> 3)) << 4);
-	const int      b_row0     = (int)((qtile * QT + (SPLIT ? 0 : wave * 32)) * p.bias_stride[1] * 2);
-	const int      b_row8     = (int)(8 * p.bias_stride[1] * 2);
-	const int      b_key      = ((lane & 7) ^ (lane >> 3)) * 8;  // first key of this lane's chunk within a tile
-	auto load_bias_tile = [&](int kt, int slot_i) {
-		if(!BRING) return;
-		const int in_row = kt * KT + b_key < (int)L ? b_voff + kt * (KT * 2) : 0x7FFF0000;
-#pragma unroll
-		for(int j = 0; j < 4; j++) lds_dma_b128(b_rsrc, bring_addr + slot_i * 4096 + j * 1024, in_row + (b_row0 + j * b_row8));
-	};
-	// fragment read: lane (n, half) takes chunk 4*sub + 2*c2 + half of row n
-	const int b_rd = n * 128 + (((n & 7) ^ half) << 4);
-
-	// Natural variant: four fragments in flight, each sub-tile's pair requested two stages before its
-	// use.  Log2 variant (BIAS_LATE): one pair only -- the registers are the scarce resource at four
-	// wavefronts per SIMD -- requested inside the previous stage, right after the matrix
-	// instructions that consume the pair before it.
-	constexpr bool BIAS_LATE = L2DOM;
-	u32x4 bfrag[4];
-	auto  load_bias_frags = [&](int kt, auto sub_c) {
-		constexpr int SUB = decltype(sub_c)::value;
-		if(!has_bias || BRING) return;
-		if(L2DOM) {
-#pragma unroll
-			for(int c2 = 0; c2 < 2; c2++)
-				bfrag[c2] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, ws_voff + (2 * SUB + c2) * 1024, kt * 4096, 0));
-			return;
+	const int n_qblocks_all = (int)((L + 31) / 32);
+	int       qb_f          = 0;  // FUSED: the query block this wavefront works on
+	if constexpr(FUSED) {
+		x_rsrc      = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(fa.x + b * fa.x_stride_b), 0, (int)(((L - 1) * fa.x_stride_n + 16 * NS) * 2), 0x00020000);
+		x_row_bytes = (int)(fa.x_stride_n * 2);
+		const int64_t head_dwords = h * (16 * NS * 32 / 2);
+		// Wq and Wgate fragments -> LDS, [matrix][step][lane] x 16 bytes.  The rows of Wq are permuted so that the
+		// registers of the q projection's result ARE the B operand of K.Q^T: register i of half-wave g must hold
+		// channel 16*(i/8) + 8*g + i%8, and it holds result row 8*(i/4) + 4*g + i%4.
+		for(int i = tid; i < 2 * NS * 64; i += NW * 64) {
+			const int ln = i & 63, st = (i >> 6) % NS, m = i / (64 * NS);
+			const int r = ln & 31, g = ln >> 5, a = r >> 3;
+			const int d = m == 0 ? 16 * (a >> 1) + 8 * ((r >> 2) & 1) + 4 * (a & 1) + (r & 3) : r;
+			const uint32_t* w32 = reinterpret_cast<const uint32_t*>(m == 0 ? fa.wq : fa.wg) + head_dwords + (8 * st + 4 * g) * 32 + d;
+			reinterpret_cast<u32x4*>(w_lds)[i] = u32x4{w32[0], w32[32], w32[64], w32[96]};
 		}
-		const int64_t key0 = (int64_t)kt * KT + 8 * half;
-		if(bias_vec && (int64_t)(kt + 1) * KT <= L) {  // wave-uniform: whole tile in range, aligned rows
-			const uint16_t* bp = reinterpret_cast<const uint16_t*>(bias_row) + key0;
-			if(row_ok) {
+		__syncthreads();  // the fragments are read below
+		// K and V of every key, 32 keys at a time (wavefront w takes blocks w, w + NW, ...), rounded to bf16 like the
+		// reference's tmp_k / tmp_v (src/csrc/dot_product_attention.cpp:286-299) and stored where the tile loader of
+		// the unfused kernel would have put them (K rows chunk-swizzled, V rows plain).  One load of the 32 rows
+		// of x serves both products.
+		const uint32_t* wk32 = reinterpret_cast<const uint32_t*>(fa.wk) + head_dwords + (4 * half) * 32 + n;
+		const uint32_t* wv32 = reinterpret_cast<const uint32_t*>(fa.wv) + head_dwords + (4 * half) * 32 + n;
+		u32x4           wkf[NS], wvf[NS];
 #pragma unroll
-				for(int f = 2 * SUB; f < 2 * SUB + 2; f++) bfrag[f] = *reinterpret_cast<const u32x4*>(bp + 16 * f);
+		for(int st = 0; st < NS; st++) {
+			wkf[st] = u32x4{wk32[(8 * st) * 32], wk32[(8 * st + 1) * 32], wk32[(8 * st + 2) * 32], wk32[(8 * st + 3) * 32]};
+			wvf[st] = u32x4{wv32[(8 * st) * 32], wv32[(8 * st + 1) * 32], wv32[(8 * st + 2) * 32], wv32[(8 * st + 3) * 32]};
+		}
+		u32x4 xf[NS];
+		int   sb_last = -1;
+		for(int sb = wave; sb < 2 * n_ktiles; sb += NW) {
+			const int key = sb * 32 + n;
+			load_x_frags(key, xf);
+			f32x16 ak, av;
+#pragma unroll
+			for(int i = 0; i < 16; i++) ak[i] = 0.f, av[i] = 0.f;
+#pragma unroll
+			for(int st = 0; st < NS; st++) {
+				ak = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wkf[st]), __builtin_bit_cast(bf16x8, xf[st]), ak, 0, 0, 0);
+				av = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wvf[st]), __builtin_bit_cast(bf16x8, xf[st]), av, 0, 0, 0);
+			}
+			unsigned char* const kdst = k_lds + key * (DP * 2) + half * 8;
+			unsigned char* const vdst = v_lds + key * (DP * 2) + half * 8;
+			const int            swz  = k_swizzle<DP>(n);
+#pragma unroll
+			for(int j = 0; j < 4; j++) {
+				*reinterpret_cast<u32x2*>(kdst + ((j ^ swz) << 4)) = u32x2{pack_bf16x2(ak[4 * j], ak[4 * j + 1]), pack_bf16x2(ak[4 * j + 2], ak[4 * j + 3])};
+				*reinterpret_cast<u32x2*>(vdst + (j << 4))         = u32x2{pack_bf16x2(av[4 * j], av[4 * j + 1]), pack_bf16x2(av[4 * j + 2], av[4 * j + 3])};
+			}
+			sb_last = sb;
+		}
+		// This wavefront's query blocks are walked from the last one down: its rows of x are the ones just used
+		// (unless the last key block was padding past L), so q and the gate of that block come for free.
+		qb_f = n_qblocks_all - 1 - (n_qblocks_all - 1 - wave + NW * 64) % NW;  // largest block index congruent to wave (negative: none)
+		if(qb_f >= 0) {
+			if(sb_last != qb_f) load_x_frags(qb_f * 32 + n, xf);
+			project_q_gate(xf);
+		}
+		__syncthreads();  // K and V of every key are in LDS
+	}
+
+	// ---- one pass per block of 32 query rows: exactly one pass unless FUSED ----
+	for(; qb_f >= 0; qb_f -= FUSED ? NW : 1) {
+		// ---- per-lane constants ----
+		const int64_t qrow   = FUSED ? (int64_t)qb_f * 32 + n : (int64_t)qtile * QT + (SPLIT ? 0 : wave * 32) + n;
+		const bool    row_ok = qrow < L;
+
+		// Q fragments (B operand of S^T = K.Q^T): lane (q = n, g = half) holds q[q][16c + 8g .. +7]
+		// scaled and rounded to bf16 (the reference also rounds the scaled q,
+		// src/csrc/dot_product_attention.cpp:95-98).
+		if constexpr(!FUSED) {
+			const uint16_t* qp = static_cast<const uint16_t*>(p.q) + b * p.q_stride[0] + h * p.q_stride[1] + qrow * p.q_stride[2];
+#pragma unroll
+			for(int c = 0; c < NC; c++) {
+				const int d0  = 16 * c + 8 * half;
+				u32x4     raw = {0u, 0u, 0u, 0u};
+				if(row_ok && d0 < D) raw = *reinterpret_cast<const u32x4*>(qp + d0);
+				u32x4 sc;
+#pragma unroll
+				for(int j = 0; j < 4; j++) sc[j] = pack_bf16x2(bf16_bits_to_f32(raw[j] & 0xffffu) * qmul, bf16_bits_to_f32(raw[j] >> 16) * qmul);
+				qf[c] = __builtin_bit_cast(bf16x8, sc);
+			}
+		}
+		// Identity fragments (A operand of the bias MFMA): lane (m = n, g = half), slot j of chunk c2
+		// is 1.0 iff m == 16*c2 + 8*g + j.  bf16 1.0 for the natural variant, fp16 1.0 for the log2 one.
+		u32x4 idf[2];
+#pragma unroll
+		for(int c2 = 0; c2 < 2; c2++) {
+			u32x4     v = {0u, 0u, 0u, 0u};
+			const int j = n - 16 * c2 - 8 * half;
+			if(j >= 0 && j < 8) v[j >> 1] = (L2DOM ? 0x3C00u : 0x3F80u) << ((j & 1) * 16);
+			idf[c2] = v;
+		}
+		// B operand of the mask MFMA: slot 0 = 1.0 (multiplies the key's mask value); log2 variant: slots 1
+		// and 2 = the reference maximum as -(m_hi + m_lo), two bf16 terms (16 significant bits, so that a
+		// reference of large magnitude -- a row whose biases are all hugely negative -- is still subtracted
+		// to within a fraction of a unit), multiplying the 1.0 that every key carries in slots 1 and 2 of A.
+		u32x4 maskB = {0u, 0u, 0u, 0u};
+		if(half == 0) maskB[0] = 0x3F80u;
+		u32x4 maskA = {0u, 0u, 0u, 0u};
+		if(L2DOM && half == 0) maskA[1] = 0x3F80u;  // slot 2; slots 0 and 1 come from the mask table
+
+		const bool has_bias = p.bias != nullptr && !all_dropped;
+		// natural variant: direct bias access through per-lane row pointers
+		const unsigned char* bias_row = nullptr;
+		bool                 bias_vec = false;
+		if(!L2DOM && has_bias) {
+			const int64_t esz = BIAS_F32 ? 4 : 2;
+			bias_row = static_cast<const unsigned char*>(p.bias) + (h * p.bias_stride[0] + (row_ok ? qrow : 0) * p.bias_stride[1]) * esz;
+			bias_vec = !BIAS_F32 && ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) && (p.bias_stride[0] % 8 == 0) && (p.bias_stride[1] % 8 == 0);
+		}
+		// log2 variant: fragment-ordered workspace; the tile base is wave-uniform
+		const u32x4* ws_wave = nullptr;
+		if(L2DOM && has_bias) {
+			const int     n_qblocks = (int)((L + 31) / 32);
+			const int64_t qb        = FUSED ? (int64_t)qb_f : SPLIT ? (int64_t)qtile : (int64_t)qtile * NW + wave;
+			// query blocks beyond the last one only hold rows >= L; clamp so that loads stay in bounds
+			const int64_t qbc = qb < n_qblocks ? qb : n_qblocks - 1;
+			ws_wave = static_cast<const u32x4*>(p.workspace) + ((h * n_qblocks + qbc) * n_ktiles) * 256;
+		}
+		// (scalar base + per-lane 16-byte offset + scalar tile offset: no 64-bit pointer in vector registers)
+		const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(ws_wave), 0, ws_wave ? n_ktiles * 4096 : 0, 0x00020000);
+		const int                    ws_voff = lane * 16;
+
+		// ---- K/V tile loader: buffer loads that write LDS directly ----
+		// One wave load moves 1 KB: lane i -> LDS chunk i of the load's 1 KB window, i.e. tile row
+		// j*RPI + i/CPR, physical chunk i%CPR.  The lane picks the global chunk that belongs there
+		// under the swizzle; lanes of padded head columns (chunk*8 >= D) stay idle.
+		const u32x4 k_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1], (uint32_t)(((L - 1) * p.k_stride[2] + D) * 2));
+		const u32x4 v_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.v) + b * p.v_stride[0] + h * p.v_stride[1], (uint32_t)(((L - 1) * p.v_stride[2] + D) * 2));
+		const int  ld_row  = lane / CPR, ld_pc = lane % CPR;
+		const int  k_chunk = ld_pc ^ k_swizzle<DP>(ld_row);
+		const int  v_chunk = ld_pc ^ v_swizzle<DP>(ld_row);
+		const int  k_voff  = (int)(ld_row * p.k_stride[2] * 2) + k_chunk * 16;
+		const int  v_voff  = (int)(ld_row * p.v_stride[2] * 2) + v_chunk * 16;
+		const bool k_act   = k_chunk * 8 < D, v_act = v_chunk * 8 < D;
+		const int  k_tile_stride = (int)(KT * p.k_stride[2] * 2), v_tile_stride = (int)(KT * p.v_stride[2] * 2);
+		const int  k_ld_stride   = (int)(RPI * p.k_stride[2] * 2), v_ld_stride = (int)(RPI * p.v_stride[2] * 2);
+		const uint32_t k_lds_addr = lds_addr_of(k_lds), v_lds_addr = lds_addr_of(v_lds);
+		auto load_tile = [&](int kt, int buf) {
+			if(FUSED) return;  // K and V of every tile are already in LDS
+#pragma unroll
+			for(int t = 0; t < (SPLIT ? NI : NI / NW); t++) {
+				const int j = SPLIT ? t : wave + NW * t;  // split: this wavefront fetches whole tiles into its private buffers
+				if(k_act) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + j * 1024, k_voff + (kt * k_tile_stride + j * k_ld_stride));
+				if(v_act) lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + j * 1024, v_voff + (kt * v_tile_stride + j * v_ld_stride));
+			}
+		};
+
+		// ---- bias ring (BRING): the 32 x 64 bias tile of this wavefront's query block, 4 KB, travels
+		// HBM -> LDS by four LDS-direct loads of whole 128-byte row segments (eight lanes per row), two
+		// tiles ahead of its use and without occupying registers.  Slot layout: [row 32][128 B], the
+		// 16-byte chunk c of row r stored at chunk position c ^ (r & 7) so that the fragment reads (one
+		// chunk per lane, 32 rows at once) spread over the banks.  Rows past L lie beyond the buffer's
+		// range; chunks of keys past L (last tile) are sent there too, so padding behind a row's L valid
+		// entries is never read.  Whatever such lanes leave in LDS is finite: the ring starts zeroed.
+		const u32x4    b_rsrc    = raw_rsrc(BRING ? static_cast<const uint16_t*>(p.bias) + h * p.bias_stride[0] : nullptr,
+											BRING ? (uint32_t)(((L - 1) * p.bias_stride[1] + L) * 2) : 0u);
+		unsigned char* const bring = smem + LDS_SETS * 6 * TILE_BYTES + (BRING ? wave * 3 * 4096 : 0);
+		const uint32_t bring_addr = lds_addr_of(bring);
+		const int      b_voff     = (int)((lane >> 3) * p.bias_stride[1] * 2) + (((lane & 7) ^ (lane >> 3)) << 4);
+		const int      b_row0     = (int)((qtile * QT + (SPLIT ? 0 : wave * 32)) * p.bias_stride[1] * 2);
+		const int      b_row8     = (int)(8 * p.bias_stride[1] * 2);
+		const int      b_key      = ((lane & 7) ^ (lane >> 3)) * 8;  // first key of this lane's chunk within a tile
+		auto load_bias_tile = [&](int kt, int slot_i) {
+			if(!BRING) return;
+			const int in_row = kt * KT + b_key < (int)L ? b_voff + kt * (KT * 2) : 0x7FFF0000;
+#pragma unroll
+			for(int j = 0; j < 4; j++) lds_dma_b128(b_rsrc, bring_addr + slot_i * 4096 + j * 1024, in_row + (b_row0 + j * b_row8));
+		};
+		// fragment read: lane (n, half) takes chunk 4*sub + 2*c2 + half of row n
+		const int b_rd = n * 128 + (((n & 7) ^ half) << 4);
+
+		// Natural variant: four fragments in flight, each sub-tile's pair requested two stages before its
+		// use.  Log2 variant (BIAS_LATE): one pair only -- the registers are the scarce resource at four
+		// wavefronts per SIMD -- requested inside the previous stage, right after the matrix
+		// instructions that consume the pair before it.
+		constexpr bool BIAS_LATE = L2DOM;
+		u32x4 bfrag[4];
+		auto  load_bias_frags = [&](int kt, auto sub_c) {
+			constexpr int SUB = decltype(sub_c)::value;
+			if(!has_bias || BRING) return;
+			if(L2DOM) {
+#pragma unroll
+				for(int c2 = 0; c2 < 2; c2++)
+					bfrag[c2] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, ws_voff + (2 * SUB + c2) * 1024, kt * 4096, 0));
+				return;
+			}
+			const int64_t key0 = (int64_t)kt * KT + 8 * half;
+			if(bias_vec && (int64_t)(kt + 1) * KT <= L) {  // wave-uniform: whole tile in range, aligned rows
+				const uint16_t* bp = reinterpret_cast<const uint16_t*>(bias_row) + key0;
+				if(row_ok) {
+#pragma unroll
+					for(int f = 2 * SUB; f < 2 * SUB + 2; f++) bfrag[f] = *reinterpret_cast<const u32x4*>(bp + 16 * f);
+				} else {
+#pragma unroll
+					for(int f = 2 * SUB; f < 2 * SUB + 2; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
+				}
 			} else {
 #pragma unroll
-				for(int f = 2 * SUB; f < 2 * SUB + 2; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
+				for(int f = 2 * SUB; f < 2 * SUB + 2; f++) {
+					float v8[8];
+					load_bias8_guarded<BIAS_F32>(bias_row, key0 + 16 * f, L, row_ok, v8);
+#pragma unroll
+					for(int j = 0; j < 4; j++) bfrag[f][j] = pack_bf16x2(v8[2 * j], v8[2 * j + 1]);
+				}
 			}
-		} else {
+		};
+
+		// ---- per-lane LDS read addresses (bytes, for buffer 0 / sub-tile 0; the rest are immediates) ----
+		int k_rd[NC];
 #pragma unroll
-			for(int f = 2 * SUB; f < 2 * SUB + 2; f++) {
-				float v8[8];
-				load_bias8_guarded<BIAS_F32>(bias_row, key0 + 16 * f, L, row_ok, v8);
+		for(int c = 0; c < NC; c++) k_rd[c] = n * DP * 2 + (((2 * c + half) ^ k_swizzle<DP>(n)) << 4);
+		// V^T fragment reads: lane l: i = l%16, G = l/16 supplies the 8-byte chunk at tile row
+		// base + 4*(G/2) + i/4, column 32*db + 16*(G%2) + 4*(i%4); it receives 4 keys of column 32*db + l%32.
+		int v_rd[NDB];
+		{
+			const int i16 = lane & 15, G = lane >> 4;
+			const int row = 4 * (G >> 1) + (i16 >> 2);
 #pragma unroll
-				for(int j = 0; j < 4; j++) bfrag[f][j] = pack_bf16x2(v8[2 * j], v8[2 * j + 1]);
+			for(int db = 0; db < NDB; db++) {
+				const int col   = 32 * db + 16 * (G & 1) + 4 * (i16 & 3);
+				const int chunk = (col >> 3) ^ v_swizzle<DP>(row);
+				v_rd[db] = row * DP * 2 + chunk * 16 + (col & 7) * 2;
 			}
 		}
-	};
+		// mask table read address: lanes of the upper half-wave always read the zero entries
+		const int mask_rd     = mask_base + (half == 0 ? n * 4 : (n_ktiles * KT + n) * 4);
+		const int mask_stride = half == 0 ? KT * 4 : 0;
 
-	// ---- per-lane LDS read addresses (bytes, for buffer 0 / sub-tile 0; the rest are immediates) ----
-	int k_rd[NC];
-#pragma unroll
-	for(int c = 0; c < NC; c++) k_rd[c] = n * DP * 2 + (((2 * c + half) ^ k_swizzle<DP>(n)) << 4);
-	// V^T fragment reads: lane l: i = l%16, G = l/16 supplies the 8-byte chunk at tile row
-	// base + 4*(G/2) + i/4, column 32*db + 16*(G%2) + 4*(i%4); it receives 4 keys of column 32*db + l%32.
-	int v_rd[NDB];
-	{
-		const int i16 = lane & 15, G = lane >> 4;
-		const int row = 4 * (G >> 1) + (i16 >> 2);
-#pragma unroll
-		for(int db = 0; db < NDB; db++) {
-			const int col   = 32 * db + 16 * (G & 1) + 4 * (i16 & 3);
-			const int chunk = (col >> 3) ^ v_swizzle<DP>(row);
-			v_rd[db] = row * DP * 2 + chunk * 16 + (col & 7) * 2;
-		}
-	}
-	// mask table read address: lanes of the upper half-wave always read the zero entries
-	const int mask_rd     = (int)MASK_BASE + (half == 0 ? n * 4 : (n_ktiles * KT + n) * 4);
-	const int mask_stride = half == 0 ? KT * 4 : 0;
-
-	// ---- online-softmax state (per lane: one query row; the two halves hold disjoint keys) ----
-	float  m_ref = 0.f;  // reference maximum: log2 units and bf16-exact (log2 variant), natural units (natural variant)
-	float  mc    = 0.f;  // natural variant: m_ref * log2 e
-	f32x4  lacc  = {0.f, 0.f, 0.f, 0.f};  // [0] = this lane's row sum (complete: the same value in both half-waves)
-	f32x16 oacc[NDB];
-#pragma unroll
-	for(int db = 0; db < NDB; db++)
-#pragma unroll
-		for(int i = 0; i < 16; i++) oacc[db][i] = 0.f;
-
-	// Move the reference of every row whose maximum is not within REF_SLACK of it (all rows when
-	// `force`), rescale what has been accumulated, and re-express s (and a sub-tile that was
-	// already issued against the old reference) relative to the new one.
-	auto rereference = [&](f32x16& s, f32x16* pending, bool force) {
-		float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
-#pragma unroll
-		for(int i = 3; i < 15; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
-		mx = half_swap_max(fmaxf(mx, s[15]));
-		float alpha;
-		if(L2DOM) {
-			// s already has m_ref subtracted (by the mask MFMA)
-			const bool  need  = force || mx > REF_SLACK;
-			const float m_want = m_ref + mx;
-			const float m_hi   = bf16_bits_to_f32(f32_to_bf16_bits(need ? m_want : m_ref));
-			const float m_lo   = bf16_bits_to_f32(f32_to_bf16_bits((need ? m_want : m_ref) - m_hi));
-			const float m_new  = m_hi + m_lo;  // exactly what the mask MFMA will subtract (unchanged when !need)
-			const float delta  = m_new - m_ref;
-			alpha = force ? 1.f : __builtin_amdgcn_exp2f(-delta);  // nothing is accumulated yet when forced (first sub-tile)
-#pragma unroll
-			for(int i = 0; i < 16; i++) s[i] -= delta;
-			if(pending) {
-#pragma unroll
-				for(int i = 0; i < 16; i++) (*pending)[i] -= delta;
-			}
-			m_ref = m_new;
-			if(half == 0) {
-				maskB[0] = 0x3F80u | (f32_to_bf16_bits(-m_hi) << 16);
-				maskB[1] = f32_to_bf16_bits(-m_lo);
-			}
-		} else {
-			const bool  need  = force || mx > m_ref + REF_SLACK * 0.6931472f;
-			const float m_new = need ? mx : m_ref;
-			alpha = force ? 1.f : __builtin_amdgcn_exp2f((m_ref - m_new) * LOG2E);
-			m_ref = m_new;
-			mc    = m_new * LOG2E;
-		}
-		lacc[0] *= alpha;
+		// ---- online-softmax state (per lane: one query row; the two halves hold disjoint keys) ----
+		float  m_ref = 0.f;  // reference maximum: log2 units and bf16-exact (log2 variant), natural units (natural variant)
+		float  mc    = 0.f;  // natural variant: m_ref * log2 e
+		f32x4  lacc  = {0.f, 0.f, 0.f, 0.f};  // [0] = this lane's row sum (complete: the same value in both half-waves)
+		f32x16 oacc[NDB];
 #pragma unroll
 		for(int db = 0; db < NDB; db++)
 #pragma unroll
-			for(int i = 0; i < 16; i++) oacc[db][i] *= alpha;
-	};
+			for(int i = 0; i < 16; i++) oacc[db][i] = 0.f;
 
-	// p = exp2(s - reference) for logits [I0, I0+N) of a sub-tile, packed to bf16 pairs.  (The row sum is
-	// taken from the packed pairs on the matrix pipe, rowsum_mfma below: 16 vector adds per sub-tile
-	// cost more, and v_dot2c_f32_bf16 on the pairs does not execute concurrently with MFMA.)
-	auto exp_part = [&](const f32x16& s, u32x4 (&pf)[2], auto i0_c, auto n_c) {
-		constexpr int I0 = decltype(i0_c)::value, N = decltype(n_c)::value;
+		// Move the reference of every row whose maximum is not within REF_SLACK of it (all rows when
+		// `force`), rescale what has been accumulated, and re-express s (and a sub-tile that was
+		// already issued against the old reference) relative to the new one.
+		auto rereference = [&](f32x16& s, f32x16* pending, bool force) {
+			float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
 #pragma unroll
-		for(int i = I0; i < I0 + N; i += 2) {
-			float p0, p1;
+			for(int i = 3; i < 15; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
+			mx = half_swap_max(fmaxf(mx, s[15]));
+			float alpha;
 			if(L2DOM) {
-				p0 = __builtin_amdgcn_exp2f(s[i]);
-				p1 = __builtin_amdgcn_exp2f(s[i + 1]);
+				// s already has m_ref subtracted (by the mask MFMA)
+				const bool  need  = force || mx > REF_SLACK;
+				const float m_want = m_ref + mx;
+				const float m_hi   = bf16_bits_to_f32(f32_to_bf16_bits(need ? m_want : m_ref));
+				const float m_lo   = bf16_bits_to_f32(f32_to_bf16_bits((need ? m_want : m_ref) - m_hi));
+				const float m_new  = m_hi + m_lo;  // exactly what the mask MFMA will subtract (unchanged when !need)
+				const float delta  = m_new - m_ref;
+				alpha = force ? 1.f : __builtin_amdgcn_exp2f(-delta);  // nothing is accumulated yet when forced (first sub-tile)
+#pragma unroll
+				for(int i = 0; i < 16; i++) s[i] -= delta;
+				if(pending) {
+#pragma unroll
+					for(int i = 0; i < 16; i++) (*pending)[i] -= delta;
+				}
+				m_ref = m_new;
+				if(half == 0) {
+					maskB[0] = 0x3F80u | (f32_to_bf16_bits(-m_hi) << 16);
+					maskB[1] = f32_to_bf16_bits(-m_lo);
+				}
 			} else {
-				p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], LOG2E, -mc));
-				p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], LOG2E, -mc));
+				const bool  need  = force || mx > m_ref + REF_SLACK * 0.6931472f;
+				const float m_new = need ? mx : m_ref;
+				alpha = force ? 1.f : __builtin_amdgcn_exp2f((m_ref - m_new) * LOG2E);
+				m_ref = m_new;
+				mc    = m_new * LOG2E;
 			}
-			pf[i >> 3][(i & 7) >> 1] = pack_bf16x2(p0, p1);
+			lacc[0] *= alpha;
+#pragma unroll
+			for(int db = 0; db < NDB; db++)
+#pragma unroll
+				for(int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+		};
+
+		// p = exp2(s - reference) for logits [I0, I0+N) of a sub-tile, packed to bf16 pairs.  (The row sum is
+		// taken from the packed pairs on the matrix pipe, rowsum_mfma below: 16 vector adds per sub-tile
+		// cost more, and v_dot2c_f32_bf16 on the pairs does not execute concurrently with MFMA.)
+		auto exp_part = [&](const f32x16& s, u32x4 (&pf)[2], auto i0_c, auto n_c) {
+			constexpr int I0 = decltype(i0_c)::value, N = decltype(n_c)::value;
+#pragma unroll
+			for(int i = I0; i < I0 + N; i += 2) {
+				float p0, p1;
+				if(L2DOM) {
+					p0 = __builtin_amdgcn_exp2f(s[i]);
+					p1 = __builtin_amdgcn_exp2f(s[i + 1]);
+				} else {
+					p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], LOG2E, -mc));
+					p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], LOG2E, -mc));
+				}
+				pf[i >> 3][(i & 7) >> 1] = pack_bf16x2(p0, p1);
+			}
+		};
+
+		// One pipeline stage.  On entry `sc` holds the finished S^T of sub-tile j, `pprev`/`vprev` the
+		// P^T and V^T fragments of sub-tile j-1.  The stage interleaves, one matrix instruction per
+		// handful of vector instructions so that both pipes stay busy within this wavefront:
+		//     matrix pipe                         vector ALU
+		//     O^T += V^T . P^T   (sub-tile j-1)   exp2 / pack of sub-tile j
+		//     S^T of sub-tile j+1 (K.Q^T, bias,   row sum of sub-tile j
+		//                          mask)
+		// and leaves S^T(j+1) in `sc`, P^T(j) in `pprev`, V^T(j) fragments in `vprev`.
+		// k_off / v_off: byte offsets of the LDS buffers holding sub-tile j+1's K rows and sub-tile j's V rows;
+		// SUBN / SUBC: which half of those tiles; FB: first bias fragment of sub-tile j+1.
+		f32x16 sc;
+		u32x4  pprev[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
+		u32x4  vprev[2][NDB];
+#pragma unroll
+		for(int cp = 0; cp < 2; cp++)
+#pragma unroll
+			for(int db = 0; db < NDB; db++) vprev[cp][db] = u32x4{0u, 0u, 0u, 0u};
+
+		// Row sums on the matrix pipe: a 16x16x32 MFMA whose A operand is a 0/1 pattern adds the 16 packed
+		// probabilities of a fragment (both half-waves) for every query; with this pattern register 0 of
+		// the result holds, in every lane, the sum for that lane's own query row.  As a B operand of the
+		// 16x16x32 shape the P fragment's lane l is column l%16, contraction group l/16, and holds query
+		// l%32: groups 0,2 belong to queries 0..15, groups 1,3 to queries 16..31.  Output register 0 of
+		// lane l is row 4*(l/16): rows 0 and 8 select the even groups, rows 4 and 12 the odd ones.
+		u32x4 ones_a;
+		{
+			const int  i16 = lane & 15, kg = lane >> 4;
+			const bool on  = ((i16 == 0 || i16 == 8) && (kg & 1) == 0) || ((i16 == 4 || i16 == 12) && (kg & 1) == 1);
+			const uint32_t w = on ? 0x3F803F80u : 0u;
+			ones_a = u32x4{w, w, w, w};
 		}
-	};
-
-	// One pipeline stage.  On entry `sc` holds the finished S^T of sub-tile j, `pprev`/`vprev` the
-	// P^T and V^T fragments of sub-tile j-1.  The stage interleaves, one matrix instruction per
-	// handful of vector instructions so that both pipes stay busy within this wavefront:
-	//     matrix pipe                         vector ALU
-	//     O^T += V^T . P^T   (sub-tile j-1)   exp2 / pack of sub-tile j
-	//     S^T of sub-tile j+1 (K.Q^T, bias,   row sum of sub-tile j
-	//                          mask)
-	// and leaves S^T(j+1) in `sc`, P^T(j) in `pprev`, V^T(j) fragments in `vprev`.
-	// k_off / v_off: byte offsets of the LDS buffers holding sub-tile j+1's K rows and sub-tile j's V rows;
-	// SUBN / SUBC: which half of those tiles; FB: first bias fragment of sub-tile j+1.
-	f32x16 sc;
-	u32x4  pprev[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
-	u32x4  vprev[2][NDB];
+		auto rowsum_mfma = [&](const u32x4& pf) {
+			lacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ones_a), __builtin_bit_cast(bf16x8, pf), lacc, 0, 0, 0);
+		};
+		auto read_kfrag = [&](int k_off, int sub, int c) -> u32x4 { return *reinterpret_cast<const u32x4*>(k_lds + k_rd[c] + k_off + sub * 32 * DP * 2); };
+		auto read_vfrags = [&](int v_off, int sub) {
 #pragma unroll
-	for(int cp = 0; cp < 2; cp++)
+			for(int cp = 0; cp < 2; cp++)
 #pragma unroll
-		for(int db = 0; db < NDB; db++) vprev[cp][db] = u32x4{0u, 0u, 0u, 0u};
+				for(int db = 0; db < NDB; db++)
+#pragma unroll
+					for(int t = 0; t < 2; t++) {
+						const int   off = v_off + (32 * sub + 16 * cp + 8 * t) * DP * 2;
+						const s16x4 r   = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(v_lds + v_rd[db] + off));
+						const u32x2 rr  = __builtin_bit_cast(u32x2, r);
+						vprev[cp][db][2 * t]     = rr[0];
+						vprev[cp][db][2 * t + 1] = rr[1];
+					}
+		};
+		auto bias_mfma = [&](f32x16 s, int f) -> f32x16 {
+			if(L2DOM) return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, idf[f & 1]), __builtin_bit_cast(f16x8, bfrag[f & 1]), s, 0, 0, 0);
+			return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, idf[f & 1]), __builtin_bit_cast(bf16x8, bfrag[f]), s, 0, 0, 0);
+		};
+		// plain (not interleaved) S^T of one sub-tile; used once, for the very first sub-tile
+		auto compute_s_plain = [&](int k_off, int sub, int mask_addr, int fb) -> f32x16 {
+			f32x16 s;
+#pragma unroll
+			for(int i = 0; i < 16; i++) s[i] = 0.f;
+#pragma unroll
+			for(int c = 0; c < NC; c++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, read_kfrag(k_off, sub, c)), qf[c], s, 0, 0, 0);
+			s = bias_mfma(s, fb);
+			s = bias_mfma(s, fb + 1);
+			maskA[0] = *reinterpret_cast<const uint32_t*>(smem + mask_addr + sub * 32 * 4);
+			return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), s, 0, 0, 0);
+		};
 
-	// Row sums on the matrix pipe: a 16x16x32 MFMA whose A operand is a 0/1 pattern adds the 16 packed
-	// probabilities of a fragment (both half-waves) for every query; with this pattern register 0 of
-	// the result holds, in every lane, the sum for that lane's own query row.  As a B operand of the
-	// 16x16x32 shape the P fragment's lane l is column l%16, contraction group l/16, and holds query
-	// l%32: groups 0,2 belong to queries 0..15, groups 1,3 to queries 16..31.  Output register 0 of
-	// lane l is row 4*(l/16): rows 0 and 8 select the even groups, rows 4 and 12 the odd ones.
-	u32x4 ones_a;
-	{
-		const int  i16 = lane & 15, kg = lane >> 4;
-		const bool on  = ((i16 == 0 || i16 == 8) && (kg & 1) == 0) || ((i16 == 4 || i16 == 12) && (kg & 1) == 1);
-		const uint32_t w = on ? 0x3F803F80u : 0u;
-		ones_a = u32x4{w, w, w, w};
-	}
-	auto rowsum_mfma = [&](const u32x4& pf) {
-		lacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ones_a), __builtin_bit_cast(bf16x8, pf), lacc, 0, 0, 0);
-	};
-	auto read_kfrag = [&](int k_off, int sub, int c) -> u32x4 { return *reinterpret_cast<const u32x4*>(k_lds + k_rd[c] + k_off + sub * 32 * DP * 2); };
-	auto read_vfrags = [&](int v_off, int sub) {
+		auto read_bias_ring = [&](int slot_off, auto sub_c) {
+			constexpr int SUB = decltype(sub_c)::value;
+#pragma unroll
+			for(int c2 = 0; c2 < 2; c2++) bfrag[2 * SUB + c2] = *reinterpret_cast<const u32x4*>(bring + slot_off + (b_rd ^ ((4 * SUB + 2 * c2) << 4)));
+		};
+		// ring_off (BRING): byte offset of the ring slot that holds the bias tile of sub-tile j+1
+		auto stage = [&](auto subn_c, int k_off, int mask_addr_next, int v_off, auto subc_c, int bias_kt, auto bias_sub_c, int ring_off) {
+			constexpr int SUBN = decltype(subn_c)::value, SUBC = decltype(subc_c)::value, FB = 2 * SUBN;
+			if(BRING) read_bias_ring(ring_off, subn_c);
+			// operands of S^T(j+1) from LDS
+			u32x4 kf[NC];
+#pragma unroll
+			for(int c = 0; c < NC; c++) kf[c] = read_kfrag(k_off, SUBN, c);
+			maskA[0] = *reinterpret_cast<const uint32_t*>(smem + mask_addr_next + SUBN * 32 * 4);
+			u32x4  pcur[2];
+			f32x16 sn;
+#pragma unroll
+			for(int i = 0; i < 16; i++) sn[i] = 0.f;
+			// One matrix instruction, then a handful of vector instructions, and so on: a dependent
+			// MFMA chain would otherwise stall the wavefront for the full 32-cycle pass of each link.
+			// The scheduling barriers keep the compiler from regrouping the chunks.
+#define AF3_CHUNK_END() __builtin_amdgcn_sched_barrier(0)
+			AF3_CHUNK_END();
+			// O^T += V^T . P^T of the previous sub-tile, exp2 of this one
+#pragma unroll
+			for(int db = 0; db < NDB; db++)
+				oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[0][db]), __builtin_bit_cast(bf16x8, pprev[0]), oacc[db], 0, 0, 0);
+			exp_part(sc, pcur, ic<0>{}, ic<2>{});
+			AF3_CHUNK_END();
+#pragma unroll
+			for(int db = 0; db < NDB; db++)
+				oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[1][db]), __builtin_bit_cast(bf16x8, pprev[1]), oacc[db], 0, 0, 0);
+			exp_part(sc, pcur, ic<2>{}, ic<2>{});
+			AF3_CHUNK_END();
+			// S^T of the next sub-tile
+			sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[0]), qf[0], sn, 0, 0, 0);
+			// V^T fragments of this sub-tile for the next stage's PV product: issued as soon as the two PV
+			// MFMAs above have consumed the previous fragments, a whole stage before their use
+			read_vfrags(v_off, SUBC);
+			exp_part(sc, pcur, ic<4>{}, ic<2>{});
+			AF3_CHUNK_END();
+			sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[1]), qf[1], sn, 0, 0, 0);
+			exp_part(sc, pcur, ic<6>{}, ic<2>{});
+			AF3_CHUNK_END();
+#pragma unroll
+			for(int c = 2; c < NC; c++) sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[c]), qf[c], sn, 0, 0, 0);
+			// (the bias MFMAs run unconditionally -- on zero fragments when there is no bias -- so that the
+			// whole stage stays one basic block)
+			sn = bias_mfma(sn, FB);
+			const float l_before = lacc[0];
+			rowsum_mfma(pcur[0]);
+			exp_part(sc, pcur, ic<8>{}, ic<2>{});
+			AF3_CHUNK_END();
+			sn = bias_mfma(sn, FB + 1);
+			exp_part(sc, pcur, ic<10>{}, ic<2>{});
+			AF3_CHUNK_END();
+			if(BIAS_LATE) load_bias_frags(bias_kt, bias_sub_c);  // pair of the sub-tile after the next one
+			sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), sn, 0, 0, 0);
+			exp_part(sc, pcur, ic<12>{}, ic<4>{});
+			AF3_CHUNK_END();
+#undef AF3_CHUNK_END
+			rowsum_mfma(pcur[1]);
+			// The running sum stays below L * 2^REF_SLACK <= 2^25 while every probability respects the
+			// reference, so this also catches a single probability near or beyond the limit (inf, NaN).
+			if(__ballot(!(lacc[0] < PSUM_LIMIT))) {  // rare
+				lacc[0] = l_before;
+				rereference(sc, &sn, false);
+				exp_part(sc, pcur, ic<0>{}, ic<16>{});
+				rowsum_mfma(pcur[0]);
+				rowsum_mfma(pcur[1]);
+			}
+			sc       = sn;
+			pprev[0] = pcur[0];
+			pprev[1] = pcur[1];
+		};
+
+		// ---- which live tiles this wavefront walks: all of them, or every NW-th one when splitting ----
+		const int my_first = SPLIT ? wave : 0, my_step = SPLIT ? NW : 1;
+		const int my_n     = SPLIT ? (nlive > wave ? (nlive - wave + NW - 1) / NW : 0) : nlive;
+		auto live_at = [&](int j) -> int { return (int)live_list[my_first + (j < my_n ? j : my_n - 1) * my_step]; };
+
+		if(my_n > 0) {
+			// ---- prologue: first two tiles, first sub-tile's S^T and its row maximum ----
+			const int kt0 = __builtin_amdgcn_readfirstlane(live_at(0));
+			load_tile(kt0, 0);
+			load_bias_tile(kt0, 0);
+			if(my_n > 1) {
+				load_tile(__builtin_amdgcn_readfirstlane(live_at(1)), 1);
+				load_bias_tile(__builtin_amdgcn_readfirstlane(live_at(1)), 1);
+			}
+#pragma unroll
+			for(int f = 0; f < 4; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
+			load_bias_frags(kt0, ic<0>{});
+			if(!BIAS_LATE) load_bias_frags(kt0, ic<1>{});
+			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+			if(!SPLIT && !FUSED) __syncthreads();
+			if(BRING) read_bias_ring(0, ic<0>{});
+			sc = compute_s_plain(FUSED ? kt0 * TILE_BYTES : 0, 0, mask_rd + kt0 * mask_stride, 0);
+			rereference(sc, nullptr, true);
+			if(BIAS_LATE) load_bias_frags(kt0, ic<1>{});
+			else if(my_n > 1) load_bias_frags(__builtin_amdgcn_readfirstlane(live_at(1)), ic<0>{});
+
+			int buf = 0;  // LDS buffer of tile `it` (it % 3)
+			// tile indices of iterations it, it+1, it+2 are carried in scalar registers; the list entry for
+			// it+3 is fetched at the top of an iteration and only consumed at its end
+			int kt = kt0, kt1 = __builtin_amdgcn_readfirstlane(live_at(1)), kt2 = __builtin_amdgcn_readfirstlane(live_at(2));
+			for(int it = 0; it < my_n; it++) {
+				const int kt3_v = live_at(it + 3);
+				const int bufn = buf == 2 ? 0 : buf + 1, bufnn = bufn == 2 ? 0 : bufn + 1;
+				// LDS offsets of tile it and of tile it+1: ring buffers, or the tiles' own places when all of K and V is resident
+				const int off_cur = (FUSED ? kt : buf) * TILE_BYTES, off_next = (FUSED ? kt1 : bufn) * TILE_BYTES;
+				// sub-tile (it, 0): next is (it, 1) in the same buffer
+				stage(ic<1>{}, off_cur, mask_rd + kt * mask_stride, off_cur, ic<0>{}, kt1, ic<0>{}, buf * 4096);
+				if(!BIAS_LATE) load_bias_frags(kt1, ic<1>{});
+				// Tile it+1 (issued one iteration ago) must have landed, and every wavefront must be done
+				// with tile it-1, whose buffer tile it+2 is about to overwrite.  Loads complete in issue
+				// order; the only loads this wavefront has issued since that tile are bias fragments: two in
+				// the log2 variant (the pair requested inside the stage above), which may stay in flight.
+				if(!FUSED) {
+					if(L2DOM && has_bias) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+					else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+				}
+				if(!SPLIT && !FUSED) __syncthreads();
+				if(it + 2 < my_n) {
+					load_tile(kt2, bufnn);
+					load_bias_tile(kt2, bufnn);  // (its slot held tile it-1, last read in the stage above)
+				}
+				// sub-tile (it, 1): next is (it+1, 0) in the next buffer (harmless stale data after the last tile)
+				stage(ic<0>{}, off_next, mask_rd + kt1 * mask_stride, off_cur, ic<1>{}, kt1, ic<1>{}, bufn * 4096);
+				if(!BIAS_LATE) load_bias_frags(kt2, ic<0>{});
+				buf = bufn;
+				kt  = kt1;
+				kt1 = kt2;
+				kt2 = __builtin_amdgcn_readfirstlane(kt3_v);
+			}
+		}
+		// the last sub-tile's PV product
 #pragma unroll
 		for(int cp = 0; cp < 2; cp++)
 #pragma unroll
 			for(int db = 0; db < NDB; db++)
-#pragma unroll
-				for(int t = 0; t < 2; t++) {
-					const int   off = v_off + (32 * sub + 16 * cp + 8 * t) * DP * 2;
-					const s16x4 r   = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(v_lds + v_rd[db] + off));
-					const u32x2 rr  = __builtin_bit_cast(u32x2, r);
-					vprev[cp][db][2 * t]     = rr[0];
-					vprev[cp][db][2 * t + 1] = rr[1];
-				}
-	};
-	auto bias_mfma = [&](f32x16 s, int f) -> f32x16 {
-		if(L2DOM) return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, idf[f & 1]), __builtin_bit_cast(f16x8, bfrag[f & 1]), s, 0, 0, 0);
-		return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, idf[f & 1]), __builtin_bit_cast(bf16x8, bfrag[f]), s, 0, 0, 0);
-	};
-	// plain (not interleaved) S^T of one sub-tile; used once, for the very first sub-tile
-	auto compute_s_plain = [&](int k_off, int sub, int mask_addr, int fb) -> f32x16 {
-		f32x16 s;
-#pragma unroll
-		for(int i = 0; i < 16; i++) s[i] = 0.f;
-#pragma unroll
-		for(int c = 0; c < NC; c++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, read_kfrag(k_off, sub, c)), qf[c], s, 0, 0, 0);
-		s = bias_mfma(s, fb);
-		s = bias_mfma(s, fb + 1);
-		maskA[0] = *reinterpret_cast<const uint32_t*>(smem + mask_addr + sub * 32 * 4);
-		return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), s, 0, 0, 0);
-	};
+				oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[cp][db]), __builtin_bit_cast(bf16x8, pprev[cp]), oacc[db], 0, 0, 0);
 
-	auto read_bias_ring = [&](int slot_off, auto sub_c) {
-		constexpr int SUB = decltype(sub_c)::value;
+		if(SPLIT) {
+			// ---- merge the partial results of the NW wavefronts (same 32 query rows, disjoint keys) ----
+			asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+			__syncthreads();  // all K/V buffers are dead: reuse the front of LDS
+			float* const mred = reinterpret_cast<float*>(smem);        // [NW][32] reference maxima
+			float* const obuf = mred + NW * 32;                        // [NW][16*NDB + 1][64]
+			if(half == 0) mred[wave * 32 + n] = my_n > 0 ? m_ref : -INFINITY;
+			__syncthreads();
+			float mstar = mred[n];
 #pragma unroll
-		for(int c2 = 0; c2 < 2; c2++) bfrag[2 * SUB + c2] = *reinterpret_cast<const u32x4*>(bring + slot_off + (b_rd ^ ((4 * SUB + 2 * c2) << 4)));
-	};
-	// ring_off (BRING): byte offset of the ring slot that holds the bias tile of sub-tile j+1
-	auto stage = [&](auto subn_c, int k_off, int mask_addr_next, int v_off, auto subc_c, int bias_kt, auto bias_sub_c, int ring_off) {
-		constexpr int SUBN = decltype(subn_c)::value, SUBC = decltype(subc_c)::value, FB = 2 * SUBN;
-		if(BRING) read_bias_ring(ring_off, subn_c);
-		// operands of S^T(j+1) from LDS
-		u32x4 kf[NC];
-#pragma unroll
-		for(int c = 0; c < NC; c++) kf[c] = read_kfrag(k_off, SUBN, c);
-		maskA[0] = *reinterpret_cast<const uint32_t*>(smem + mask_addr_next + SUBN * 32 * 4);
-		u32x4  pcur[2];
-		f32x16 sn;
-#pragma unroll
-		for(int i = 0; i < 16; i++) sn[i] = 0.f;
-		// One matrix instruction, then a handful of vector instructions, and so on: a dependent
-		// MFMA chain would otherwise stall the wavefront for the full 32-cycle pass of each link.
-		// The scheduling barriers keep the compiler from regrouping the chunks.
-#define AF3_CHUNK_END() __builtin_amdgcn_sched_barrier(0)
-		AF3_CHUNK_END();
-		// O^T += V^T . P^T of the previous sub-tile, exp2 of this one
-#pragma unroll
-		for(int db = 0; db < NDB; db++)
-			oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[0][db]), __builtin_bit_cast(bf16x8, pprev[0]), oacc[db], 0, 0, 0);
-		exp_part(sc, pcur, ic<0>{}, ic<2>{});
-		AF3_CHUNK_END();
-#pragma unroll
-		for(int db = 0; db < NDB; db++)
-			oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[1][db]), __builtin_bit_cast(bf16x8, pprev[1]), oacc[db], 0, 0, 0);
-		exp_part(sc, pcur, ic<2>{}, ic<2>{});
-		AF3_CHUNK_END();
-		// S^T of the next sub-tile
-		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[0]), qf[0], sn, 0, 0, 0);
-		// V^T fragments of this sub-tile for the next stage's PV product: issued as soon as the two PV
-		// MFMAs above have consumed the previous fragments, a whole stage before their use
-		read_vfrags(v_off, SUBC);
-		exp_part(sc, pcur, ic<4>{}, ic<2>{});
-		AF3_CHUNK_END();
-		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[1]), qf[1], sn, 0, 0, 0);
-		exp_part(sc, pcur, ic<6>{}, ic<2>{});
-		AF3_CHUNK_END();
-#pragma unroll
-		for(int c = 2; c < NC; c++) sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[c]), qf[c], sn, 0, 0, 0);
-		// (the bias MFMAs run unconditionally -- on zero fragments when there is no bias -- so that the
-		// whole stage stays one basic block)
-		sn = bias_mfma(sn, FB);
-		const float l_before = lacc[0];
-		rowsum_mfma(pcur[0]);
-		exp_part(sc, pcur, ic<8>{}, ic<2>{});
-		AF3_CHUNK_END();
-		sn = bias_mfma(sn, FB + 1);
-		exp_part(sc, pcur, ic<10>{}, ic<2>{});
-		AF3_CHUNK_END();
-		if(BIAS_LATE) load_bias_frags(bias_kt, bias_sub_c);  // pair of the sub-tile after the next one
-		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, maskA), __builtin_bit_cast(bf16x8, maskB), sn, 0, 0, 0);
-		exp_part(sc, pcur, ic<12>{}, ic<4>{});
-		AF3_CHUNK_END();
-#undef AF3_CHUNK_END
-		rowsum_mfma(pcur[1]);
-		// The running sum stays below L * 2^REF_SLACK <= 2^25 while every probability respects the
-		// reference, so this also catches a single probability near or beyond the limit (inf, NaN).
-		if(__ballot(!(lacc[0] < PSUM_LIMIT))) {  // rare
-			lacc[0] = l_before;
-			rereference(sc, &sn, false);
-			exp_part(sc, pcur, ic<0>{}, ic<16>{});
-			rowsum_mfma(pcur[0]);
-			rowsum_mfma(pcur[1]);
-		}
-		sc       = sn;
-		pprev[0] = pcur[0];
-		pprev[1] = pcur[1];
-	};
-
-	// ---- which live tiles this wavefront walks: all of them, or every NW-th one when splitting ----
-	const int my_first = SPLIT ? wave : 0, my_step = SPLIT ? NW : 1;
-	const int my_n     = SPLIT ? (nlive > wave ? (nlive - wave + NW - 1) / NW : 0) : nlive;
-	auto live_at = [&](int j) -> int { return (int)live_list[my_first + (j < my_n ? j : my_n - 1) * my_step]; };
-
-	if(my_n > 0) {
-		// ---- prologue: first two tiles, first sub-tile's S^T and its row maximum ----
-		const int kt0 = __builtin_amdgcn_readfirstlane(live_at(0));
-		load_tile(kt0, 0);
-		load_bias_tile(kt0, 0);
-		if(my_n > 1) {
-			load_tile(__builtin_amdgcn_readfirstlane(live_at(1)), 1);
-			load_bias_tile(__builtin_amdgcn_readfirstlane(live_at(1)), 1);
-		}
-#pragma unroll
-		for(int f = 0; f < 4; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
-		load_bias_frags(kt0, ic<0>{});
-		if(!BIAS_LATE) load_bias_frags(kt0, ic<1>{});
-		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-		if(!SPLIT) __syncthreads();
-		if(BRING) read_bias_ring(0, ic<0>{});
-		sc = compute_s_plain(0, 0, mask_rd + kt0 * mask_stride, 0);
-		rereference(sc, nullptr, true);
-		if(BIAS_LATE) load_bias_frags(kt0, ic<1>{});
-		else if(my_n > 1) load_bias_frags(__builtin_amdgcn_readfirstlane(live_at(1)), ic<0>{});
-
-		int buf = 0;  // LDS buffer of tile `it` (it % 3)
-		// tile indices of iterations it, it+1, it+2 are carried in scalar registers; the list entry for
-		// it+3 is fetched at the top of an iteration and only consumed at its end
-		int kt = kt0, kt1 = __builtin_amdgcn_readfirstlane(live_at(1)), kt2 = __builtin_amdgcn_readfirstlane(live_at(2));
-		for(int it = 0; it < my_n; it++) {
-			const int kt3_v = live_at(it + 3);
-			const int bufn = buf == 2 ? 0 : buf + 1, bufnn = bufn == 2 ? 0 : bufn + 1;
-			// sub-tile (it, 0): next is (it, 1) in the same buffer
-			stage(ic<1>{}, buf * TILE_BYTES, mask_rd + kt * mask_stride, buf * TILE_BYTES, ic<0>{}, kt1, ic<0>{}, buf * 4096);
-			if(!BIAS_LATE) load_bias_frags(kt1, ic<1>{});
-			// Tile it+1 (issued one iteration ago) must have landed, and every wavefront must be done
-			// with tile it-1, whose buffer tile it+2 is about to overwrite.  Loads complete in issue
-			// order; the only loads this wavefront has issued since that tile are bias fragments: two in
-			// the log2 variant (the pair requested inside the stage above), which may stay in flight.
-			if(L2DOM && has_bias) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-			else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-			if(!SPLIT) __syncthreads();
-			if(it + 2 < my_n) {
-				load_tile(kt2, bufnn);
-				load_bias_tile(kt2, bufnn);  // (its slot held tile it-1, last read in the stage above)
-			}
-			// sub-tile (it, 1): next is (it+1, 0) in the next buffer (harmless stale data after the last tile)
-			stage(ic<0>{}, bufn * TILE_BYTES, mask_rd + kt1 * mask_stride, buf * TILE_BYTES, ic<1>{}, kt1, ic<1>{}, bufn * 4096);
-			if(!BIAS_LATE) load_bias_frags(kt2, ic<0>{});
-			buf = bufn;
-			kt  = kt1;
-			kt1 = kt2;
-			kt2 = __builtin_amdgcn_readfirstlane(kt3_v);
-		}
-	}
-	// the last sub-tile's PV product
-#pragma unroll
-	for(int cp = 0; cp < 2; cp++)
-#pragma unroll
-		for(int db = 0; db < NDB; db++)
-			oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[cp][db]), __builtin_bit_cast(bf16x8, pprev[cp]), oacc[db], 0, 0, 0);
-
-	if(SPLIT) {
-		// ---- merge the partial results of the NW wavefronts (same 32 query rows, disjoint keys) ----
-		asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-		__syncthreads();  // all K/V buffers are dead: reuse the front of LDS
-		float* const mred = reinterpret_cast<float*>(smem);        // [NW][32] reference maxima
-		float* const obuf = mred + NW * 32;                        // [NW][16*NDB + 1][64]
-		if(half == 0) mred[wave * 32 + n] = my_n > 0 ? m_ref : -INFINITY;
-		__syncthreads();
-		float mstar = mred[n];
-#pragma unroll
-		for(int w = 1; w < NW; w++) mstar = fmaxf(mstar, mred[w * 32 + n]);
-		const float scale_w = my_n > 0 ? __builtin_amdgcn_exp2f((m_ref - mstar) * (L2DOM ? 1.f : LOG2E)) : 0.f;
-		lacc[0] *= scale_w;
-#pragma unroll
-		for(int db = 0; db < NDB; db++)
-#pragma unroll
-			for(int i = 0; i < 16; i++) oacc[db][i] *= scale_w;
-		if(wave > 0) {
-			float* mine = obuf + wave * (16 * NDB + 1) * 64 + lane;
+			for(int w = 1; w < NW; w++) mstar = fmaxf(mstar, mred[w * 32 + n]);
+			const float scale_w = my_n > 0 ? __builtin_amdgcn_exp2f((m_ref - mstar) * (L2DOM ? 1.f : LOG2E)) : 0.f;
+			lacc[0] *= scale_w;
 #pragma unroll
 			for(int db = 0; db < NDB; db++)
 #pragma unroll
-				for(int i = 0; i < 16; i++) mine[(db * 16 + i) * 64] = oacc[db][i];
-			mine[16 * NDB * 64] = lacc[0];
-		}
-		__syncthreads();
-		if(wave > 0) return;
+				for(int i = 0; i < 16; i++) oacc[db][i] *= scale_w;
+			if(wave > 0) {
+				float* mine = obuf + wave * (16 * NDB + 1) * 64 + lane;
 #pragma unroll
-		for(int w = 1; w < NW; w++) {
-			const float* theirs = obuf + w * (16 * NDB + 1) * 64 + lane;
+				for(int db = 0; db < NDB; db++)
+#pragma unroll
+					for(int i = 0; i < 16; i++) mine[(db * 16 + i) * 64] = oacc[db][i];
+				mine[16 * NDB * 64] = lacc[0];
+			}
+			__syncthreads();
+			if(wave > 0) return;
+#pragma unroll
+			for(int w = 1; w < NW; w++) {
+				const float* theirs = obuf + w * (16 * NDB + 1) * 64 + lane;
+#pragma unroll
+				for(int db = 0; db < NDB; db++)
+#pragma unroll
+					for(int i = 0; i < 16; i++) oacc[db][i] += theirs[(db * 16 + i) * 64];
+				lacc[0] += theirs[16 * NDB * 64];
+			}
+		}
+
+		// ---- epilogue: O^T register i of block db is head column 32*db + 8*(i/4) + 4*half + i%4 ----
+		const float l_tot = lacc[0];
+		const float inv   = 1.f / l_tot;
+		if(row_ok) {
+			const int64_t ooff = b * p.out_stride[0] + h * p.out_stride[1] + qrow * p.out_stride[2];
 #pragma unroll
 			for(int db = 0; db < NDB; db++)
 #pragma unroll
-				for(int i = 0; i < 16; i++) oacc[db][i] += theirs[(db * 16 + i) * 64];
-			lacc[0] += theirs[16 * NDB * 64];
+				for(int g4 = 0; g4 < 4; g4++) {
+					const int d0 = 32 * db + 8 * g4 + 4 * half;
+					if(d0 >= D) continue;
+					float o0 = oacc[db][4 * g4] * inv, o1 = oacc[db][4 * g4 + 1] * inv;
+					float o2 = oacc[db][4 * g4 + 2] * inv, o3 = oacc[db][4 * g4 + 3] * inv;
+					if constexpr(FUSED) {
+						const u32x2 gw = {gate_pk[g4 >> 1][2 * (g4 & 1)], gate_pk[g4 >> 1][2 * (g4 & 1) + 1]};
+						o0 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] & 0xffffu)), o1 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] >> 16));
+						o2 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] & 0xffffu)), o3 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] >> 16));
+					} else if(p.gate) {  // out *= sigmoid(gate): four consecutive head columns = one 8-byte load
+						const u32x2 gw = *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(p.gate) + b * p.gate_stride[0] + h * p.gate_stride[1] + qrow * p.gate_stride[2] + d0);
+						o0 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] & 0xffffu)), o1 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] >> 16));
+						o2 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] & 0xffffu)), o3 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] >> 16));
+					}
+					if(p.out_dtype == AF3_BF16) {
+						u32x2 w = {pack_bf16x2(o0, o1), pack_bf16x2(o2, o3)};
+						*reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.out) + ooff + d0) = w;
+					} else {
+						float4 w = {o0, o1, o2, o3};
+						*reinterpret_cast<float4*>(static_cast<float*>(p.out) + ooff + d0) = w;
+					}
+				}
 		}
-	}
-
-	// ---- epilogue: O^T register i of block db is head column 32*db + 8*(i/4) + 4*half + i%4 ----
-	const float l_tot = lacc[0];
-	const float inv   = 1.f / l_tot;
-	if(row_ok) {
-		const int64_t ooff = b * p.out_stride[0] + h * p.out_stride[1] + qrow * p.out_stride[2];
-#pragma unroll
-		for(int db = 0; db < NDB; db++)
-#pragma unroll
-			for(int g4 = 0; g4 < 4; g4++) {
-				const int d0 = 32 * db + 8 * g4 + 4 * half;
-				if(d0 >= D) continue;
-				float o0 = oacc[db][4 * g4] * inv, o1 = oacc[db][4 * g4 + 1] * inv;
-				float o2 = oacc[db][4 * g4 + 2] * inv, o3 = oacc[db][4 * g4 + 3] * inv;
-				if(p.gate) {  // out *= sigmoid(gate): four consecutive head columns = one 8-byte load
-					const u32x2 gw = *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(p.gate) + b * p.gate_stride[0] + h * p.gate_stride[1] + qrow * p.gate_stride[2] + d0);
-					o0 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] & 0xffffu)), o1 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] >> 16));
-					o2 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] & 0xffffu)), o3 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] >> 16));
-				}
-				if(p.out_dtype == AF3_BF16) {
-					u32x2 w = {pack_bf16x2(o0, o1), pack_bf16x2(o2, o3)};
-					*reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.out) + ooff + d0) = w;
-				} else {
-					float4 w = {o0, o1, o2, o3};
-					*reinterpret_cast<float4*>(static_cast<float*>(p.out) + ooff + d0) = w;
-				}
+		if constexpr(FUSED) {  // q and gate of this wavefront's next block
+			if(qb_f - NW >= 0) {
+				u32x4 xf[NS];
+				load_x_frags((qb_f - NW) * 32 + n, xf);
+				project_q_gate(xf);
 			}
+		}
 	}
 }
 
@@ -797,6 +926,22 @@ int64_t mfma_bf16_workspace_bytes(const af3_dpa_params& p) {
 	return ws_bytes_needed(p);
 }
 
+// bias -> fp16(bias * log2 e) in fragment order, into p.workspace
+static int launch_bias_prepass(const af3_dpa_params& p, hipStream_t s) {
+	const bool     bf32      = p.bias_dtype == AF3_F32;
+	const int      n_qblocks = (int)((p.L + 31) / 32), n_ktiles = (int)((p.L + KT - 1) / KT);
+	const int64_t  total     = p.H * n_qblocks * (int64_t)n_ktiles * 256;
+	const unsigned g         = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
+	const bool     vec_ok    = ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) && (p.bias_stride[0] % 8 == 0) && (p.bias_stride[1] % 8 == 0);
+	if(bf32)
+		hipLaunchKernelGGL(bias_prepass_kernel<true>, dim3(g), dim3(256), 0, s, p.bias, static_cast<u32x4*>(p.workspace), p.H, p.L, p.bias_stride[0], p.bias_stride[1], n_qblocks,
+						   n_ktiles, vec_ok);
+	else
+		hipLaunchKernelGGL(bias_prepass_kernel<false>, dim3(g), dim3(256), 0, s, p.bias, static_cast<u32x4*>(p.workspace), p.H, p.L, p.bias_stride[0], p.bias_stride[1], n_qblocks,
+						   n_ktiles, vec_ok);
+	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
 template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT = false>
 static int launch_one(const af3_dpa_params& p, hipStream_t s) {
 	constexpr int QT       = SPLIT ? 32 : NW * 32;
@@ -806,12 +951,77 @@ static int launch_one(const af3_dpa_params& p, hipStream_t s) {
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
 	const size_t smem = (size_t)(SPLIT ? NW : 1) * 6 * KT * DP * 2 + (BMODE == 2 ? NW * 3 * 4096 : 0) + ((size_t)n_ktiles * KT + 64) * 4 + (size_t)n_ktiles * 2 + 16;
-	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BMODE, SPLIT>;
+	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BMODE, SPLIT, false>;
 	if(smem > 64 * 1024) {  // beyond the default dynamic-LDS limit: raise it for this kernel (idempotent, host side)
 		if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
 	}
-	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, n_qtiles, n_groups);
+	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, n_qtiles, n_groups, fused_grid_args{});
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+// ---- fused grid attention: projections + attention + gate in one kernel ----
+constexpr int64_t FUSED_LDS_LIMIT = 160 * 1024;
+static size_t fused_lds_bytes(int64_t L) {
+	const int64_t n_ktiles = (L + KT - 1) / KT;
+	return (size_t)(2 * n_ktiles * KT * 32 * 2 + 2 * 8 * 1024 + (n_ktiles * KT + 64) * 4 + n_ktiles * 2 + 16);
+}
+
+bool grid_fused_eligible(const af3_grid_attention_params& g) {
+	if(g.dtype != AF3_BF16 || g.C != 128 || g.head != 4) return false;  // AlphaFold 3's pair stack: 128 channels, 4 heads of 32
+	if(g.N > MAX_L_MFMA || (int64_t)fused_lds_bytes(g.N) > FUSED_LDS_LIMIT) return false;
+	if(!aligned16(g.pair) || g.pair_stride[0] % 8 || g.pair_stride[1] % 8 || g.pair_stride[1] < g.C) return false;
+	if(g.N * g.pair_stride[1] * 2 >= 0x7fffffffLL) return false;
+	for(const void* w : {g.q_proj, g.k_proj, g.v_proj, g.gating_query})
+		if(!w || (reinterpret_cast<uintptr_t>(w) & 3)) return false;
+	if((reinterpret_cast<uintptr_t>(g.out) & 7) || g.out_stride[0] % 4 || g.out_stride[1] % 4 || g.out_stride[1] < g.C) return false;
+	if(g.bias && g.bias_dtype != AF3_BF16 && g.bias_dtype != AF3_F32) return false;
+	return true;
+}
+
+static af3_dpa_params grid_as_dpa(const af3_grid_attention_params& g) {
+	af3_dpa_params p{};
+	p.B = g.B, p.H = g.head, p.L = g.N, p.D = g.C / g.head;
+	p.bias = g.bias, p.bias_stride[0] = g.bias_stride[0], p.bias_stride[1] = g.bias_stride[1], p.bias_dtype = g.bias_dtype;
+	p.key_mask = g.key_mask, p.key_mask_stride_b = g.key_mask_stride_b;
+	p.out = g.out, p.out_stride[0] = g.out_stride[0], p.out_stride[1] = p.D, p.out_stride[2] = g.out_stride[1];
+	p.io_dtype = p.out_dtype = p.mma_dtype = AF3_BF16;
+	p.softmax_scale = 1.f / sqrtf((float)p.D);
+	p.q_descale = p.k_descale = p.v_descale = 1.f;
+	p.workspace = g.workspace, p.workspace_bytes = g.workspace_bytes;
+	return p;
+}
+
+int64_t grid_fused_workspace_bytes(const af3_grid_attention_params& g) {
+	if(!grid_fused_eligible(g) || !g.bias) return 0;
+	return ws_bytes_needed(grid_as_dpa(g));
+}
+
+template <int NW>
+static int launch_fused_nw(const af3_dpa_params& p, const fused_grid_args& fa, hipStream_t s) {
+	const int64_t n_groups = p.B * p.H;
+	const int64_t blocks   = ((n_groups + 7) / 8) * 8;
+	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
+	const size_t smem = fused_lds_bytes(p.L);
+	auto         kern = dpa_mfma_bf16_kernel<32, NW, true, 0, false, true>;
+	if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
+	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, 1, n_groups, fa);
+	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+int launch_grid_fused(const af3_grid_attention_params& g, hipStream_t s) {
+	af3_dpa_params p = grid_as_dpa(g);
+	if(p.bias) {
+		if(!p.workspace || p.workspace_bytes < ws_bytes_needed(p) || (reinterpret_cast<uintptr_t>(p.workspace) & 15)) return AF3_ERR_BAD_ARGUMENT;
+		const int rc = launch_bias_prepass(p, s);
+		if(rc != AF3_OK) return rc;
+	}
+	fused_grid_args fa{};
+	fa.x = static_cast<const uint16_t*>(g.pair), fa.x_stride_b = g.pair_stride[0], fa.x_stride_n = g.pair_stride[1];
+	fa.wq = g.q_proj, fa.wk = g.k_proj, fa.wv = g.v_proj, fa.wg = g.gating_query;
+	// wavefronts per workgroup: 12 (three per SIMD) unless 8 leaves fewer of them idle in the last round of query blocks
+	const int n_qblocks = (int)((p.L + 31) / 32);
+	const int best      = ((n_qblocks + 7) / 8) * 8 < ((n_qblocks + 11) / 12) * 12 ? 8 : 12;
+	return best == 12 ? launch_fused_nw<12>(p, fa, s) : launch_fused_nw<8>(p, fa, s);
 }
 
 template <int DP, bool L2DOM, int BMODE>
@@ -845,17 +1055,8 @@ int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s) {
 	const bool use_ws = p.bias && p.workspace && mfma_bf16_workspace_bytes(p) > 0 && p.workspace_bytes >= ws_bytes_needed(p) &&
 						(reinterpret_cast<uintptr_t>(p.workspace) & 15) == 0;
 	if(use_ws) {
-		const int      n_qblocks = (int)((p.L + 31) / 32), n_ktiles = (int)((p.L + KT - 1) / KT);
-		const int64_t  total     = p.H * n_qblocks * (int64_t)n_ktiles * 256;
-		const unsigned g         = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
-		const bool     vec_ok    = ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) && (p.bias_stride[0] % 8 == 0) && (p.bias_stride[1] % 8 == 0);
-		if(bf32)
-			hipLaunchKernelGGL(bias_prepass_kernel<true>, dim3(g), dim3(256), 0, s, p.bias, static_cast<u32x4*>(p.workspace), p.H, p.L, p.bias_stride[0], p.bias_stride[1],
-							   n_qblocks, n_ktiles, vec_ok);
-		else
-			hipLaunchKernelGGL(bias_prepass_kernel<false>, dim3(g), dim3(256), 0, s, p.bias, static_cast<u32x4*>(p.workspace), p.H, p.L, p.bias_stride[0], p.bias_stride[1],
-							   n_qblocks, n_ktiles, vec_ok);
-		if(hipGetLastError() != hipSuccess) return AF3_ERR_LAUNCH;
+		const int rc = launch_bias_prepass(p, s);
+		if(rc != AF3_OK) return rc;
 	}
 	const bool l2dom = use_ws || !p.bias;
 	// in-place bf16 bias: through the LDS ring when its rows can be fetched in aligned 16-byte chunks that

@@ -5,7 +5,9 @@
 
 and the module that wraps the first one, GridSelfAttentionCpp (src/af3_kernels/Attention.py:23-82).
 
-On the GPU the op is three launches instead of the reference's per-(row, head) loop nest:
+On the GPU the grid op in AlphaFold 3's shape (bfloat16, 128 channels, 4 heads) is ONE kernel for the projections,
+the attention and the gate (af3_grid_attention_forward: q, k, v and the gate never touch device memory) followed by
+the output projection GEMM.  Every other shape, and the diffusion op, is three launches:
   1. ONE library GEMM for the four projections: x [rows, C] . W [C, 4C], output columns ordered
      (head, [k, v, q, gate], channel)  (hipBLASLt through torch: a plain GEMM is library territory);
   2. the attention kernel, reading q, k, v as strided views of that GEMM's output (no
@@ -15,12 +17,17 @@ On the GPU the op is three launches instead of the reference's per-(row, head) l
 Weights arrive in the layout the reference's callers produce with vnni_repack_tensor(W.T, 2, C/head)
 and are unpacked once per weight set into the fused matrix (cached per live weight tensor and version).
 """
+import ctypes
 import weakref
 from typing import Optional
 
 import torch
 
-from . import ops
+from . import _lib, ops
+
+# One workgroup of the fused kernel serves one (batch row, head) and holds a compute unit's LDS: launches with
+# fewer workgroups than this leave most of the 256 compute units idle and take the three-launch path instead.
+_FUSED_MIN_GROUPS = 128
 
 _W_CACHE = {}
 _W_CACHE_MAX = 64
@@ -108,6 +115,43 @@ def _attend(y: torch.Tensor, B: int, N: int, head: int, mask, bias) -> torch.Ten
     return out
 
 
+def _fused_grid_kernel(pair: torch.Tensor, mask, bias, ws, head: int) -> Optional[torch.Tensor]:
+    """Projections, attention and gate in ONE kernel (af3_grid_attention_forward) when the library supports the
+    shape (bfloat16, 128 channels, 4 heads, K and V of a head fit in LDS); None otherwise.  Returns [B, N, C]."""
+    if ops._exact_bias or any(w.dtype != pair.dtype for w in ws):
+        return None
+    B, N, C = pair.shape
+    if pair.stride(-1) != 1:
+        pair = pair.contiguous()
+    g = _lib.GridAttentionParams()
+    g.pair, g.pair_stride = pair.data_ptr(), (ctypes.c_int64 * 2)(pair.stride(0), pair.stride(1))
+    g.q_proj, g.k_proj, g.v_proj, g.gating_query = (w.data_ptr() for w in ws)
+    g.B, g.N, g.C, g.head = B, N, C, head
+    g.dtype = ops._DTYPE_CODE[pair.dtype]
+    out = torch.empty(B, N, C, dtype=pair.dtype, device=pair.device)
+    g.out, g.out_stride = out.data_ptr(), (ctypes.c_int64 * 2)(N * C, C)
+    if bias is not None:
+        bias = ops._inner_contig(bias)
+        if bias.dtype not in ops._DTYPE_CODE or bias.dim() != 3 or bias.shape[0] != head or bias.shape[1] < N or bias.shape[2] < N:
+            return None
+        g.bias, g.bias_stride, g.bias_dtype = bias.data_ptr(), (ctypes.c_int64 * 2)(bias.stride(0), bias.stride(1)), ops._DTYPE_CODE[bias.dtype]
+    keep = ops._lift_mask(mask, N) if mask is not None else None
+    if keep is not None:
+        if keep.shape[0] not in (1, B):
+            raise ValueError(f"mask must be [N] or [B, N] with B={B}, N={N}, got {tuple(mask.shape)}")
+        g.key_mask, g.key_mask_stride_b = keep.data_ptr(), (0 if keep.shape[0] == 1 else keep.stride(0))
+    lib = _lib.load()
+    if not lib.af3_grid_attention_supported(ctypes.byref(g)):
+        return None
+    ws_bytes = lib.af3_grid_attention_workspace_bytes(ctypes.byref(g))
+    if ws_bytes > 0:
+        scratch = torch.empty(ws_bytes, dtype=torch.uint8, device=pair.device)
+        g.workspace, g.workspace_bytes = scratch.data_ptr(), ws_bytes
+    with ops._on_device(pair.device):
+        _lib.check(lib.af3_grid_attention_forward(ctypes.byref(g), ops._stream_ptr(pair.device)), "af3_grid_attention_forward")
+    return out
+
+
 def _attention_cpp(
     pair: torch.Tensor,
     mask: torch.Tensor,
@@ -136,8 +180,10 @@ def _attention_cpp(
     code = ops._DTYPE_CODE.get(dtype)
     if code not in (ops.AF3_F32, ops.AF3_BF16):
         raise ValueError(f"unsupported dtype {dtype}: float32 or bfloat16")
-    y = _project(pair.reshape(B * N, C), (q_proj, k_proj, v_proj, gating_query), None, head)
-    gated = _attend(y, B, N, head, mask, bias)
+    ws = (q_proj, k_proj, v_proj, gating_query)
+    gated = _fused_grid_kernel(pair, mask, bias, ws, head) if B * head >= _FUSED_MIN_GROUPS else None
+    if gated is None:
+        gated = _attend(_project(pair.reshape(B * N, C), ws, None, head), B, N, head, mask, bias)
     return torch.matmul(gated.view(B * N, C), out_proj.to(dtype)).view(B, N, C)
 
 

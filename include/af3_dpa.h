@@ -195,6 +195,47 @@ int af3_quantize_qkv_fp8_e4m3(const void* q, const void* k, const void* v, int32
 							  float* descales, float* scratch, void* hip_stream);
 
 /*
+ * Grid (triangle) self-attention up to the sigmoid gate, in ONE kernel:
+ *     q, k, v, g = pair . Wq, Wk, Wv, Wgate   (per head, C/head channels each)
+ *     out[b, n, h*K : (h+1)*K] = softmax(q k^T / sqrt(K) + bias[h], key mask)[n, :] . v  *  sigmoid(g[n])
+ * q, k, v and the gate never touch device memory: K and V of a (batch row, head) are projected into LDS once,
+ * q and the gate per block of 32 query rows.
+ * Replaces: _attention_impl<bfloat16> without its closing output projection -- src/csrc/dot_product_attention.cpp:
+ * 200-362 (projections :286-345, logits / bias / mask / softmax :313-333, weighted average :346-352, sigmoid gate
+ * :334-361), bound as `_attention` at src/csrc/init.cpp.  The output projection (:364-371) is a plain [B*N, C] x
+ * [C, C] matrix product on the result and is left to the caller's BLAS.
+ * Supported (af3_grid_attention_supported() == 1): dtype AF3_BF16, C == 128, head == 4, N small enough for K and V
+ * of one head to stay in LDS (N <= 1024); anything else returns AF3_ERR_BAD_ARGUMENT and the caller composes the
+ * op from a projection product and af3_dpa_forward with its `gate` argument.
+ */
+typedef struct af3_grid_attention_params {
+	const void* pair;            /* [B, N, C] normalised pair rows, innermost stride 1 */
+	int64_t     pair_stride[2];  /* elements: batch row, token */
+	/* weight^T of the four projections in the layout the reference's callers produce with
+	 * vnni_repack_tensor(W.T, 2, C/head): [head][C/2][C/head][2] (src/af3_kernels/Attention.py:59-62) */
+	const void* q_proj;
+	const void* k_proj;
+	const void* v_proj;
+	const void* gating_query;
+	const void* bias;            /* [head, N, N] (or NULL), AF3_BF16 or AF3_F32 */
+	int64_t     bias_stride[2];  /* elements: head, query row */
+	int32_t     bias_dtype;
+	int32_t     dtype;           /* of pair, the weights and out */
+	const uint8_t* key_mask;     /* [B, N] or [N] bytes, non-zero = attend; NULL = all */
+	int64_t     key_mask_stride_b; /* 0 broadcasts one mask row over the batch */
+	void*       out;             /* [B, N, C], innermost stride 1 */
+	int64_t     out_stride[2];
+	int64_t     B, N, C, head;
+	void*       workspace;       /* af3_grid_attention_workspace_bytes() bytes, 256-byte aligned; required when bias != NULL */
+	int64_t     workspace_bytes;
+} af3_grid_attention_params;
+
+int     af3_grid_attention_forward(const af3_grid_attention_params* params, void* hip_stream);
+int64_t af3_grid_attention_workspace_bytes(const af3_grid_attention_params* params);
+/* 1 when af3_grid_attention_forward handles these arguments, 0 when the caller must compose the op. Host only. */
+int     af3_grid_attention_supported(const af3_grid_attention_params* params);
+
+/*
  * N-dimensional pad (ndim <= AF3_PAD_MAX_DIMS): copy src (shape src_shape, element strides
  * src_strides) into the low corner of a contiguous dst of shape dst_shape (>= src_shape in
  * every axis) and fill the rest with the 32-bit pattern `fill_bits` truncated to elem_size

@@ -19,7 +19,7 @@ def test_host_program_links_the_library_and_lists_its_cases():
     r = subprocess.run([BIN, "--list"], capture_output=True, text=True, timeout=60)
     assert r.returncode == 0, r.stderr
     lines = r.stdout.strip().splitlines()
-    assert lines[0] == "abi version 2" and len(lines) >= 5
+    assert lines[0] == "abi version 3" and len(lines) >= 5
 
 
 @pytest.mark.gpu

@@ -79,17 +79,72 @@ GRID_CASES = [
 
 @pytest.mark.parametrize("B,N,C,head,dtype", GRID_CASES)
 def test_attention_cpp_matches_formula(af3, oracle, B, N, C, head, dtype):
-    x, mask, bias, wq, wk, wv, wg, wo, _ = make(B, N, C, head, dtype, seed=B * 1000 + N, with_out=True, with_qbias=False)
-    print(f"_attention_cpp B,N,C,head={B, N, C, head} {dtype}", flush=True)
+    run_grid_case(af3, oracle, B, N, C, head, dtype, one_kernel=False)
+
+
+def run_grid_case(af3, oracle, B, N, C, head, dtype, one_kernel, mask_p=0.85, bias_dtype=None):
+    """one_kernel: route through af3_grid_attention_forward (projections + attention + gate in one kernel) whatever the
+    batch size, and check that it was really taken; otherwise force the three-launch composition."""
+    from af3_kernels_amd import fused
+    x, mask, bias, wq, wk, wv, wg, wo, _ = make(B, N, C, head, dtype, seed=B * 1000 + N, with_out=True, with_qbias=False, mask_p=mask_p)
+    if bias_dtype is not None:
+        bias = bias.to(bias_dtype)
+    print(f"_attention_cpp B,N,C,head={B, N, C, head} {dtype} one_kernel={one_kernel}", flush=True)
     d = lambda t: t.cuda()
-    out = af3._attention_cpp(d(x), d(mask), d(bias), pack(af3, d(wq), head), pack(af3, d(wk), head), pack(af3, d(wv), head),
-                             pack(af3, d(wg), head), d(wo), head, False, 128 if N > 256 else 64, 0)
-    torch.cuda.synchronize()
+    taken = []
+    real, saved_min = fused._fused_grid_kernel, fused._FUSED_MIN_GROUPS
+
+    def spy(*a, **k):
+        r = real(*a, **k)
+        taken.append(r is not None)
+        return r
+
+    fused._fused_grid_kernel, fused._FUSED_MIN_GROUPS = spy, (1 if one_kernel else 1 << 60)
+    try:
+        out = af3._attention_cpp(d(x), d(mask), d(bias), pack(af3, d(wq), head), pack(af3, d(wk), head), pack(af3, d(wv), head),
+                                 pack(af3, d(wg), head), d(wo), head, False, 128 if N > 256 else 64, 0)
+        torch.cuda.synchronize()
+    finally:
+        fused._fused_grid_kernel, fused._FUSED_MIN_GROUPS = real, saved_min
+    assert taken == ([True] if one_kernel else [])
     assert out.shape == x.shape and out.dtype == dtype and out.is_cuda
-    args = [f32np(t) if t is not None and t.dtype != torch.bool else (t.numpy() if t is not None else None) for t in (x, mask, bias, wq, wk, wv, wg, wo)]
+    args = [f32np(t) if t.dtype != torch.bool else t.numpy() for t in (x, mask, bias, wq, wk, wv, wg, wo)]
     want = oracle.fused_attention_formula(*args, None, head=head)
     ref = oracle.fused_attention_reference(*args, None, head=head, dtype=oracle.BF16, BLK_SZ=64) if dtype == torch.bfloat16 else None
     check(out, want, ref, dtype)
+    return out
+
+
+ONE_KERNEL_CASES = [
+    # B, N: 128 channels, 4 heads, bfloat16
+    (4, 72), (9, 200), (3, 37), (2, 384), (1, 768), (5, 64), (2, 1000), (3, 33), (2, 1),
+]
+
+
+@pytest.mark.parametrize("B,N", ONE_KERNEL_CASES)
+def test_grid_attention_one_kernel_matches_formula(af3, oracle, B, N):
+    run_grid_case(af3, oracle, B, N, 128, 4, torch.bfloat16, one_kernel=True)
+
+
+def test_grid_attention_one_kernel_variants(af3, oracle):
+    """fp32 bias, mostly and fully dropped keys, a strided (transposed) pair view, and agreement with the three-launch path."""
+    run_grid_case(af3, oracle, 4, 100, 128, 4, torch.bfloat16, one_kernel=True, bias_dtype=torch.float32)
+    run_grid_case(af3, oracle, 3, 200, 128, 4, torch.bfloat16, one_kernel=True, mask_p=0.05)
+    a = run_grid_case(af3, oracle, 6, 150, 128, 4, torch.bfloat16, one_kernel=True)
+    b = run_grid_case(af3, oracle, 6, 150, 128, 4, torch.bfloat16, one_kernel=False)
+    assert float((a.float() - b.float()).abs().max()) <= 3e-2
+    from af3_kernels_amd import fused
+    N, head = 96, 4
+    x, mask, bias, wq, wk, wv, wg, wo, _ = make(N, N, 128, head, torch.bfloat16, 5, True, False)
+    d = lambda t: t.cuda()
+    packed = [pack(af3, d(w), head) for w in (wq, wk, wv, wg)]
+    xt = d(x).transpose(0, 1)                                  # [N, N, C] view with swapped leading strides
+    none = torch.zeros(N, N, dtype=torch.bool)
+    none[::2] = mask[::2]                                      # every other batch row has no live key at all
+    got = fused._fused_grid_kernel(xt, d(none), d(bias), packed, head)
+    assert got is not None
+    want = oracle.fused_attention_formula(f32np(x.transpose(0, 1)), none.numpy(), f32np(bias), f32np(wq), f32np(wk), f32np(wv), f32np(wg), None, None, head=head)
+    check(got, want, None, torch.bfloat16)
 
 
 SELF_CASES = [

@@ -208,8 +208,11 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	const int64_t slot  = wg >> 3;
 	const int64_t group = (slot / n_qtiles) * 8 + xcd;
 	const int     qtile = (int)(slot % n_qtiles);
-	if(group >= n_groups) return;
-	const int64_t b = group / p.H, h = group % p.H;
+	if(!FUSED && group >= n_groups) return;
+	// FUSED (4 heads): an XCD serves two heads -- their bias (2.4 MB) stays in its 4 MB L2 -- and the two
+	// workgroups that read the same rows x[b] through that L2 are neighbours in dispatch order.
+	const int64_t b = FUSED ? (slot >> 1) * 4 + (xcd >> 1) : group / p.H, h = FUSED ? 2 * (xcd & 1) + (slot & 1) : group % p.H;
+	if(FUSED && b >= p.B) return;
 
 	const int     tid = threadIdx.x, lane = tid & 63;
 	const int     wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -999,7 +1002,7 @@ int64_t grid_fused_workspace_bytes(const af3_grid_attention_params& g) {
 template <int NW>
 static int launch_fused_nw(const af3_dpa_params& p, const fused_grid_args& fa, hipStream_t s) {
 	const int64_t n_groups = p.B * p.H;
-	const int64_t blocks   = ((n_groups + 7) / 8) * 8;
+	const int64_t blocks   = 16 * ((p.B + 3) / 4);  // see the kernel's workgroup -> (batch row, head) map
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
 	const size_t smem = fused_lds_bytes(p.L);
 	auto         kern = dpa_mfma_bf16_kernel<32, NW, true, 0, false, true>;

@@ -92,3 +92,77 @@ def make_inputs(case, device="cpu", batch=None):
         mask = mask[:B]
     q, k, v, bias = [t.to(dt).to(device) for t in (q, k, v, bias)]
     return q, k, v, mask.to(device), bias
+
+
+# ------------------------------------------------------------------------------------------
+# the fused callers of the attention core (shapes of examples/grid_self_attention.py:141-167 and
+# examples/self_attention.py: pair [N, N, 128] with 4 heads; tokens [N, 768] with 16 heads)
+# ------------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class FusedCase:
+    name: str
+    kind: str              # "grid" (_attention_cpp) | "self" (self_attention_cpp)
+    B: int                 # batch rows (grid: = N; self: 1)
+    N: int
+    C: int
+    head: int
+    keep: float = 0.92     # Bernoulli key mask
+    seed: int = 0
+
+    @property
+    def flops_projections(self) -> float:
+        return 2.0 * self.B * self.N * self.C * 4 * self.C
+
+    @property
+    def flops_attention(self) -> float:
+        return 4.0 * self.B * self.N * self.N * self.C
+
+    @property
+    def flops_out_projection(self) -> float:
+        return 2.0 * self.B * self.N * self.C * self.C if self.kind == "grid" else 0.0
+
+    @property
+    def flops(self) -> float:
+        return self.flops_projections + self.flops_attention + self.flops_out_projection
+
+    @property
+    def bytes(self) -> float:
+        """Algorithmic bytes of the whole op: rows in, rows out, bias, mask, weights (bf16)."""
+        return 2.0 * (2 * self.B * self.N * self.C + self.head * self.N * self.N + 5 * self.C * self.C) + self.B * self.N
+
+
+FUSED_CASES = {
+    "grid_n384": FusedCase("grid_n384", "grid", 384, 384, 128, 4),
+    "grid_n768": FusedCase("grid_n768", "grid", 768, 768, 128, 4),
+    "self_n1536": FusedCase("self_n1536", "self", 1, 1536, 768, 16),
+}
+
+
+def make_fused_inputs(case, device="cpu", batch=None):
+    """Returns dict(x, mask, bias, wq, wk, wv, wg, wo, q_bias) of bfloat16 tensors; the weights are weight^T in
+    natural [C_in, C_out] layout, scaled by C^-1/2 so that projected rows have unit scale.  `batch` truncates the
+    batch axis of a grid case."""
+    if isinstance(case, str):
+        case = FUSED_CASES[case]
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(case.seed)
+    B = case.B if batch is None else min(batch, case.B)
+    dt = torch.bfloat16
+    draw = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
+    ws = [(draw(case.C, case.C) * case.C ** -0.5).to(dt).to(device) for _ in range(5)]
+    bias = draw(case.head, case.N, case.N).to(dt).to(device)
+    q_bias = draw(case.C).to(dt).to(device)
+    mgen = torch.Generator(device="cpu")
+    mgen.manual_seed(case.seed + 1)
+    if case.kind == "grid":
+        mask = torch.rand(case.B, case.N, generator=mgen) < case.keep
+        mask[:, 0] = True
+        mask = mask[:B]
+        # (rows are drawn per batch row so that a truncated sample sees the same leading rows)
+        x = torch.stack([draw(case.N, case.C) for _ in range(B)]).to(dt).to(device)
+    else:
+        mask = torch.rand(case.N, generator=mgen) < case.keep
+        mask[0] = True
+        x = draw(case.N, case.C).to(dt).to(device)
+    return dict(x=x, mask=mask.to(device), bias=bias, wq=ws[0], wk=ws[1], wv=ws[2], wg=ws[3], wo=ws[4] if case.kind == "grid" else None,
+                q_bias=q_bias if case.kind == "self" else None)

@@ -1,6 +1,7 @@
 """Benchmark of the biased dot-product-attention hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--case cfg4] [--no-cpu-baseline]
+    python bench.py --case grid_n768      (the fused grid self-attention caller; also grid_n384, self_n1536)
 
 A step is one call of dot_product_attention_cpp (the drop-in for the reference's
 af3_kernels.dot_product_attention_cpp) on synthetic inputs already resident in HBM.  The default
@@ -91,6 +92,94 @@ def cpu_baseline(case, budget_s=12.0):
             "ms_full_workload_extrapolated": round(t / batch * case.B * 1e3, 1)}
 
 
+def bench_fused(args, case):
+    """--case grid_n384 | grid_n768 | self_n1536: a step is one call of _attention_cpp / self_attention_cpp (the drop-ins
+    for the reference's fused callers of the attention core) on synthetic rows already resident in HBM."""
+    import torch
+    import af3_kernels_amd as af3
+    from af3_kernels_amd import fused
+    from af3_kernels_amd.synthetic import make_fused_inputs
+    af3._lib.load()
+    dev = torch.device("cuda:0")
+    t = make_fused_inputs(case, device=dev)
+    K = case.C // case.head
+    pk = [af3.vnni_repack_tensor(t[k].contiguous(), 2, K) for k in ("wq", "wk", "wv", "wg")]
+    if case.kind == "grid":
+        fn = lambda: af3._attention_cpp(t["x"], t["mask"], t["bias"], *pk, t["wo"], case.head)
+        one_kernel = fused._fused_grid_kernel(t["x"], t["mask"], t["bias"], pk, case.head) is not None
+        core = (lambda: fused._fused_grid_kernel(t["x"], t["mask"], t["bias"], pk, case.head)) if one_kernel else None
+    else:
+        fn = lambda: af3.self_attention_cpp(t["x"], t["mask"], t["bias"], pk[0], t["q_bias"], pk[1], pk[2], pk[3], case.head)
+        one_kernel, core = False, None
+    for _ in range(args.warmup):
+        out = fn()
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream(dev)
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record(stream)
+    for _ in range(args.steps):
+        out = fn()
+    e.record(stream)
+    torch.cuda.synchronize()
+    ms_per_step = s.elapsed_time(e) / args.steps
+    assert torch.isfinite(out).all()
+    roofline = None
+    if core is not None:   # the dominant kernel on its own, per launch (HIP events on the stream it is launched on)
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for a, b in evs:
+            a.record(stream)
+            core()
+            b.record(stream)
+        torch.cuda.synchronize()
+        per = sorted(a.elapsed_time(b) for a, b in evs)
+        kernel_ms = sum(per) / len(per)
+        kflops = case.flops_projections + case.flops_attention
+        ach = kflops / (kernel_ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS["bf16"], 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES.get(case.name), "kernel": "grid attention, one kernel (bias prepass + projections + attention + gate)",
+                    "kernel_ms_avg": round(kernel_ms, 4), "kernel_ms_median": round(per[len(per) // 2], 4), "algorithmic_flops_per_launch": kflops,
+                    "algorithmic_bytes_per_launch": case.bytes}
+    tflops = case.flops / (ms_per_step * 1e-3) / 1e12
+    line = {"metric": f"fused {case.kind} self-attention TFLOP/s ({case.name})", "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+            "data": "synthetic",
+            "config": {"workload": f"{case.name}: rows [{case.B}, {case.N}, {case.C}] head={case.head} bf16, Bernoulli({case.keep}) key mask; "
+                                   f"{'one kernel + output projection GEMM' if one_kernel else 'projection GEMM + attention kernel' + (' + output projection GEMM' if case.kind == 'grid' else '')}",
+                       "flops": case.flops},
+            "roofline": roofline}
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline_fused(case)
+    print(json.dumps(line))
+
+
+def cpu_baseline_fused(case, budget_s=12.0):
+    """The CPU restatement of _attention_impl / self_attention_impl (oracle/af3_oracle.c, OpenMP over batch row x head like
+    src/csrc/dot_product_attention.cpp:276-277, :452) in bfloat16, timed on a bounded sample of the batch rows."""
+    from af3_kernels_amd.synthetic import make_fused_inputs
+    from oracle import af3_oracle
+    threads = int(os.environ.get("OMP_NUM_THREADS", len(os.sched_getaffinity(0))))
+    per_row = case.flops / case.B
+
+    def run(nb):
+        t = make_fused_inputs(case, batch=nb)
+        f = lambda k: None if t[k] is None else t[k].float().numpy()
+        args = (f("x"), t["mask"].numpy(), f("bias"), f("wq"), f("wk"), f("wv"), f("wg"), f("wo"), f("q_bias"))
+        af3_oracle.fused_attention_reference(*args, head=case.head, dtype=af3_oracle.BF16, BLK_SZ=128)   # warm-up
+        t0 = time.time()
+        af3_oracle.fused_attention_reference(*args, head=case.head, dtype=af3_oracle.BF16, BLK_SZ=128)
+        return time.time() - t0
+
+    batch = min(case.B, threads)
+    t = run(batch)
+    target = int(min(case.B, max(batch, batch * budget_s / max(t, 1e-3))))
+    if target > batch:
+        batch = target
+        t = run(batch)
+    return {"value": round(per_row * batch / t / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{batch} of {case.B} batch rows of {case.name} (same N, C, heads, bias), {t:.2f} s wall, OpenMP restatement of the reference's fused loop nest in bf16",
+            "ms_full_workload_extrapolated": round(t / batch * case.B * 1e3, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -107,8 +196,10 @@ def main():
 
     import torch
     import af3_kernels_amd as af3
-    from af3_kernels_amd.synthetic import CASES, make_inputs
+    from af3_kernels_amd.synthetic import CASES, FUSED_CASES, make_inputs
     af3._lib.load()
+    if args.case in FUSED_CASES:
+        return bench_fused(args, FUSED_CASES[args.case])
     case = CASES[args.case]
     dev = torch.device("cuda:0")
     q, k, v, mask, bias = make_inputs(case, device=dev)

@@ -18,6 +18,9 @@
 #include "af3_dpa.h"
 
 extern "C" int      af3o_dpa_formula(const float* q, const float* k, const float* v, const float* bias, const uint8_t* keep, float* out, int64_t B, int64_t H, int64_t L, int64_t D);
+extern "C" int      af3o_fused_attention_formula(const float* x, const uint8_t* keep, const float* bias, const float* wq, const float* wk, const float* wv, const float* wg,
+                                                 const float* wo, const float* qbias, float* out, int64_t B, int64_t L, int64_t C, int64_t H);
+extern "C" int      af3o_vnni_repack(const uint16_t* in, uint16_t* out, int64_t M, int64_t N, int64_t blk);
 extern "C" uint16_t af3o_f32_to_bf16_bits(float f);
 extern "C" float    af3o_bf16_bits_to_f32(uint16_t h);
 
@@ -147,12 +150,93 @@ int run(const Case& c, hipStream_t stream) {
 	return ok ? 0 : 1;
 }
 
+// Grid self-attention up to the gate (af3_grid_attention_forward) on B batch rows of N tokens, 128 channels, 4 heads:
+// weights handed over in the reference's VNNI panel layout, result against the fp64 formula without output projection.
+int run_grid(int64_t B, int64_t N, hipStream_t stream) {
+	const int64_t C = 128, H = 4;
+	Rng           rng{0x9e1d0000ull + (uint64_t)N};
+	auto          bf = [](float f) { return af3o_bf16_bits_to_f32(af3o_f32_to_bf16_bits(f)); };
+	std::vector<float> x(B * N * C), bias(H * N * N), w[4], want(B * N * C);
+	for(auto& v : x) v = bf(rng.n());
+	for(auto& v : bias) v = bf(rng.n());
+	for(auto& m : w) {
+		m.resize(C * C);
+		for(auto& v : m) v = bf(rng.n() / std::sqrt((float)C));
+	}
+	std::vector<uint8_t> keep(B * N, 1);
+	for(int64_t j = N - N / 5; j < N; j++) keep[(B - 1) * N + j] = 0;
+	if(af3o_fused_attention_formula(x.data(), keep.data(), bias.data(), w[0].data(), w[1].data(), w[2].data(), w[3].data(), nullptr, nullptr, want.data(), B, N, C, H) != 0) return 2;
+
+	auto to_bits = [](const std::vector<float>& src) {
+		std::vector<uint16_t> dst(src.size());
+		for(size_t i = 0; i < src.size(); i++) dst[i] = af3o_f32_to_bf16_bits(src[i]);
+		return dst;
+	};
+	const std::vector<uint16_t> hx = to_bits(x), hb = to_bits(bias);
+	std::vector<uint16_t>       hw[4], ho(B * N * C);
+	for(int i = 0; i < 4; i++) {
+		const std::vector<uint16_t> nat = to_bits(w[i]);
+		hw[i].resize(C * C);
+		if(af3o_vnni_repack(nat.data(), hw[i].data(), C, C, C / H) != 0) return 2;
+	}
+	void *dx, *db, *dm, *dout, *dw[4], *dws = nullptr;
+	HIP_OK(hipMalloc(&dx, hx.size() * 2));
+	HIP_OK(hipMalloc(&db, hb.size() * 2));
+	HIP_OK(hipMalloc(&dm, keep.size()));
+	HIP_OK(hipMalloc(&dout, ho.size() * 2));
+	HIP_OK(hipMemcpy(dx, hx.data(), hx.size() * 2, hipMemcpyHostToDevice));
+	HIP_OK(hipMemcpy(db, hb.data(), hb.size() * 2, hipMemcpyHostToDevice));
+	HIP_OK(hipMemcpy(dm, keep.data(), keep.size(), hipMemcpyHostToDevice));
+	for(int i = 0; i < 4; i++) {
+		HIP_OK(hipMalloc(&dw[i], C * C * 2));
+		HIP_OK(hipMemcpy(dw[i], hw[i].data(), C * C * 2, hipMemcpyHostToDevice));
+	}
+	af3_grid_attention_params g;
+	std::memset(&g, 0, sizeof g);
+	g.pair = dx, g.pair_stride[0] = N * C, g.pair_stride[1] = C;
+	g.q_proj = dw[0], g.k_proj = dw[1], g.v_proj = dw[2], g.gating_query = dw[3];
+	g.bias = db, g.bias_stride[0] = N * N, g.bias_stride[1] = N, g.bias_dtype = AF3_BF16;
+	g.key_mask = static_cast<const uint8_t*>(dm), g.key_mask_stride_b = N;
+	g.out = dout, g.out_stride[0] = N * C, g.out_stride[1] = C;
+	g.B = B, g.N = N, g.C = C, g.head = H, g.dtype = AF3_BF16;
+	if(!af3_grid_attention_supported(&g)) {
+		std::fprintf(stderr, "af3_grid_attention_supported: 0 for B=%lld N=%lld\n", (long long)B, (long long)N);
+		return 1;
+	}
+	const int64_t ws = af3_grid_attention_workspace_bytes(&g);
+	HIP_OK(hipMalloc(&dws, (size_t)ws));
+	g.workspace = dws, g.workspace_bytes = ws;
+	const int rc = af3_grid_attention_forward(&g, stream);
+	if(rc != AF3_OK) {
+		std::fprintf(stderr, "af3_grid_attention_forward: %s\n", af3_status_string(rc));
+		return 1;
+	}
+	HIP_OK(hipStreamSynchronize(stream));
+	HIP_OK(hipMemcpy(ho.data(), dout, ho.size() * 2, hipMemcpyDeviceToHost));
+	double err = 0.0, top = 1.0;
+	bool   finite = true;
+	for(size_t i = 0; i < ho.size(); i++) {
+		const float gv = af3o_bf16_bits_to_f32(ho[i]);
+		finite = finite && std::isfinite(gv);
+		err    = std::fmax(err, std::fabs((double)gv - (double)want[i]));
+		top    = std::fmax(top, std::fabs((double)want[i]));
+	}
+	for(void* ptr : {dx, db, dm, dout, dw[0], dw[1], dw[2], dw[3], dws}) HIP_OK(hipFree(ptr));
+	const double tol = 3e-2 * top;  // q, k, v and the gate are rounded to bf16 inside the op, like the reference's
+	const bool   ok  = finite && err <= tol;
+	std::printf("grid attention one kernel %lldx%lldx128, 4 heads  workspace=%lld B  max_abs_err=%.3e (tol %.1e)  %s\n", (long long)B, (long long)N, (long long)ws, err, tol,
+				ok ? "ok" : "FAIL");
+	std::fflush(stdout);
+	return ok ? 0 : 1;
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
 	if(argc > 1 && std::strcmp(argv[1], "--list") == 0) {
 		std::printf("abi version %d\n", af3_abi_version());
 		for(const Case& c : CASES) std::printf("%s\n", c.name);
+		std::printf("grid attention one kernel 3x100x128, 3x256x128\n");
 		return 0;
 	}
 	HIP_OK(hipSetDevice(0));
@@ -161,6 +245,11 @@ int main(int argc, char** argv) {
 	int bad = 0;
 	for(const Case& c : CASES) {
 		const int r = run(c, stream);
+		if(r == 2) return 2;
+		bad += r;
+	}
+	for(const int64_t n : {int64_t{100}, int64_t{256}}) {
+		const int r = run_grid(3, n, stream);
 		if(r == 2) return 2;
 		bad += r;
 	}

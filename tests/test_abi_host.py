@@ -29,4 +29,4 @@ def test_c_callers_get_the_formula_through_the_abi_alone():
     r = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr, flush=True)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count(" ok") >= 5 and "FAIL" not in r.stdout
+    assert r.stdout.count(" ok") >= 7 and "FAIL" not in r.stdout

@@ -175,3 +175,94 @@ def test_mask_lifting_follows_the_reference_wrapper():
     m4 = torch.ones(3, 1, 1, 4, dtype=torch.bool)
     assert _lift_mask(m4, 4).shape == (3, 4)
     assert _lift_mask(m1, 4).data_ptr() == m1.data_ptr()                 # bool masks are reinterpreted, not copied
+
+
+def test_struct_mirrors_match_what_a_c_compiler_lays_out(tmp_path):
+    """sizeof / offsetof of both parameter structs as gcc sees include/af3_dpa.h, against the ctypes mirrors."""
+    import shutil
+    import subprocess
+    from af3_kernels_amd._lib import DpaParams, GridAttentionParams
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    fields = {"af3_dpa_params": (DpaParams, ["q", "B", "q_stride", "bias_stride", "io_dtype", "softmax_scale", "force_generic", "device_descales", "workspace", "q_lo", "gate", "gate_stride"]),
+              "af3_grid_attention_params": (GridAttentionParams, ["pair", "pair_stride", "q_proj", "gating_query", "bias", "bias_stride", "bias_dtype", "dtype", "key_mask", "key_mask_stride_b",
+                                                                 "out", "out_stride", "B", "head", "workspace", "workspace_bytes"])}
+    lines = ["#include <stdio.h>", "#include <stddef.h>", '#include "af3_dpa.h"', "int main(void) {"]
+    for sname, (_, names) in fields.items():
+        lines.append(f'printf("{sname} %zu\\n", sizeof({sname}));')
+        lines += [f'printf("{sname}.{n} %zu\\n", offsetof({sname}, {n}));' for n in names]
+    lines += ["return 0; }"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    got = dict(l.split() for l in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    for sname, (cls, names) in fields.items():
+        assert int(got[sname]) == ctypes.sizeof(cls)
+        for n in names:
+            assert int(got[f"{sname}.{n}"]) == getattr(cls, n).offset, (sname, n)
+
+
+def _grid_params(**kw):
+    from af3_kernels_amd._lib import GridAttentionParams, AF3_BF16
+    g = GridAttentionParams()
+    B, N, C = 64, 256, 128
+    g.pair = g.out = g.q_proj = g.k_proj = g.v_proj = g.gating_query = 0x1000   # never dereferenced on the host
+    g.pair_stride = g.out_stride = (ctypes.c_int64 * 2)(N * C, C)
+    g.B, g.N, g.C, g.head = B, N, C, 4
+    g.dtype = g.bias_dtype = AF3_BF16
+    for k, v in kw.items():
+        setattr(g, k, v)
+    return g
+
+
+def test_grid_attention_entry_points_validate_on_the_host():
+    from af3_kernels_amd import _lib
+    lib = _lib.load()
+    sup, ws, fwd = lib.af3_grid_attention_supported, lib.af3_grid_attention_workspace_bytes, lib.af3_grid_attention_forward
+    assert sup(ctypes.byref(_grid_params())) == 1
+    assert ws(ctypes.byref(_grid_params())) == 0                                       # no bias, no workspace
+    nb = (ctypes.c_int64 * 2)(256 * 256, 256)
+    assert ws(ctypes.byref(_grid_params(bias=0x1000, bias_stride=nb))) == 4 * 8 * 4 * 4096   # heads x query blocks x key tiles x 4 KB
+    assert sup(ctypes.byref(_grid_params(C=256))) == 0 and sup(ctypes.byref(_grid_params(head=8))) == 0
+    assert sup(ctypes.byref(_grid_params(dtype=0))) == 0                               # float32 rows: composed by the caller
+    assert sup(ctypes.byref(_grid_params(N=1100, pair_stride=(ctypes.c_int64 * 2)(1100 * 128, 128), out_stride=(ctypes.c_int64 * 2)(1100 * 128, 128)))) == 0   # K and V no longer fit in LDS
+    assert sup(ctypes.byref(_grid_params(pair=0x1004))) == 0                           # rows not 16-byte aligned
+    assert fwd(None, None) == -1
+    assert fwd(ctypes.byref(_grid_params(q_proj=None)), None) == -1
+    assert fwd(ctypes.byref(_grid_params(N=0)), None) == -3
+    assert fwd(ctypes.byref(_grid_params(head=3)), None) == -3                         # 128 channels do not split into 3 heads
+    assert fwd(ctypes.byref(_grid_params(pair_stride=(ctypes.c_int64 * 2)(256 * 128, 64))), None) == -4
+    assert fwd(ctypes.byref(_grid_params(C=256, pair_stride=(ctypes.c_int64 * 2)(256 * 256, 256), out_stride=(ctypes.c_int64 * 2)(256 * 256, 256))), None) == -7   # valid but unsupported
+    assert fwd(ctypes.byref(_grid_params(bias=0x1000, bias_stride=nb)), None) == -7    # a bias needs the workspace
+
+
+def test_fused_wrappers_match_the_reference_signatures():
+    import inspect
+    import af3_kernels_amd as af3
+    sig = inspect.signature(af3._attention_cpp)
+    assert list(sig.parameters) == ["pair", "mask", "bias", "q_proj", "k_proj", "v_proj", "gating_query", "out_proj", "head", "use_flash_attention", "BLK_SZ", "FLASH_SZ"]
+    assert [sig.parameters[n].default for n in ("use_flash_attention", "BLK_SZ", "FLASH_SZ")] == [False, 128, 1024]
+    sig = inspect.signature(af3.self_attention_cpp)
+    assert list(sig.parameters) == ["pair", "mask", "bias", "q_proj", "q_bias", "k_proj", "v_proj", "gating_query", "head", "use_flash_attention", "BLK_SZ", "FLASH_SZ"]
+    mod = af3.GridSelfAttentionCpp(64, 2, transpose=True)
+    assert sorted(dict(mod.named_parameters())) == sorted(
+        ["act_norm.weight", "act_norm.bias", "pair_bias_projection.weight", "q_projection.weight", "k_projection.weight", "v_projection.weight",
+         "gating_query.weight", "output_projection.weight"])
+    x = torch.randn(2, 8, 64)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        af3._attention_cpp(x, torch.ones(2, 8, dtype=torch.bool), torch.zeros(2, 8, 8), *([torch.zeros(64, 64)] * 5), 2)
+
+
+def test_weight_unpacking_inverts_the_panel_layout(oracle):
+    """fused._unpack_panels undoes vnni_repack_tensor(W_t, 2, K) (checked against the oracle's repack) and the float32 panels."""
+    from af3_kernels_amd import fused
+    C, head = 64, 4
+    K = C // head
+    g = torch.Generator().manual_seed(2)
+    w = torch.randn(C, C, generator=g).to(torch.bfloat16)
+    packed = torch.from_numpy(oracle.vnni_repack(w.view(torch.int16).numpy().view(np.uint16), K).view(np.int16)).view(torch.bfloat16)
+    assert torch.equal(fused._unpack_panels(packed, head), w)
+    wf = torch.randn(C, C, generator=g)
+    panels = wf.view(C, head, K).permute(1, 0, 2).contiguous().view(C, C)
+    assert torch.equal(fused._unpack_panels(panels, head), wf)

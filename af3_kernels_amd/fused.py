@@ -218,9 +218,31 @@ def self_attention_cpp(
     return _attend(y, 1, N, head, mask, bias).view(N, C)
 
 
+def layernorm_pair_bias(pair: torch.Tensor, ln_weight: torch.Tensor, ln_bias: torch.Tensor, eps: float, proj_weight: torch.Tensor):
+    """act_norm + pair_bias_projection + permute(2, 0, 1) of the reference module (src/af3_kernels/Attention.py:51-52) in
+    one pass over the pair tensor: returns (normed [N1, N2, C], bias [head, N1, N2]).  One HIP kernel for bfloat16 pairs
+    with 128 channels and 4 heads; the same torch ops as the reference otherwise."""
+    ops._require_device(pair, ln_weight, ln_bias, proj_weight)
+    head, C = proj_weight.shape
+    if not (pair.dtype == torch.bfloat16 and pair.dim() == 3 and C == 128 and head == 4 and pair.shape[-1] == C and pair.numel() > 0
+            and ln_weight.dtype == ln_bias.dtype == proj_weight.dtype == torch.bfloat16 and pair.stride(2) == 1 and pair.stride(0) % 8 == 0
+            and pair.stride(1) % 8 == 0 and pair.data_ptr() % 16 == 0):
+        normed = torch.nn.functional.layer_norm(pair, (C,), ln_weight, ln_bias, eps)
+        return normed, torch.nn.functional.linear(normed, proj_weight).permute(2, 0, 1)
+    n_i, n_j = pair.shape[:2]
+    normed = torch.empty(n_i, n_j, C, dtype=pair.dtype, device=pair.device)
+    bias = torch.empty(head, n_i, n_j, dtype=pair.dtype, device=pair.device)
+    arr = ctypes.c_int64 * 2
+    with ops._on_device(pair.device):
+        _lib.check(_lib.load().af3_layernorm_pair_bias(pair.data_ptr(), arr(pair.stride(0), pair.stride(1)), ln_weight.contiguous().data_ptr(), ln_bias.contiguous().data_ptr(),
+                                                       float(eps), proj_weight.contiguous().data_ptr(), normed.data_ptr(), bias.data_ptr(), arr(n_i * n_j, n_j), n_i, n_j, C, head,
+                                                       ops._DTYPE_CODE[pair.dtype], ops._stream_ptr(pair.device)), "af3_layernorm_pair_bias")
+    return normed, bias
+
+
 class GridSelfAttentionCpp(torch.nn.Module):
     """Same constructor, parameters and forward as the reference module (src/af3_kernels/Attention.py:23-82):
-    LayerNorm and the pair-bias projection stay torch ops, the rest is _attention_cpp."""
+    LayerNorm and the pair-bias projection are one kernel (layernorm_pair_bias), the rest is _attention_cpp."""
 
     def __init__(self, c_pair: int = 128, num_head: int = 4, transpose: bool = False):
         super().__init__()
@@ -255,8 +277,7 @@ class GridSelfAttentionCpp(torch.nn.Module):
         return self.q_proj, self.k_proj, self.v_proj, self.gq, self.out_proj
 
     def forward(self, pair: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
-        normed = self.act_norm(pair)
-        bias = self.pair_bias_projection(normed).permute(2, 0, 1)          # [head, N, N]
+        normed, bias = layernorm_pair_bias(pair, self.act_norm.weight, self.act_norm.bias, self.act_norm.eps, self.pair_bias_projection.weight)  # bias [head, N, N]
         rows = normed.transpose(0, 1) if self.transpose else normed         # attend along columns when transposed
         out = _attention_cpp(rows, mask, bias, *self._packed_weights(), self.num_head, False, 128 if pair.shape[1] > 256 else 64, 0)
         return out.transpose(0, 1) if self.transpose else out

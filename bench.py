@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--case cfg4] [--no-cpu-baseline]
     python bench.py --case grid_n768      (the fused grid self-attention caller; also grid_n384, self_n1536)
+    python bench.py --case ln_bias_n768   (LayerNorm + pair-bias projection in front of it)
 
 A step is one call of dot_product_attention_cpp (the drop-in for the reference's
 af3_kernels.dot_product_attention_cpp) on synthetic inputs already resident in HBM.  The default
@@ -152,6 +153,58 @@ def bench_fused(args, case):
     print(json.dumps(line))
 
 
+def bench_layernorm_pair_bias(args, n):
+    """--case ln_bias_n768: a step is one call of layernorm_pair_bias (LayerNorm over 128 channels + per-head bias projection,
+    the torch ops in front of the reference's grid attention) on a synthetic [n, n, 128] bf16 pair tensor resident in HBM."""
+    import numpy as np
+    import torch
+    import af3_kernels_amd as af3
+    af3._lib.load()
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    C, H = 128, 4
+    x = torch.randn(n, n, C, generator=g).to(torch.bfloat16).to(dev)
+    gamma = (1.0 + 0.1 * torch.randn(C, generator=g)).to(torch.bfloat16).to(dev)
+    beta = (0.1 * torch.randn(C, generator=g)).to(torch.bfloat16).to(dev)
+    wb = (torch.randn(H, C, generator=g) / C ** 0.5).to(torch.bfloat16).to(dev)
+    fn = lambda: af3.layernorm_pair_bias(x, gamma, beta, 1e-5, wb)
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream(dev)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in evs:
+        a.record(stream)
+        out = fn()
+        b.record(stream)
+    torch.cuda.synchronize()
+    per = sorted(a.elapsed_time(b) for a, b in evs)
+    kernel_ms = sum(per) / len(per)
+    ms_per_step = evs[0][0].elapsed_time(evs[-1][1]) / args.steps
+    nbytes = 2.0 * (2 * n * n * C + H * n * n)     # rows in, rows out, bias out (bf16)
+    ach = nbytes / (kernel_ms * 1e-3) / 1e9
+    line = {"metric": f"LayerNorm + pair-bias projection GB/s (ln_bias_n{n})", "value": round(nbytes / (ms_per_step * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic", "config": {"workload": f"ln_bias_n{n}: pair [{n}, {n}, 128] bf16, 4 heads", "bytes": nbytes},
+            "roofline": {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+                         "kernel": "layernorm_pair_bias_kernel", "kernel_ms_avg": round(kernel_ms, 4), "algorithmic_bytes_per_launch": nbytes}}
+    if not args.no_cpu_baseline:
+        from oracle import af3_oracle
+        rows = min(n, 64)
+        hx = x[:rows].float().cpu().numpy()
+        hg, hb, hw = gamma.float().cpu().numpy(), beta.float().cpu().numpy(), wb.float().cpu().numpy()
+        af3_oracle.layernorm_pair_bias(hx[:2], hg, hb, hw, 1e-5, round_bf16=True)
+        t0 = time.time()
+        reps = 0
+        while time.time() - t0 < 5.0:
+            af3_oracle.layernorm_pair_bias(hx, hg, hb, hw, 1e-5, round_bf16=True)
+            reps += 1
+        t = (time.time() - t0) / reps
+        line["cpu_baseline"] = {"value": round(nbytes * rows / n / t / 1e9, 2), "unit": "GB/s", "cores": int(os.environ.get("OMP_NUM_THREADS", len(os.sched_getaffinity(0)))),
+                                "kind": "port", "sample": f"{rows} of {n} pair rows x {reps} repeats, {t:.3f} s each, OpenMP double-precision formula with bf16 rounding"}
+    print(json.dumps(line))
+
+
 def cpu_baseline_fused(case, budget_s=12.0):
     """The CPU restatement of _attention_impl / self_attention_impl (oracle/af3_oracle.c, OpenMP over batch row x head like
     src/csrc/dot_product_attention.cpp:276-277, :452) in bfloat16, timed on a bounded sample of the batch rows."""
@@ -200,6 +253,8 @@ def main():
     af3._lib.load()
     if args.case in FUSED_CASES:
         return bench_fused(args, FUSED_CASES[args.case])
+    if args.case.startswith("ln_bias_n"):
+        return bench_layernorm_pair_bias(args, int(args.case[len("ln_bias_n"):]))
     case = CASES[args.case]
     dev = torch.device("cuda:0")
     q, k, v, mask, bias = make_inputs(case, device=dev)

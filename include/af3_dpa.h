@@ -236,6 +236,19 @@ int64_t af3_grid_attention_workspace_bytes(const af3_grid_attention_params* para
 int     af3_grid_attention_supported(const af3_grid_attention_params* params);
 
 /*
+ * The step in front of grid self-attention in one pass over the pair tensor: LayerNorm over the C channels of every
+ * token (biased variance, eps inside the square root) and the projection of the normalised, bf16-rounded row to one
+ * bias value per head, written as bias[h][i][j] -- the layout the attention entry points read.
+ * Replaces the torch ops of src/af3_kernels/Attention.py:51-52 (act_norm, pair_bias_projection, permute(2, 0, 1));
+ * the reference has no native code for this step.
+ * pair [n_i, n_j, C] with element strides pair_stride[2] (innermost stride 1, multiples of 8), ln_weight / ln_bias [C],
+ * proj_weight [head, C] (nn.Linear weight, contiguous), normed [n_i, n_j, C] contiguous, bias_stride = {head, row i}.
+ * Supported: dtype AF3_BF16, C == 128, head == 4, 16-byte aligned pointers; AF3_ERR_BAD_ARGUMENT otherwise.
+ */
+int af3_layernorm_pair_bias(const void* pair, const int64_t* pair_stride, const void* ln_weight, const void* ln_bias, float eps, const void* proj_weight,
+							void* normed, void* bias, const int64_t* bias_stride, int64_t n_i, int64_t n_j, int64_t C, int64_t head, int32_t dtype, void* hip_stream);
+
+/*
  * N-dimensional pad (ndim <= AF3_PAD_MAX_DIMS): copy src (shape src_shape, element strides
  * src_strides) into the low corner of a contiguous dst of shape dst_shape (>= src_shape in
  * every axis) and fill the rest with the 32-bit pattern `fill_bits` truncated to elem_size

@@ -681,3 +681,40 @@ int af3o_fused_attention_formula(const float* x, const uint8_t* keep, const floa
 	free(ga);
 	return fail ? -1 : 0;
 }
+
+/* ---- the step in front of grid self-attention ("next" row) -------------------------------- */
+
+/*
+ * LayerNorm over the C channels of every token and the per-head bias projection of the normalised row, in
+ * double precision: normed = (x - mean) / sqrt(var + eps) * gamma + beta (biased variance, torch.nn.LayerNorm),
+ * bias[h][t] = normed[t] . wb[h]  (src/af3_kernels/Attention.py:51-52: act_norm, pair_bias_projection, permute(2,0,1);
+ * examples/grid_self_attention.py:71-72).  x [T][C], wb [H][C] (nn.Linear weight), normed [T][C], bias [H][T].
+ * round_bf16 != 0 rounds the normalised row to bf16 before it is stored and projected, and the bias after, which is what
+ * the reference's bf16 module does between its torch ops.
+ */
+int af3o_layernorm_pair_bias(const float* x, const float* gamma, const float* beta, const float* wb, double eps, float* normed, float* bias, int64_t T, int64_t C, int64_t H,
+							 int round_bf16) {
+#pragma omp parallel for schedule(static)
+	for(int64_t t = 0; t < T; t++) {
+		const float* xr   = x + t * C;
+		double       mean = 0.0, var = 0.0;
+		for(int64_t c = 0; c < C; c++) mean += xr[c];
+		mean /= (double)C;
+		for(int64_t c = 0; c < C; c++) var += ((double)xr[c] - mean) * ((double)xr[c] - mean);
+		var /= (double)C;
+		const double rstd = 1.0 / sqrt(var + eps);
+		for(int64_t c = 0; c < C; c++) {
+			float y = (float)(((double)xr[c] - mean) * rstd * (double)gamma[c] + (double)beta[c]);
+			if(round_bf16) y = af3o_bf16_bits_to_f32(af3o_f32_to_bf16_bits(y));
+			normed[t * C + c] = y;
+		}
+		for(int64_t h = 0; h < H; h++) {
+			double d = 0.0;
+			for(int64_t c = 0; c < C; c++) d += (double)normed[t * C + c] * (double)wb[h * C + c];
+			float b = (float)d;
+			if(round_bf16) b = af3o_bf16_bits_to_f32(af3o_f32_to_bf16_bits(b));
+			bias[h * T + t] = b;
+		}
+	}
+	return 0;
+}

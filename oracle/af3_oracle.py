@@ -59,6 +59,8 @@ def lib():
         L.af3o_fused_attention_reference.restype = ctypes.c_int
         L.af3o_fused_attention_formula.argtypes = [fp, u8, fp, fp, fp, fp, fp, fp, fp, fp, i64, i64, i64, i64]
         L.af3o_fused_attention_formula.restype = ctypes.c_int
+        L.af3o_layernorm_pair_bias.argtypes = [fp, fp, fp, fp, ctypes.c_double, fp, fp, i64, i64, i64, ctypes.c_int]
+        L.af3o_layernorm_pair_bias.restype = ctypes.c_int
         _lib = L
     return _lib
 
@@ -134,6 +136,20 @@ def fused_attention_formula(x, mask, bias, wq, wk, wv, wg, wo=None, qbias=None, 
     """The torch modules of examples/grid_self_attention.py:46-94 (after LayerNorm and bias projection)
     and examples/self_attention.py:64-96 in double precision."""
     return _fused(lib().af3o_fused_attention_formula, x, mask, bias, wq, wk, wv, wg, wo, qbias, head, ())
+
+
+def layernorm_pair_bias(pair, gamma, beta, wb, eps=1e-5, round_bf16=False):
+    """LayerNorm over the last axis of pair [..., C] and the per-head bias projection with wb [H, C] (nn.Linear weight), in
+    double precision (src/af3_kernels/Attention.py:51-52).  Returns (normed [..., C], bias [H, ...])."""
+    pair = np.asarray(pair, dtype=np.float32)
+    lead, C = pair.shape[:-1], pair.shape[-1]
+    x, xp = _f(pair.reshape(-1, C))
+    g, gp = _f(gamma); b, bp = _f(beta); w, wp = _f(wb)
+    H, T = w.shape[0], x.shape[0]
+    normed, bias = np.empty((T, C), np.float32), np.empty((H, T), np.float32)
+    fpt = ctypes.POINTER(ctypes.c_float)
+    lib().af3o_layernorm_pair_bias(xp, gp, bp, wp, float(eps), normed.ctypes.data_as(fpt), bias.ctypes.data_as(fpt), T, C, H, int(bool(round_bf16)))
+    return normed.reshape(*lead, C), bias.reshape(H, *lead)
 
 
 def f32_to_bf16_bits(x):

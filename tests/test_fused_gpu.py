@@ -266,3 +266,48 @@ def test_output_gate_in_every_kernel(af3, oracle, dtype, force_generic, D):
     # the same call without a gate is the bare attention
     plain = ops._dpa_forward_impl(q, k, v, ops._lift_mask(mask.cuda(), L), bias.cuda(), code, force_generic)
     assert float(np.abs(f32np(plain) - oracle.dpa_formula(hq, hk, hv, mask.numpy(), f32np(bias))).max()) <= (1e-4 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("n_i,n_j,transposed", [(5, 64, False), (7, 200, False), (3, 37, False), (40, 40, True), (1, 1, False), (2, 1000, False)])
+def test_layernorm_pair_bias_matches_formula(af3, oracle, n_i, n_j, transposed):
+    """LayerNorm + per-head bias projection in one kernel against the oracle's fp64 formula: normed within one bf16 ulp of
+    the exact value, bias within the bf16 budget of a 128-term dot product of bf16-rounded rows."""
+    C, H = 128, 4
+    g = torch.Generator().manual_seed(n_i * 100 + n_j)
+    x = (torch.randn(n_i, n_j, C, generator=g) * 2.0 + 0.5).to(torch.bfloat16)
+    gamma = (1.0 + 0.2 * torch.randn(C, generator=g)).to(torch.bfloat16)
+    beta = (0.1 * torch.randn(C, generator=g)).to(torch.bfloat16)
+    wb = (torch.randn(H, C, generator=g) / C ** 0.5).to(torch.bfloat16)
+    dx = x.cuda()
+    if transposed:                 # a strided view: rows and columns swapped
+        dx = dx.transpose(0, 1)
+        x = x.transpose(0, 1)
+    print(f"layernorm_pair_bias {n_i}x{n_j} transposed={transposed}", flush=True)
+    normed, bias = af3.layernorm_pair_bias(dx, gamma.cuda(), beta.cuda(), 1e-5, wb.cuda())
+    torch.cuda.synchronize()
+    assert normed.shape == x.shape and bias.shape == (H, x.shape[0], x.shape[1]) and normed.dtype == bias.dtype == torch.bfloat16
+    want_n, _ = oracle.layernorm_pair_bias(f32np(x), f32np(gamma), f32np(beta), f32np(wb), 1e-5)
+    got_n = f32np(normed)
+    assert np.isfinite(got_n).all()
+    assert (np.abs(got_n - want_n) <= np.maximum(np.abs(want_n), 1e-2) * 2.0 ** -8 + 1e-6).all()      # half an ulp of bf16 (+ fp32 slack)
+    # the projection is checked on the rows the kernel actually stored
+    want_b = np.einsum("ijc,hc->hij", got_n.astype(np.float64), f32np(wb).astype(np.float64))
+    assert np.abs(f32np(bias) - want_b).max() <= 2e-2 * max(1.0, np.abs(want_b).max())
+    # and the reference's sequence of torch ops on the same device agrees to bf16 rounding
+    ref_n = torch.nn.functional.layer_norm(dx, (C,), gamma.cuda(), beta.cuda(), 1e-5)
+    ref_b = torch.nn.functional.linear(ref_n, wb.cuda()).permute(2, 0, 1)
+    assert float((normed.float() - ref_n.float()).abs().max()) <= 2.0 ** -6 * max(1.0, float(ref_n.float().abs().max()))
+    assert float((bias.float() - ref_b.float()).abs().max()) <= 3e-2 * max(1.0, float(ref_b.float().abs().max()))
+
+
+def test_layernorm_pair_bias_falls_back_to_torch_ops_for_other_shapes(af3, oracle):
+    """Shapes the kernel does not take (64 channels, float32) run the reference's own torch ops on the device."""
+    for C, H, dtype in ((64, 2, torch.bfloat16), (128, 4, torch.float32)):
+        g = torch.Generator().manual_seed(C)
+        x = torch.randn(6, 9, C, generator=g).to(dtype)
+        gamma, beta = torch.ones(C, dtype=dtype), torch.zeros(C, dtype=dtype)
+        wb = (torch.randn(H, C, generator=g) / C ** 0.5).to(dtype)
+        normed, bias = af3.layernorm_pair_bias(x.cuda(), gamma.cuda(), beta.cuda(), 1e-5, wb.cuda())
+        want_n, want_b = oracle.layernorm_pair_bias(f32np(x), f32np(gamma), f32np(beta), f32np(wb), 1e-5)
+        tol = 1e-4 if dtype == torch.float32 else 4e-2
+        assert np.abs(f32np(normed) - want_n).max() <= tol and np.abs(f32np(bias) - want_b).max() <= tol

@@ -315,3 +315,29 @@ def test_fused_reference_restatement_bf16_within_tolerance(oracle):
     want = oracle.fused_attention_formula(*case, head=4)
     assert np.abs(got - want).max() <= 3e-2 * max(1.0, np.abs(want).max())
     assert np.abs(got - want).sum() / np.abs(want).sum() <= 2e-2
+
+
+def test_layernorm_pair_bias_matches_torch_library_ops(oracle):
+    """The oracle's LayerNorm + bias projection against torch.nn.functional.layer_norm / linear in float64; constant rows
+    (zero variance) give beta; doubling a head's projection row doubles that head's bias only."""
+    rng = np.random.default_rng(21)
+    N1, N2, C, H = 5, 7, 32, 3
+    x = (rng.standard_normal((N1, N2, C)) * 3 + 10).astype(np.float32)          # a large mean: catches a one-pass variance
+    gamma, beta = rng.standard_normal(C).astype(np.float32), rng.standard_normal(C).astype(np.float32)
+    wb = rng.standard_normal((H, C)).astype(np.float32)
+    normed, bias = oracle.layernorm_pair_bias(x, gamma, beta, wb, 1e-5)
+    t = lambda a: torch.from_numpy(a).double()
+    want_n = torch.nn.functional.layer_norm(t(x), (C,), t(gamma), t(beta), 1e-5)
+    want_b = torch.nn.functional.linear(want_n, t(wb)).permute(2, 0, 1)
+    assert normed.shape == (N1, N2, C) and bias.shape == (H, N1, N2)
+    assert np.abs(normed - want_n.numpy()).max() <= 2e-6 and np.abs(bias - want_b.numpy()).max() <= 2e-5
+    const = np.full((2, 2, C), 4.0, np.float32)
+    n2, b2 = oracle.layernorm_pair_bias(const, gamma, beta, wb, 1e-5)
+    assert np.abs(n2 - beta).max() <= 1e-6 and np.abs(b2 - (wb @ beta)[:, None, None]).max() <= 1e-5
+    wb2 = wb.copy()
+    wb2[1] *= 2
+    _, b3 = oracle.layernorm_pair_bias(x, gamma, beta, wb2, 1e-5)
+    assert np.allclose(b3[1], 2 * bias[1], rtol=1e-6) and np.array_equal(b3[[0, 2]], bias[[0, 2]])
+    # bf16 rounding variant: normed values are bf16-representable and within half an ulp of the exact ones
+    n4, b4 = oracle.layernorm_pair_bias(x, gamma, beta, wb, 1e-5, round_bf16=True)
+    assert np.array_equal(oracle.round_bf16(n4), n4) and np.abs(n4 - normed).max() <= np.abs(normed).max() * 2.0 ** -8

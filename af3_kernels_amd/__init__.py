@@ -10,7 +10,7 @@ libaf3_dpa.so (hand-written HIP for gfx950) through the C ABI of include/af3_dpa
 Inputs must live on a ROCm device; there is no CPU path and no PyTorch fallback.
 """
 from . import _lib
-from .fused import GridSelfAttentionCpp, _attention_cpp, layernorm_pair_bias, self_attention_cpp  # noqa: F401
+from .fused import GridSelfAttentionCpp, Linear, _attention_cpp, gated_linear_unit_cpp, layernorm_pair_bias, self_attention_cpp  # noqa: F401
 from .ops import (  # noqa: F401
     convert,
     dot_product_attention_cpp,
@@ -28,5 +28,5 @@ from .ops import (  # noqa: F401
 __all__ = [
     "dot_product_attention_cpp", "dot_product_attention_fp8", "pad_and_align_tensor", "vnni_repack_tensor",
     "reset_debug_timers", "print_debug_timers", "print_debug_thread_imbalance", "convert", "quantize_fp8_e4m3",
-    "selected_kernel", "set_exact_bias", "_attention_cpp", "self_attention_cpp", "GridSelfAttentionCpp", "layernorm_pair_bias",
+    "selected_kernel", "set_exact_bias", "_attention_cpp", "self_attention_cpp", "GridSelfAttentionCpp", "layernorm_pair_bias", "gated_linear_unit_cpp", "Linear",
 ]

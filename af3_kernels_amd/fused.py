@@ -281,3 +281,58 @@ class GridSelfAttentionCpp(torch.nn.Module):
         rows = normed.transpose(0, 1) if self.transpose else normed         # attend along columns when transposed
         out = _attention_cpp(rows, mask, bias, *self._packed_weights(), self.num_head, False, 128 if pair.shape[1] > 256 else 64, 0)
         return out.transpose(0, 1) if self.transpose else out
+
+
+def _plain_weight(weight: torch.Tensor, vnni_repacked: bool, N_BLK: int) -> torch.Tensor:
+    """[K, N] weight as the reference's callers hand it over -- plain, or VNNI panels of width N_BLK
+    (vnni_repack_tensor(W, 2, N_BLK): [N/N_BLK][K/2][N_BLK][2]) -- back to plain [K, N]."""
+    if not vnni_repacked:
+        return weight
+    K, N = weight.shape
+    blk = min(N_BLK, N) if N_BLK > 0 else N
+    if weight.dtype != torch.bfloat16 or N % blk != 0 or K % 2 != 0:
+        raise ValueError("a VNNI-repacked weight is bfloat16 [K, N] with K even and N a multiple of N_BLK")
+    return weight.reshape(N // blk, K // 2, blk, 2).permute(1, 3, 0, 2).reshape(K, N)
+
+
+def gated_linear_unit_cpp(x: torch.Tensor, weight: torch.Tensor, vnni_repacked: bool = False, M_BLK: int = 128, N_BLK: int = 128) -> torch.Tensor:
+    """silu(x @ W[:, :N]) * (x @ W[:, N:]) -- drop-in for the reference's gated_linear_unit_cpp (src/af3_kernels/__init__.py:
+    21-28; src/csrc/gated_linear_unit.cpp:20-80).  x [..., K], weight [K, 2N] (plain or VNNI-repacked with N_BLK); returns
+    [..., N] in x's dtype.  bfloat16 with K = 64 or 128 and N % 32 == 0 is one HIP kernel (the [.., 2N] product is never
+    stored); other shapes run the formula's torch ops on the device.  M_BLK and N_BLK are CPU blocking sizes (N_BLK also
+    names the panel width of a repacked weight) and change nothing else."""
+    ops._require_device(x, weight)
+    if weight.dim() != 2 or weight.shape[0] != x.shape[-1] or weight.shape[1] % 2 != 0:
+        raise ValueError(f"weight must be [K, 2N] with K = x.shape[-1] = {x.shape[-1]}, got {tuple(weight.shape)}")
+    K, N = weight.shape[0], weight.shape[1] // 2
+    lead = x.shape[:-1]
+    if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and K in (64, 128) and N % 32 == 0 and x.numel() > 0):
+        y = torch.matmul(x, _plain_weight(weight, vnni_repacked, N_BLK).to(x.dtype))
+        a, b = torch.chunk(y, 2, dim=-1)
+        return torch.nn.functional.silu(a) * b
+    wt = _cached((weight,), (bool(vnni_repacked), N_BLK, "glu"), lambda: _plain_weight(weight, vnni_repacked, N_BLK).t().contiguous())
+    x2 = x.reshape(-1, K)
+    if not x2.is_contiguous() or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    out = torch.empty(x2.shape[0], N, dtype=x.dtype, device=x.device)
+    with ops._on_device(x.device):
+        _lib.check(_lib.load().af3_gated_linear_unit(x2.data_ptr(), wt.data_ptr(), out.data_ptr(), x2.shape[0], K, N, ops._DTYPE_CODE[x.dtype],
+                                                     ops._stream_ptr(x.device)), "af3_gated_linear_unit")
+    return out.view(*lead, N)
+
+
+class Linear(torch.nn.Module):
+    """Bias-free linear layer with the reference's constructor (src/af3_kernels/__init__.py:138-163).  The reference repacks
+    the weight into VNNI panels for its CPU GEMM; here the product is a library GEMM (hipBLASLt) on the plain weight."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None, M_BLK: int = 128, N_BLK: int = 128) -> None:
+        super().__init__()
+        assert bias is False
+        self.in_features, self.out_features = in_features, out_features
+        self.weight = torch.nn.Parameter(torch.empty((out_features, in_features), device=device, dtype=dtype))
+        self.register_parameter("bias", None)
+        self.M_BLK, self.N_BLK = M_BLK, N_BLK
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        ops._require_device(input, self.weight)
+        return torch.nn.functional.linear(input, self.weight)

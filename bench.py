@@ -3,6 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--case cfg4] [--no-cpu-baseline]
     python bench.py --case grid_n768      (the fused grid self-attention caller; also grid_n384, self_n1536)
     python bench.py --case ln_bias_n768   (LayerNorm + pair-bias projection in front of it)
+    python bench.py --case glu_n1536      (the gated linear unit of the transition blocks)
 
 A step is one call of dot_product_attention_cpp (the drop-in for the reference's
 af3_kernels.dot_product_attention_cpp) on synthetic inputs already resident in HBM.  The default
@@ -205,6 +206,54 @@ def bench_layernorm_pair_bias(args, n):
     print(json.dumps(line))
 
 
+def bench_glu(args, n):
+    """--case glu_n1536: a step is one call of gated_linear_unit_cpp on x [n, n, 128] bf16 with weight [128, 1024] (the reference
+    harness's largest set, examples/gated_linear_unit.py:36-40), inputs resident in HBM."""
+    import torch
+    import af3_kernels_amd as af3
+    af3._lib.load()
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    K, N = 128, 512
+    x = torch.randn(n, n, K, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(K, 2 * N, generator=g) / K ** 0.5).to(torch.bfloat16).to(dev)
+    fn = lambda: af3.gated_linear_unit_cpp(x, w, False, 128, 128)
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream(dev)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in evs:
+        a.record(stream)
+        out = fn()
+        b.record(stream)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    per = sorted(a.elapsed_time(b) for a, b in evs)
+    kernel_ms = sum(per) / len(per)
+    ms_per_step = evs[0][0].elapsed_time(evs[-1][1]) / args.steps
+    M = n * n
+    nbytes = 2.0 * (M * K + M * N + 2 * K * N)
+    flops = 2.0 * M * K * 2 * N
+    ach = nbytes / (kernel_ms * 1e-3) / 1e9
+    line = {"metric": f"gated linear unit GB/s (glu_n{n})", "value": round(nbytes / (ms_per_step * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"glu_n{n}: x [{n}, {n}, 128] bf16, weight [128, 1024]", "bytes": nbytes, "flops": flops, "tflops": round(flops / (ms_per_step * 1e-3) / 1e12, 1)},
+            "roofline": {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+                         "kernel": "glu_kernel<8>", "kernel_ms_avg": round(kernel_ms, 4), "algorithmic_bytes_per_launch": nbytes}}
+    if not args.no_cpu_baseline:
+        from oracle import af3_oracle
+        rows = min(M, 16384)
+        hx, hw = x.view(M, K)[:rows].float().cpu().numpy(), w.float().cpu().numpy()
+        af3_oracle.gated_linear_unit(hx[:256], hw, round_bf16=True)
+        t0 = time.time()
+        af3_oracle.gated_linear_unit(hx, hw, round_bf16=True)
+        t = time.time() - t0
+        line["cpu_baseline"] = {"value": round(nbytes * rows / M / t / 1e9, 3), "unit": "GB/s", "cores": int(os.environ.get("OMP_NUM_THREADS", len(os.sched_getaffinity(0)))),
+                                "kind": "port", "sample": f"{rows} of {M} rows, {t:.2f} s wall, OpenMP restatement with the reference's bf16 roundings (scalar inner products)"}
+    print(json.dumps(line))
+
+
 def cpu_baseline_fused(case, budget_s=12.0):
     """The CPU restatement of _attention_impl / self_attention_impl (oracle/af3_oracle.c, OpenMP over batch row x head like
     src/csrc/dot_product_attention.cpp:276-277, :452) in bfloat16, timed on a bounded sample of the batch rows."""
@@ -253,6 +302,8 @@ def main():
     af3._lib.load()
     if args.case in FUSED_CASES:
         return bench_fused(args, FUSED_CASES[args.case])
+    if args.case.startswith("glu_n"):
+        return bench_glu(args, int(args.case[len("glu_n"):]))
     if args.case.startswith("ln_bias_n"):
         return bench_layernorm_pair_bias(args, int(args.case[len("ln_bias_n"):]))
     case = CASES[args.case]

@@ -249,6 +249,17 @@ int af3_layernorm_pair_bias(const void* pair, const int64_t* pair_stride, const 
 							void* normed, void* bias, const int64_t* bias_stride, int64_t n_i, int64_t n_j, int64_t C, int64_t head, int32_t dtype, void* hip_stream);
 
 /*
+ * Gated linear unit: out[m][n] = silu(x[m] . Wa[:, n]) * (x[m] . Wb[:, n]) in one kernel (the [M, 2N] product is never
+ * stored).  x [M, K] contiguous, out [M, N] contiguous, weight_t = [Wa | Wb]^T, i.e. [2N, K] row-major (the
+ * nn.Linear layout [out_features, in_features]: rows 0..N-1 gate, rows N..2N-1 value).
+ * Replaces: at::Tensor gated_linear_unit(input, weight, vnni_repacked, M_BLK, N_BLK) -- src/csrc/gated_linear_unit.h,
+ * implemented at src/csrc/gated_linear_unit.cpp:20-80, :131-138 (the reference takes the weight as [K, 2N], plain or
+ * VNNI-repacked; its CPU blocking arguments have no counterpart).
+ * Supported: dtype AF3_BF16, K == 64 or 128, N % 32 == 0, 16-byte aligned x and weight_t; AF3_ERR_BAD_ARGUMENT otherwise.
+ */
+int af3_gated_linear_unit(const void* x, const void* weight_t, void* out, int64_t M, int64_t K, int64_t N, int32_t dtype, void* hip_stream);
+
+/*
  * N-dimensional pad (ndim <= AF3_PAD_MAX_DIMS): copy src (shape src_shape, element strides
  * src_strides) into the low corner of a contiguous dst of shape dst_shape (>= src_shape in
  * every axis) and fill the rest with the 32-bit pattern `fill_bits` truncated to elem_size

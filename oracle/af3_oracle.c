@@ -718,3 +718,38 @@ int af3o_layernorm_pair_bias(const float* x, const float* gamma, const float* be
 	}
 	return 0;
 }
+
+/* ---- gated linear unit ("next" row) -------------------------------------------------------- */
+
+/*
+ * out[m][n] = silu(a) * b with a = x[m] . w[:, n], b = x[m] . w[:, N + n]  (examples/gated_linear_unit.py:18-22),
+ * x [M][K], w [K][2N] row-major.  round_bf16 == 0: double precision throughout.  round_bf16 != 0: the reference's
+ * bf16 pipeline (src/csrc/gated_linear_unit.cpp:56-61): both products accumulated in fp32 and rounded to bf16,
+ * silu evaluated in fp32 on the rounded value and rounded, the product rounded.
+ */
+int af3o_gated_linear_unit(const float* x, const float* w, float* out, int64_t M, int64_t K, int64_t N, int round_bf16) {
+#pragma omp parallel for schedule(static)
+	for(int64_t m = 0; m < M; m++) {
+		for(int64_t n = 0; n < N; n++) {
+			if(!round_bf16) {
+				double a = 0.0, b = 0.0;
+				for(int64_t k = 0; k < K; k++) {
+					a += (double)x[m * K + k] * (double)w[k * 2 * N + n];
+					b += (double)x[m * K + k] * (double)w[k * 2 * N + N + n];
+				}
+				out[m * N + n] = (float)(a / (1.0 + exp(-a)) * b);
+			} else {
+				float a = 0.f, b = 0.f;
+				for(int64_t k = 0; k < K; k++) {
+					a += x[m * K + k] * w[k * 2 * N + n];
+					b += x[m * K + k] * w[k * 2 * N + N + n];
+				}
+				a             = af3o_bf16_bits_to_f32(af3o_f32_to_bf16_bits(a));
+				b             = af3o_bf16_bits_to_f32(af3o_f32_to_bf16_bits(b));
+				const float s = af3o_bf16_bits_to_f32(af3o_f32_to_bf16_bits(a / (1.f + expf(-a))));
+				out[m * N + n] = af3o_bf16_bits_to_f32(af3o_f32_to_bf16_bits(s * b));
+			}
+		}
+	}
+	return 0;
+}

@@ -61,6 +61,8 @@ def lib():
         L.af3o_fused_attention_formula.restype = ctypes.c_int
         L.af3o_layernorm_pair_bias.argtypes = [fp, fp, fp, fp, ctypes.c_double, fp, fp, i64, i64, i64, ctypes.c_int]
         L.af3o_layernorm_pair_bias.restype = ctypes.c_int
+        L.af3o_gated_linear_unit.argtypes = [fp, fp, fp, i64, i64, i64, ctypes.c_int]
+        L.af3o_gated_linear_unit.restype = ctypes.c_int
         _lib = L
     return _lib
 
@@ -150,6 +152,19 @@ def layernorm_pair_bias(pair, gamma, beta, wb, eps=1e-5, round_bf16=False):
     fpt = ctypes.POINTER(ctypes.c_float)
     lib().af3o_layernorm_pair_bias(xp, gp, bp, wp, float(eps), normed.ctypes.data_as(fpt), bias.ctypes.data_as(fpt), T, C, H, int(bool(round_bf16)))
     return normed.reshape(*lead, C), bias.reshape(H, *lead)
+
+
+def gated_linear_unit(x, weight, round_bf16=False):
+    """silu(x @ W[:, :N]) * (x @ W[:, N:]) for x [..., K], weight [K, 2N] (examples/gated_linear_unit.py:18-22), in double
+    precision, or with the reference's bf16 roundings (src/csrc/gated_linear_unit.cpp:56-61) when round_bf16."""
+    x = np.asarray(x, dtype=np.float32)
+    lead, K = x.shape[:-1], x.shape[-1]
+    x2, xp = _f(x.reshape(-1, K))
+    w, wp = _f(weight)
+    N = w.shape[1] // 2
+    out = np.empty((x2.shape[0], N), np.float32)
+    lib().af3o_gated_linear_unit(xp, wp, out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), x2.shape[0], K, N, int(bool(round_bf16)))
+    return out.reshape(*lead, N)
 
 
 def f32_to_bf16_bits(x):

@@ -311,3 +311,47 @@ def test_layernorm_pair_bias_falls_back_to_torch_ops_for_other_shapes(af3, oracl
         want_n, want_b = oracle.layernorm_pair_bias(f32np(x), f32np(gamma), f32np(beta), f32np(wb), 1e-5)
         tol = 1e-4 if dtype == torch.float32 else 4e-2
         assert np.abs(f32np(normed) - want_n).max() <= tol and np.abs(f32np(bias) - want_b).max() <= tol
+
+
+@pytest.mark.parametrize("lead,K,N,repacked", [((37, 37), 128, 256, False), ((200,), 128, 512, True), ((3, 50), 64, 512, False), ((65,), 128, 1024, True),
+                                               ((1,), 64, 32, False), ((2, 31), 128, 96, False)])
+def test_gated_linear_unit_matches_formula(af3, oracle, lead, K, N, repacked):
+    """The one-kernel GLU against the fp64 formula on the same bf16 inputs: 2e-2 * max(1, |out|) like the other bf16 ops, and
+    no worse than twice the error of the reference's own bf16 arithmetic restated on the CPU."""
+    g = torch.Generator().manual_seed(K + N)
+    x = torch.randn(*lead, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(K, 2 * N, generator=g) / K ** 0.5).to(torch.bfloat16)
+    dw = af3.vnni_repack_tensor(w.cuda(), 2, 128) if repacked else w.cuda()
+    print(f"gated_linear_unit_cpp x={tuple(x.shape)} weight={tuple(w.shape)} repacked={repacked}", flush=True)
+    out = af3.gated_linear_unit_cpp(x.cuda(), dw, repacked, 128, 128)
+    torch.cuda.synchronize()
+    assert out.shape == (*lead, N) and out.dtype == torch.bfloat16
+    want = oracle.gated_linear_unit(f32np(x), f32np(w))
+    ref = oracle.gated_linear_unit(f32np(x), f32np(w), round_bf16=True)
+    got = f32np(out)
+    assert np.isfinite(got).all()
+    scale = max(1.0, float(np.abs(want).max()))
+    err, ref_err = float(np.abs(got - want).max()), float(np.abs(ref - want).max())
+    assert err <= 2e-2 * scale and err <= 2.0 * ref_err + 4e-3 * scale, (err, ref_err)
+
+
+def test_gated_linear_unit_other_shapes_and_linear_module(af3, oracle):
+    """Shapes outside the kernel's (float32, K = 48) run the formula's torch ops on the device; the Linear module is x @ W^T."""
+    g = torch.Generator().manual_seed(9)
+    for K, N, dtype, tol in ((48, 40, torch.bfloat16, 3e-2), (128, 64, torch.float32, 1e-4)):
+        x = torch.randn(7, 11, K, generator=g).to(dtype)
+        w = (torch.randn(K, 2 * N, generator=g) / K ** 0.5).to(dtype)
+        out = af3.gated_linear_unit_cpp(x.cuda(), w.cuda())
+        want = oracle.gated_linear_unit(f32np(x), f32np(w))
+        assert np.abs(f32np(out) - want).max() <= tol * max(1.0, float(np.abs(want).max()))
+    lin = af3.Linear(128, 512, False, dtype=torch.bfloat16, M_BLK=128, N_BLK=128).cuda()
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(512, 128, generator=g) / 128 ** 0.5).to(torch.bfloat16))
+        x = torch.randn(37, 37, 128, generator=g).to(torch.bfloat16)
+        y = lin(x.cuda())
+    want = f32np(x).astype(np.float64) @ f32np(lin.weight).astype(np.float64).T
+    assert y.shape == (37, 37, 512) and np.abs(f32np(y) - want).max() <= 2e-2 * max(1.0, np.abs(want).max())
+    with pytest.raises(RuntimeError):
+        lin(x)                                                             # CPU input: no CPU path
+    with pytest.raises(ValueError):
+        af3.gated_linear_unit_cpp(x.cuda(), torch.zeros(64, 512, dtype=torch.bfloat16, device="cuda"))   # K mismatch

@@ -341,3 +341,28 @@ def test_layernorm_pair_bias_matches_torch_library_ops(oracle):
     # bf16 rounding variant: normed values are bf16-representable and within half an ulp of the exact ones
     n4, b4 = oracle.layernorm_pair_bias(x, gamma, beta, wb, 1e-5, round_bf16=True)
     assert np.array_equal(oracle.round_bf16(n4), n4) and np.abs(n4 - normed).max() <= np.abs(normed).max() * 2.0 ** -8
+
+
+def test_gated_linear_unit_matches_torch_library_ops(oracle):
+    """The GLU formula against torch.matmul / chunk / silu in float64; the bf16-rounded restatement stays within the bf16
+    budget; zero gate weights give zero; a gate of +large passes the value through."""
+    rng = np.random.default_rng(31)
+    K, N = 32, 24
+    x = rng.standard_normal((3, 5, K)).astype(np.float32)
+    w = (rng.standard_normal((K, 2 * N)) / np.sqrt(K)).astype(np.float32)
+    got = oracle.gated_linear_unit(x, w)
+    y = torch.from_numpy(x).double() @ torch.from_numpy(w).double()
+    a, b = torch.chunk(y, 2, dim=-1)
+    want = (torch.nn.functional.silu(a) * b).numpy()
+    assert got.shape == (3, 5, N) and np.abs(got - want).max() <= 2e-6
+    xb, wbf = oracle.round_bf16(x), oracle.round_bf16(w)
+    exact, rounded = oracle.gated_linear_unit(xb, wbf), oracle.gated_linear_unit(xb, wbf, round_bf16=True)
+    assert np.abs(rounded - exact).max() <= 2e-2 * max(1.0, np.abs(exact).max())
+    w0 = w.copy()
+    w0[:, :N] = 0.0
+    assert np.array_equal(oracle.gated_linear_unit(x, w0), np.zeros((3, 5, N), np.float32))
+    wl = w.copy()
+    wl[:, :N] = 0.0
+    xl = np.concatenate([x, np.ones((3, 5, 1), np.float32)], axis=-1)          # one extra channel that only feeds the gate
+    wl = np.concatenate([wl, np.concatenate([np.full((1, N), 40.0, np.float32), np.zeros((1, N), np.float32)], axis=1)], axis=0)
+    assert np.abs(oracle.gated_linear_unit(xl, wl) - 40.0 * (x @ w[:, N:])).max() <= 1e-3    # silu(40) = 40 to fp32

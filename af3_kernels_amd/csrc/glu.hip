@@ -4,13 +4,27 @@
 // Reference: gated_linear_unit_impl, src/csrc/gated_linear_unit.cpp:20-80 (per 128 x 128 block: BRGEMM, SiLU, BRGEMM,
 // multiply); formula examples/gated_linear_unit.py:18-22.
 //
-// HBM-bound (rows in, rows out); the work split keeps every byte to one trip:
+// HBM-bound (rows in, rows out).  Work split:
 //   * a workgroup owns up to 512 output columns: wavefront w holds the weight fragments of gate columns
 //     [32w, 32w+32) and of the matching value columns in registers for its whole life;
-//   * it walks blocks of 32 rows (persistent, grid-strided); a block of x (32 x K bf16) is fetched once, 16 bytes per
-//     thread, coalesced, into a double-buffered LDS tile from which all wavefronts read their MFMA operand;
+//   * it walks blocks of 32 rows (persistent, grid-strided); a block of x (32 x K bf16, one contiguous piece of memory) is
+//     fetched once, every thread a few bytes, coalesced, into a double-buffered LDS tile from which all wavefronts read
+//     their MFMA operand (reading the operand straight from memory in every wavefront -- 16 bytes per lane from 32 different
+//     rows, sixteen wavefronts per block -- was tried: twice as slow);
 //   * out^T[col][row] = W^T . x^T on v_mfma_f32_32x32x16_bf16: lane = row, registers = 4 x 4 consecutive columns, so
-//     silu * value is in-lane and the result leaves as 8-byte stores.
+//     silu * value is in-lane;
+//   * the 32 x 32 result tile is turned through a private LDS patch so that it leaves as 16-byte stores, four lanes per
+//     64-byte row segment (8-byte stores straight from the accumulator layout made the memory system handle four times
+//     as many write requests).
+// Two details keep a wavefront from waiting for its own stores to be acknowledged in every block:
+//   * loads and stores go through buffer descriptors of one block each (wave-uniform base, hardware range check), so rows
+//     past M read zeros / store nothing without a branch around the instruction -- after a branch the compiler waits for
+//     ALL outstanding memory operations where only the next block's rows are needed;
+//   * the registers that feed the stores are kept out of circulation until the next block's stores (the compiler waits for
+//     a store before it lets anything overwrite the store's data registers, and would otherwise hand them to the next
+//     block's first matrix instruction).
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace af3 {
@@ -20,18 +34,19 @@ namespace {
 constexpr int GLU_MAX_WAVES = 16;
 
 template <int KS>  // contraction steps of 16 channels: K = 16 * KS
-__global__ void __launch_bounds__(GLU_MAX_WAVES * 64) glu_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ wt, uint16_t* __restrict__ out, int64_t M, int64_t N,
-																  int n_waves) {
+__global__ void __launch_bounds__(GLU_MAX_WAVES * 64) glu_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ wt, uint16_t* __restrict__ out, int64_t M, int64_t N) {
 	constexpr int K          = 16 * KS;
 	constexpr int ROW_BYTES  = K * 2;
-	constexpr int CHUNKS     = 32 * ROW_BYTES / 16;  // 16-byte pieces of one block of x
 	constexpr int TILE_BYTES = 32 * ROW_BYTES;
+	constexpr int TPB        = TILE_BYTES / (GLU_MAX_WAVES * 64);  // bytes of a block per thread: 8 (K = 128) or 4 (K = 64)
+	constexpr int OUT_STRIDE = 80;  // bytes per row of the output patch: 64 of data, padded so that rows start in different banks
 	__shared__ __attribute__((aligned(16))) unsigned char xs[2][TILE_BYTES];
+	__shared__ __attribute__((aligned(16))) unsigned char os[GLU_MAX_WAVES][32 * OUT_STRIDE];
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int n = lane & 31, half = lane >> 5;
 	const int64_t col0   = ((int64_t)blockIdx.y * GLU_MAX_WAVES + wave) * 32;  // first gate column of this wavefront
-	const bool    active = wave < n_waves && col0 < N;
+	const bool    active = col0 < N;  // wavefronts past the last column only help to move x
 
 	// weight fragments (A operand): lane (column n, g = half), step s: W^T[col][16s + 8g .. +7]; wt is [2N, K] row-major
 	u32x4 wa[KS], wb[KS];
@@ -45,56 +60,74 @@ __global__ void __launch_bounds__(GLU_MAX_WAVES * 64) glu_kernel(const uint16_t*
 	}
 
 	const int64_t n_blocks = (M + 31) / 32;
-	// x block loader: thread t < CHUNKS moves piece t (row t / (CHUNKS/32), 16-byte chunk t % (CHUNKS/32)); the chunk index is
-	// XOR-swizzled with the row so that the operand reads below (same chunk, 8 consecutive rows per LDS cycle) spread over the banks
-	constexpr int CPR  = ROW_BYTES / 16;
-	const int     ld_r = tid / CPR, ld_c = tid % CPR;
-	const int     ld_dst = ld_r * ROW_BYTES + ((ld_c ^ (ld_r & 7)) << 4);
-	auto fetch = [&](int64_t blk) -> u32x4 {
-		const int64_t row = blk * 32 + ld_r;
-		if(tid < CHUNKS && row < M) return *reinterpret_cast<const u32x4*>(x + row * K + ld_c * 8);
-		return u32x4{0u, 0u, 0u, 0u};
+	auto rows_in = [&](int64_t blk) -> int { return (int)(M - blk * 32 < 32 ? M - blk * 32 : 32); };
+	// x block mover: thread t moves bytes [TPB*t, TPB*t + TPB) of the block.  In LDS the 16-byte chunk index of a row is
+	// XOR-swizzled with the row so that the operand reads below (same chunk, consecutive rows) spread over the banks.
+	typedef typename std::conditional<TPB == 8, u32x2, uint32_t>::type piece_t;
+	const int ld_off = tid * TPB;
+	const int ld_row = ld_off / ROW_BYTES, ld_col = ld_off % ROW_BYTES;
+	const int ld_dst = ld_row * ROW_BYTES + (((ld_col >> 4) ^ (ld_row & 7)) << 4) + (ld_col & 15);
+	auto fetch = [&](int64_t blk) -> piece_t {
+		const __amdgpu_buffer_rsrc_t r =
+			__builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(reinterpret_cast<const unsigned char*>(x)) + blk * TILE_BYTES, 0, rows_in(blk) * ROW_BYTES, 0x00020000);
+		if constexpr(TPB == 8) return __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, ld_off, 0, 0));
+		else return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, ld_off, 0, 0);
 	};
+	// operand reads (lane = row n, chunk 2s + half, swizzled) and the output patch
+	const int            x_rd  = n * ROW_BYTES;
+	const int            sw    = n & 7;
+	unsigned char* const patch = os[wave];
+	const int            p_wr  = n * OUT_STRIDE + half * 8;
+	const int            p_rd  = (lane >> 2) * OUT_STRIDE + (lane & 3) * 16;
+	const int            o_off = (int)(((lane >> 2) * N + col0 + (lane & 3) * 8) * 2);  // bytes from the block's first row (N < 2^20 checked by the launcher)
 
 	int64_t blk = blockIdx.x;
 	if(blk >= n_blocks) return;  // (whole workgroup)
-	u32x4 staged = fetch(blk);
-	if(tid < CHUNKS) *reinterpret_cast<u32x4*>(xs[0] + ld_dst) = staged;
+	piece_t staged = fetch(blk);
+	*reinterpret_cast<piece_t*>(xs[0] + ld_dst) = staged;
 	__syncthreads();
-	int buf = 0;
+	int   buf = 0;
+	u32x4 sv[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};  // the data of the two stores of a block
 	for(; blk < n_blocks; blk += gridDim.x) {
-		const int64_t next = blk + gridDim.x;
-		if(next < n_blocks) staged = fetch(next);  // in flight during this block's matrix work
-		if(active) {
-			f32x16 ga, va;
+		const int64_t next     = blk + gridDim.x;
+		const bool    has_next = next < n_blocks;  // (uniform)
+		staged = fetch(has_next ? next : blk);       // in flight during this block's matrix work (the last block is fetched again: no branch)
+		const unsigned char* const xb = xs[buf] + x_rd;
+		f32x16 ga, va;
 #pragma unroll
-			for(int i = 0; i < 16; i++) ga[i] = 0.f, va[i] = 0.f;
+		for(int i = 0; i < 16; i++) ga[i] = 0.f, va[i] = 0.f;
 #pragma unroll
-			for(int s = 0; s < KS; s++) {
-				const u32x4 xf = *reinterpret_cast<const u32x4*>(xs[buf] + n * ROW_BYTES + (((2 * s + half) ^ (n & 7)) << 4));
-				ga = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wa[s]), __builtin_bit_cast(bf16x8, xf), ga, 0, 0, 0);
-				va = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wb[s]), __builtin_bit_cast(bf16x8, xf), va, 0, 0, 0);
-			}
-			const int64_t row = blk * 32 + n;
-			if(row < M) {
-				uint16_t* orow = out + row * N + col0 + 4 * half;
-#pragma unroll
-				for(int g4 = 0; g4 < 4; g4++) {
-					float o[4];
-#pragma unroll
-					for(int r = 0; r < 4; r++) {
-						const float a = ga[4 * g4 + r];
-						o[r] = a * va[4 * g4 + r] * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-a * LOG2E));  // silu(a) * b
-					}
-					*reinterpret_cast<u32x2*>(orow + 8 * g4) = u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
-				}
-			}
+		for(int s = 0; s < KS; s++) {
+			const u32x4 xf = *reinterpret_cast<const u32x4*>(xb + (((2 * s + half) ^ sw) << 4));
+			ga = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wa[s]), __builtin_bit_cast(bf16x8, xf), ga, 0, 0, 0);
+			va = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wb[s]), __builtin_bit_cast(bf16x8, xf), va, 0, 0, 0);
 		}
-		if(next < n_blocks) {
-			if(tid < CHUNKS) *reinterpret_cast<u32x4*>(xs[buf ^ 1] + ld_dst) = staged;  // (last read two barriers ago)
-			__syncthreads();
-			buf ^= 1;
+		// silu(a) * b, rounded to bf16, into this wavefront's patch: lane (row n, half) owns columns 8*g4 + 4*half .. +3
+#pragma unroll
+		for(int g4 = 0; g4 < 4; g4++) {
+			float o[4];
+#pragma unroll
+			for(int r = 0; r < 4; r++) {
+				const float a = ga[4 * g4 + r];
+				o[r] = a * va[4 * g4 + r] * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-a * LOG2E));
+			}
+			*reinterpret_cast<u32x2*>(patch + p_wr + g4 * 16) = u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
 		}
+		// (the same wavefront writes and reads the patch, and its LDS operations complete in order; the wave barriers
+		// only keep the compiler from moving the reads above the writes, or the next block's writes above the reads)
+		__builtin_amdgcn_wave_barrier();
+		asm volatile("" : "+v"(sv[0]), "+v"(sv[1]));  // sv's registers stay reserved from the previous block's stores up to here
+		sv[0] = *reinterpret_cast<const u32x4*>(patch + p_rd);
+		sv[1] = *reinterpret_cast<const u32x4*>(patch + p_rd + 16 * OUT_STRIDE);
+		__builtin_amdgcn_wave_barrier();
+		const __amdgpu_buffer_rsrc_t orsrc = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<unsigned char*>(out) + blk * 32 * N * 2, 0, active ? (int)(rows_in(blk) * N * 2) : 0, 0x00020000);
+		typedef __attribute__((ext_vector_type(4))) unsigned int store_t;
+		__builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(store_t, sv[0]), orsrc, o_off, 0, 0);
+		__builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(store_t, sv[1]), orsrc, o_off + (int)(16 * N * 2), 0, 0);
+		// publish the next block (its LDS buffer was last read before the previous barrier)
+		*reinterpret_cast<piece_t*>(xs[buf ^ 1] + ld_dst) = staged;
+		__syncthreads();
+		buf ^= 1;
 	}
 }
 
@@ -108,21 +141,21 @@ extern "C" int af3_gated_linear_unit(const void* x, const void* weight_t, void* 
 	if(!x || !weight_t || !out) return AF3_ERR_NULL_POINTER;
 	if(M <= 0 || N <= 0 || K <= 0 || M > ((int64_t)1 << 40)) return AF3_ERR_BAD_SHAPE;
 	if(dtype != AF3_BF16) return AF3_ERR_BAD_DTYPE;
-	if((K != 64 && K != 128) || N % 32 != 0) return AF3_ERR_BAD_ARGUMENT;
-	if((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(weight_t) & 15) || (reinterpret_cast<uintptr_t>(out) & 7)) return AF3_ERR_BAD_ARGUMENT;
-	const int64_t col_tiles = N / 32;
-	const int     n_waves   = (int)(col_tiles < GLU_MAX_WAVES ? col_tiles : GLU_MAX_WAVES);
-	// the x loader needs one thread per 16-byte piece of a block: 32 * K / 8 threads
-	const int     threads   = (n_waves * 64 < 4 * K ? 4 * (int)K : n_waves * 64);
-	const int64_t n_blocks  = (M + 31) / 32;
-	const dim3    grid((unsigned)(n_blocks < 512 ? n_blocks : 512), (unsigned)((col_tiles + GLU_MAX_WAVES - 1) / GLU_MAX_WAVES));
-	const auto    s = static_cast<hipStream_t>(stream);
-	const auto*   xp = static_cast<const uint16_t*>(x);
-	const auto*   wp = static_cast<const uint16_t*>(weight_t);
-	auto*         op = static_cast<uint16_t*>(out);
+	if((K != 64 && K != 128) || N % 32 != 0 || N >= (1 << 20)) return AF3_ERR_BAD_ARGUMENT;
+	if((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(weight_t) & 15) || (reinterpret_cast<uintptr_t>(out) & 15)) return AF3_ERR_BAD_ARGUMENT;
+	const int64_t  col_tiles = N / 32;
+	const unsigned gy        = (unsigned)((col_tiles + GLU_MAX_WAVES - 1) / GLU_MAX_WAVES);
+	const int64_t  n_blocks  = (M + 31) / 32;
+	// persistent: one resident workgroup of sixteen wavefronts per compute unit
+	const int64_t  want = 256 / gy > 0 ? 256 / gy : 1;
+	const dim3     grid((unsigned)(n_blocks < want ? n_blocks : want), gy);
+	const auto     s  = static_cast<hipStream_t>(stream);
+	const auto*    xp = static_cast<const uint16_t*>(x);
+	const auto*    wp = static_cast<const uint16_t*>(weight_t);
+	auto*          op = static_cast<uint16_t*>(out);
 	if(K == 128)
-		hipLaunchKernelGGL(glu_kernel<8>, grid, dim3(threads), 0, s, xp, wp, op, M, N, n_waves);
+		hipLaunchKernelGGL(glu_kernel<8>, grid, dim3(GLU_MAX_WAVES * 64), 0, s, xp, wp, op, M, N);
 	else
-		hipLaunchKernelGGL(glu_kernel<4>, grid, dim3(threads), 0, s, xp, wp, op, M, N, n_waves);
+		hipLaunchKernelGGL(glu_kernel<4>, grid, dim3(GLU_MAX_WAVES * 64), 0, s, xp, wp, op, M, N);
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }

@@ -103,15 +103,45 @@ def _project(rows: torch.Tensor, ws, q_bias: Optional[torch.Tensor], head: int) 
 
 
 def _attend(y: torch.Tensor, B: int, N: int, head: int, mask, bias) -> torch.Tensor:
-    """Stage 2: the attention kernel on strided [B, head, N, K] views of stage 1's output (no "b n (h d) -> b h n d"
-    copies); sigmoid(gate) is applied in its epilogue and the result lands in "b n (h d)" order.  Returns [B, N, C]."""
+    """Stage 2: the attention kernel on q, k, v and the gate where stage 1 left them -- [B, head, N, K] views of y with
+    strides (N*4C, 4K, 4C, 1), no "b n (h d) -> b h n d" copies; sigmoid(gate) is applied in the kernel's epilogue and the
+    result lands in "b n (h d)" order.  The argument block is filled from y's address directly: building the four views
+    with tensor ops costs more host time than the kernel of a short sequence runs.  Returns [B, N, C]."""
     C = y.shape[1] // 4
     K = C // head
-    k, v, q, g = (y.view(B, N, head, 4, K)[:, :, :, i].permute(0, 2, 1, 3) for i in range(4))
+    if not y.is_contiguous():
+        y = y.contiguous()
     out = torch.empty(B, N, C, dtype=y.dtype, device=y.device)
+    if out.numel() == 0:
+        return out
     keep = ops._lift_mask(mask, N) if mask is not None else None
-    ops._dpa_forward_impl(q, k, v, keep, bias.to(y.dtype) if bias is not None else None, ops._DTYPE_CODE[y.dtype], False, gate=g,
-                          out=out.view(B, N, head, K).permute(0, 2, 1, 3))
+    if keep is not None and keep.shape[0] not in (1, B):
+        raise ValueError(f"mask must be [N] or [B, N] with B={B}, N={N}, got {tuple(mask.shape)}")
+    if bias is not None:
+        bias = ops._inner_contig(bias if bias.dtype == y.dtype else bias.to(y.dtype))
+        if bias.dim() != 3 or bias.shape[0] != head or bias.shape[1] < N or bias.shape[2] < N:
+            raise ValueError(f"bias must be [head, N, N] with head={head}, N={N}, got {tuple(bias.shape)}")
+    code, esz, base = ops._DTYPE_CODE[y.dtype], y.element_size(), y.data_ptr()
+    p = _lib.DpaParams()
+    p.k, p.v, p.q, p.gate = (base + i * K * esz for i in range(4))   # per token and head: (k | v | q | gate)
+    strides = (ctypes.c_int64 * 3)(N * 4 * C, 4 * K, 4 * C)
+    p.q_stride = p.k_stride = p.v_stride = p.gate_stride = strides
+    p.out, p.out_stride = out.data_ptr(), (ctypes.c_int64 * 3)(N * C, K, C)
+    p.B, p.H, p.L, p.D = B, head, N, K
+    if bias is not None:
+        p.bias, p.bias_stride, p.bias_dtype = bias.data_ptr(), (ctypes.c_int64 * 2)(bias.stride(0), bias.stride(1)), code
+    if keep is not None:
+        p.key_mask, p.key_mask_stride_b = keep.data_ptr(), (0 if keep.shape[0] == 1 else keep.stride(0))
+    p.io_dtype = p.out_dtype = p.mma_dtype = code
+    p.softmax_scale = float(K) ** -0.5
+    p.q_descale = p.k_descale = p.v_descale = 1.0
+    lib = _lib.load()
+    ws_bytes = lib.af3_dpa_workspace_bytes(ctypes.byref(p))
+    if ws_bytes > 0 and not ops._exact_bias:
+        scratch = torch.empty(ws_bytes, dtype=torch.uint8, device=y.device)
+        p.workspace, p.workspace_bytes = scratch.data_ptr(), ws_bytes
+    with ops._on_device(y.device):
+        _lib.check(lib.af3_dpa_forward(ctypes.byref(p), ops._stream_ptr(y.device)), "af3_dpa_forward")
     return out
 
 

@@ -355,3 +355,35 @@ def test_gated_linear_unit_other_shapes_and_linear_module(af3, oracle):
         lin(x)                                                             # CPU input: no CPU path
     with pytest.raises(ValueError):
         af3.gated_linear_unit_cpp(x.cuda(), torch.zeros(64, 512, dtype=torch.bfloat16, device="cuda"))   # K mismatch
+
+
+def test_fused_callers_match_the_golden_vectors(af3):
+    """The committed vectors (float64 numpy forms on bf16-representable inputs, tests/golden/make_golden.py) through the
+    drop-in functions: both routes of the grid op, the diffusion op, LayerNorm + pair bias, the gated linear unit."""
+    import os
+    from af3_kernels_amd import fused
+    gdir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    bf = lambda a: torch.from_numpy(a).to(torch.bfloat16).cuda()
+    g = np.load(os.path.join(gdir, "grid_attention_B3_N40_C128.npz"))
+    head = int(g["head"])
+    packed = [pack(af3, bf(g[n]), head) for n in ("wq", "wk", "wv", "wg")]
+    saved = fused._FUSED_MIN_GROUPS
+    try:
+        for min_groups in (1, 1 << 60):            # one kernel, then the three-launch composition
+            fused._FUSED_MIN_GROUPS = min_groups
+            out = af3._attention_cpp(bf(g["x"]), torch.from_numpy(g["mask"]).cuda(), bf(g["bias"]), *packed, bf(g["wo"]), head)
+            check(out, g["expected"], None, torch.bfloat16)
+    finally:
+        fused._FUSED_MIN_GROUPS = saved
+    g = np.load(os.path.join(gdir, "self_attention_N50_C96.npz"))
+    head = int(g["head"])
+    packed = [pack(af3, bf(g[n]), head) for n in ("wq", "wk", "wv", "wg")]
+    out = af3.self_attention_cpp(bf(g["x"]), torch.from_numpy(g["mask"]).cuda(), bf(g["bias"]), packed[0], bf(g["q_bias"]), packed[1], packed[2], packed[3], head)
+    check(out, g["expected"], None, torch.bfloat16)
+    g = np.load(os.path.join(gdir, "layernorm_pair_bias_6x9x128.npz"))
+    normed, bias = af3.layernorm_pair_bias(bf(g["pair"]), bf(g["gamma"]), bf(g["beta"]), float(g["eps"]), bf(g["wb"]))
+    assert np.abs(f32np(normed) - g["normed"]).max() <= 2.0 ** -7 * max(1.0, np.abs(g["normed"]).max())
+    assert np.abs(f32np(bias) - g["bias"]).max() <= 2e-2 * max(1.0, np.abs(g["bias"]).max())
+    g = np.load(os.path.join(gdir, "glu_70x128_N64.npz"))
+    out = af3.gated_linear_unit_cpp(bf(g["x"]), bf(g["weight"]))
+    assert np.abs(f32np(out) - g["expected"]).max() <= 2e-2 * max(1.0, np.abs(g["expected"]).max())

@@ -11,7 +11,7 @@ import pytest
 import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-GOLDEN = sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "*.npz")))
+GOLDEN = sorted(glob.glob(os.path.join(ROOT, "tests", "golden", "cfg*.npz")) + glob.glob(os.path.join(ROOT, "tests", "golden", "edge_*.npz")))   # the attention core's vectors
 
 
 @pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-4] for p in GOLDEN])
@@ -26,6 +26,23 @@ def test_oracle_reproduces_golden(oracle, path):
     keep = np.broadcast_to(g["mask"].reshape(-1, L), (B, L)) if g["mask"].ndim == 1 else g["mask"]
     rows = keep.any(1)
     assert np.abs(ref[rows] - g["expected"][rows]).max() < 2e-5
+
+
+def test_oracle_reproduces_the_fused_callers_golden_vectors(oracle):
+    """The C oracle against the vectors tests/golden/make_golden.py wrote from the independent float64 numpy forms
+    (oracle/dpa_numpy.py): grid and diffusion self-attention, LayerNorm + pair bias, gated linear unit."""
+    gdir = os.path.join(ROOT, "tests", "golden")
+    g = np.load(os.path.join(gdir, "grid_attention_B3_N40_C128.npz"))
+    got = oracle.fused_attention_formula(g["x"], g["mask"], g["bias"], g["wq"], g["wk"], g["wv"], g["wg"], g["wo"], None, head=int(g["head"]))
+    assert np.abs(got - g["expected"]).max() < 3e-6
+    g = np.load(os.path.join(gdir, "self_attention_N50_C96.npz"))
+    got = oracle.fused_attention_formula(g["x"], g["mask"], g["bias"], g["wq"], g["wk"], g["wv"], g["wg"], None, g["q_bias"], head=int(g["head"]))
+    assert got.shape == (50, 96) and np.abs(got - g["expected"]).max() < 3e-6
+    g = np.load(os.path.join(gdir, "layernorm_pair_bias_6x9x128.npz"))
+    normed, bias = oracle.layernorm_pair_bias(g["pair"], g["gamma"], g["beta"], g["wb"], float(g["eps"]))
+    assert np.abs(normed - g["normed"]).max() < 3e-6 and np.abs(bias - g["bias"]).max() < 3e-6
+    g = np.load(os.path.join(gdir, "glu_70x128_N64.npz"))
+    assert np.abs(oracle.gated_linear_unit(g["x"], g["weight"]) - g["expected"]).max() < 1e-5
 
 
 def test_golden_cfg1_is_the_named_case():

@@ -196,6 +196,8 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	unsigned char* const w_lds     = v_lds + n_ktiles * TILE_BYTES;  // FUSED only
 	const int            mask_base = FUSED ? 2 * n_ktiles * TILE_BYTES + 2 * NS * 1024 : MASK_BASE;
 	uint32_t* const      mask_tab  = reinterpret_cast<uint32_t*>(smem + mask_base);
+	// unfused variants with an output gate: the gate rows of each wavefront's query block, [32][DP] bf16, behind the tile list
+	const int            gate_base = (mask_base + (n_ktiles * KT + 64) * 4 + n_ktiles * 2 + 15) & ~15;
 	int16_t* const       live_list = reinterpret_cast<int16_t*>(mask_tab + n_ktiles * KT + 64);
 	__shared__ int       s_nvalid, s_nlive;
 
@@ -432,6 +434,23 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		// (scalar base + per-lane 16-byte offset + scalar tile offset: no 64-bit pointer in vector registers)
 		const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(ws_wave), 0, ws_wave ? n_ktiles * 4096 : 0, 0x00020000);
 		const int                    ws_voff = lane * 16;
+
+		// ---- output gate: fetched into LDS now, by loads that write LDS directly and hold no registers, and read in the
+		// epilogue.  (Loading it in the epilogue exposed a full memory latency per workgroup: 8 % of the kernel's time.)
+		// The first tile wait of the prologue below also covers these loads: they are older. ----
+		unsigned char* const gate_lds = smem + gate_base + (SPLIT ? 0 : wave * (32 * DP * 2));
+		if(!FUSED && p.gate && (!SPLIT || wave == 0)) {
+			const u32x4   g_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.gate) + b * p.gate_stride[0] + h * p.gate_stride[1], (uint32_t)(((L - 1) * p.gate_stride[2] + D) * 2));
+			constexpr int RPL    = 512 / DP;  // rows per 1 KB wave load
+			const int     g_row  = lane / CPR, g_c = lane % CPR;
+			const int64_t row0   = qrow - n;  // first row of this wavefront's block
+#pragma unroll
+			for(int t = 0; t < 32 / RPL; t++) {
+				const int64_t row  = row0 + t * RPL + g_row;
+				const int     voff = (g_c * 8 < D && row < L) ? (int)(row * p.gate_stride[2] * 2) + g_c * 16 : 0x7FFF0000;  // past the range: nothing is fetched
+				lds_dma_b128(g_rsrc, lds_addr_of(gate_lds) + t * 1024, voff);
+			}
+		}
 
 		// ---- K/V tile loader: buffer loads that write LDS directly ----
 		// One wave load moves 1 KB: lane i -> LDS chunk i of the load's 1 KB window, i.e. tile row
@@ -858,6 +877,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 			}
 		}
 
+		if(!FUSED && p.gate) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the gate rows; long since landed unless there was no tile at all)
 		// ---- epilogue: O^T register i of block db is head column 32*db + 8*(i/4) + 4*half + i%4 ----
 		// (8-byte stores, 16 bytes per row and instruction.  Turning the tile through LDS for 16-byte stores of whole 64-byte
 		// row segments was measured: 0.4 % faster in the fused variant, 1.5 % slower in the unfused ones, which spill at 128
@@ -878,8 +898,8 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 						const u32x2 gw = {gate_pk[g4 >> 1][2 * (g4 & 1)], gate_pk[g4 >> 1][2 * (g4 & 1) + 1]};
 						o0 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] & 0xffffu)), o1 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] >> 16));
 						o2 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] & 0xffffu)), o3 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] >> 16));
-					} else if(p.gate) {  // out *= sigmoid(gate): four consecutive head columns = one 8-byte load
-						const u32x2 gw = *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(p.gate) + b * p.gate_stride[0] + h * p.gate_stride[1] + qrow * p.gate_stride[2] + d0);
+					} else if(p.gate) {  // out *= sigmoid(gate): this row's four consecutive head columns, fetched into LDS at the start
+						const u32x2 gw = *reinterpret_cast<const u32x2*>(gate_lds + n * (DP * 2) + d0 * 2);
 						o0 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] & 0xffffu)), o1 *= sigmoidf_fast(bf16_bits_to_f32(gw[0] >> 16));
 						o2 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] & 0xffffu)), o3 *= sigmoidf_fast(bf16_bits_to_f32(gw[1] >> 16));
 					}
@@ -912,7 +932,7 @@ bool mfma_bf16_eligible(const af3_dpa_params& p) {
 		if(p.q_stride[i] % 8 || p.k_stride[i] % 8 || p.v_stride[i] % 8) return false;
 	// buffer addressing of one (batch, head) slab uses 32-bit byte offsets
 	if(p.L * p.k_stride[2] * 2 >= 0x7fffffffLL || p.L * p.v_stride[2] * 2 >= 0x7fffffffLL) return false;
-	if(p.gate && ((reinterpret_cast<uintptr_t>(p.gate) & 7) || p.gate_stride[0] % 4 || p.gate_stride[1] % 4 || p.gate_stride[2] % 4)) return false;
+	if(p.gate && (!aligned16(p.gate) || p.gate_stride[0] % 8 || p.gate_stride[1] % 8 || p.gate_stride[2] % 8 || p.L * p.gate_stride[2] * 2 >= 0x7fffffffLL)) return false;
 	if(p.out_dtype == AF3_BF16) {
 		if((reinterpret_cast<uintptr_t>(p.out) & 7) || p.out_stride[0] % 4 || p.out_stride[1] % 4 || p.out_stride[2] % 4) return false;
 	} else {
@@ -948,6 +968,15 @@ static int launch_bias_prepass(const af3_dpa_params& p, hipStream_t s) {
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
 }
 
+constexpr size_t LDS_LIMIT = 160 * 1024;  // per workgroup on gfx950
+
+// dynamic LDS of one variant: K/V buffers, bias ring, mask table, tile list, gate rows of every wavefront that writes results
+template <int DP, int NW, int BMODE, bool SPLIT>
+static size_t lds_bytes(const af3_dpa_params& p) {
+	const size_t n_ktiles = (size_t)((p.L + KT - 1) / KT);
+	return (size_t)(SPLIT ? NW : 1) * 6 * KT * DP * 2 + (BMODE == 2 ? NW * 3 * 4096 : 0) + (n_ktiles * KT + 64) * 4 + n_ktiles * 2 + 16 + (p.gate ? (size_t)(SPLIT ? 1 : NW) * 32 * DP * 2 : 0);
+}
+
 template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT = false>
 static int launch_one(const af3_dpa_params& p, hipStream_t s) {
 	constexpr int QT       = SPLIT ? 32 : NW * 32;
@@ -956,7 +985,8 @@ static int launch_one(const af3_dpa_params& p, hipStream_t s) {
 	const int64_t n_groups = p.B * p.H;
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
-	const size_t smem = (size_t)(SPLIT ? NW : 1) * 6 * KT * DP * 2 + (BMODE == 2 ? NW * 3 * 4096 : 0) + ((size_t)n_ktiles * KT + 64) * 4 + (size_t)n_ktiles * 2 + 16;
+	const size_t smem = lds_bytes<DP, NW, BMODE, SPLIT>(p);
+	if(smem > LDS_LIMIT) return AF3_ERR_BAD_SHAPE;  // (launch_nw only picks variants that fit)
 	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BMODE, SPLIT, false>;
 	if(smem > 64 * 1024) {  // beyond the default dynamic-LDS limit: raise it for this kernel (idempotent, host side)
 		if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
@@ -1047,12 +1077,13 @@ static int launch_nw(const af3_dpa_params& p, hipStream_t s) {
 		// share each K/V tile instead (measured, B=1 H=16 D=24: L=1536 25.6 us against 32.7 us with
 		// single-wave workgroups; L=768 14.0 us split in two against 14.3 / 17.8; L=384 8.5 us split in four).
 		if(blocks1 >= 512) return launch_one<DP, 4, L2DOM, BMODE>(p, s);
-		if(DP == 32 && ktiles >= 4 && blocks1 <= 256) return launch_one<DP, 4, L2DOM, BMODE, true>(p, s);
-		if(ktiles >= 2) return launch_one<DP, 2, L2DOM, BMODE, true>(p, s);
+		// (the split variants' private buffers plus a long row's mask table can exceed the LDS of a compute unit: then the next one)
+		if(DP == 32 && ktiles >= 4 && blocks1 <= 256 && lds_bytes<DP, 4, BMODE, true>(p) <= LDS_LIMIT) return launch_one<DP, 4, L2DOM, BMODE, true>(p, s);
+		if(ktiles >= 2 && lds_bytes<DP, 2, BMODE, true>(p) <= LDS_LIMIT) return launch_one<DP, 2, L2DOM, BMODE, true>(p, s);
 		return launch_one<DP, 1, L2DOM, BMODE>(p, s);
 	}
-	if(DP == 32 && ktiles >= 4 && blocks1 <= 256) return launch_one<DP, 4, L2DOM, BMODE, true>(p, s);
-	if(ktiles >= 2 && blocks1 <= 768) return launch_one<DP, 2, L2DOM, BMODE, true>(p, s);
+	if(DP == 32 && ktiles >= 4 && blocks1 <= 256 && lds_bytes<DP, 4, BMODE, true>(p) <= LDS_LIMIT) return launch_one<DP, 4, L2DOM, BMODE, true>(p, s);
+	if(ktiles >= 2 && blocks1 <= 768 && lds_bytes<DP, 2, BMODE, true>(p) <= LDS_LIMIT) return launch_one<DP, 2, L2DOM, BMODE, true>(p, s);
 	return launch_one<DP, 1, L2DOM, BMODE>(p, s);
 }
 

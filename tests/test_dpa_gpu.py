@@ -140,6 +140,13 @@ def test_small_grids_split_keys_over_wavefronts(af3, oracle, B, H, L, D, live):
     assert np.abs(f32np(out) - want).max() <= TOL[torch.bfloat16]
 
 
+def test_long_rows_with_few_heads_pick_a_variant_that_fits_in_lds(af3, oracle):
+    """B*H = 1 with L = 5000: the four-wave key split with the bias ring would need more LDS than a compute unit has
+    (private K/V buffers + ring + a 20 KB mask table); the launcher must pick the next variant instead of failing."""
+    q, k, v, m, bias = rand_inputs(1, 1, 5000, 32, torch.bfloat16, seed=77)
+    run_case(af3, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+
+
 def test_bf16_mfma_and_fp32_fma_kernels_agree(af3):
     q, k, v, m, bias = dev(*rand_inputs(2, 4, 200, 32, torch.bfloat16, seed=5, mask="random"))
     a = af3.dot_product_attention_cpp(q, k, v, m, bias)

@@ -168,7 +168,7 @@ template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT, bool FUSED>
 // (at least 2 wavefronts per SIMD: keeps the register budget at 256 so that the compiler writes MFMA
 // results to ordinary VGPRs instead of AGPRs, which every softmax operand would have to be copied out of;
 // the key-split variants are limited to fewer than 2 wavefronts per SIMD by their LDS buffers anyway)
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FUSED ? (NW + 3) / 4 : DP == 32 && !SPLIT ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups, fused_grid_args fa) {
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FUSED ? (NW <= 4 ? 3 : (NW + 3) / 4) : DP == 32 && !SPLIT ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups, fused_grid_args fa) {
 	constexpr int NC         = DP / 16;            // contraction chunks of QK^T
 	constexpr int NDB        = DP / 32;            // 32-row blocks of O^T
 	constexpr int CPR        = DP / 8;             // 16-byte chunks per K/V row
@@ -1057,6 +1057,9 @@ int launch_grid_fused(const af3_grid_attention_params& g, hipStream_t s) {
 	// wavefronts per workgroup: 12 (three per SIMD) unless 8 leaves fewer of them idle in the last round of query blocks
 	const int n_qblocks = (int)((p.L + 31) / 32);
 	const int best      = ((n_qblocks + 7) / 8) * 8 < ((n_qblocks + 11) / 12) * 12 ? 8 : 12;
+	// short rows: three 4-wave workgroups per compute unit instead of one large one, so that one workgroup's projection of
+	// K and V overlaps the others' attention (measured at N = 256: 41.6 against 47.4 us)
+	if(fused_lds_bytes(p.L) * 3 <= (size_t)FUSED_LDS_LIMIT && n_qblocks % 4 == 0) return launch_fused_nw<4>(p, fa, s);
 	return best == 12 ? launch_fused_nw<12>(p, fa, s) : launch_fused_nw<8>(p, fa, s);
 }
 

@@ -118,6 +118,7 @@ def run_grid_case(af3, oracle, B, N, C, head, dtype, one_kernel, mask_p=0.85, bi
 ONE_KERNEL_CASES = [
     # B, N: 128 channels, 4 heads, bfloat16
     (4, 72), (9, 200), (3, 37), (2, 384), (1, 768), (5, 64), (2, 1000), (3, 33), (2, 1),
+    (3, 256), (2, 128), (2, 250),      # short rows: 4-wave workgroups, three per compute unit
 ]
 
 

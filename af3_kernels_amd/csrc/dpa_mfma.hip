@@ -312,6 +312,10 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	};
 	const int n_qblocks_all = (int)((L + 31) / 32);
 	int       qb_f          = 0;  // FUSED: the query block this wavefront works on
+	// FUSED: q and gate of the block this wavefront takes second, projected while its rows of x were in registers for K and V
+	[[maybe_unused]] bf16x8 q_next[NC];
+	[[maybe_unused]] u32x4  gate_next[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
+	[[maybe_unused]] int    qb_next      = -1;  // which block q_next / gate_next belong to
 	if constexpr(FUSED) {
 		x_rsrc      = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(fa.x + b * fa.x_stride_b), 0, (int)(((L - 1) * fa.x_stride_n + 16 * NS) * 2), 0x00020000);
 		x_row_bytes = (int)(fa.x_stride_n * 2);
@@ -339,8 +343,12 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 			wkf[st] = u32x4{wk32[(8 * st) * 32], wk32[(8 * st + 1) * 32], wk32[(8 * st + 2) * 32], wk32[(8 * st + 3) * 32]};
 			wvf[st] = u32x4{wv32[(8 * st) * 32], wv32[(8 * st + 1) * 32], wv32[(8 * st + 2) * 32], wv32[(8 * st + 3) * 32]};
 		}
-		u32x4 xf[NS];
-		int   sb_last = -1;
+		// This wavefront's query blocks are walked from the last one down: its rows of x are the ones used last here (unless
+		// the last key block was padding past L), so q and the gate of that block come for free; those of the block before it
+		// are projected when its rows pass by and kept in registers until its turn.
+		const int qb_last = n_qblocks_all - 1 - (n_qblocks_all - 1 - wave + NW * 64) % NW;  // largest block index congruent to wave (negative: none)
+		u32x4     xf[NS];
+		int       sb_last = -1;
 		for(int sb = wave; sb < 2 * n_ktiles; sb += NW) {
 			const int key = sb * 32 + n;
 			load_x_frags(key, xf);
@@ -360,11 +368,16 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 				*reinterpret_cast<u32x2*>(kdst + ((j ^ swz) << 4)) = u32x2{pack_bf16x2(ak[4 * j], ak[4 * j + 1]), pack_bf16x2(ak[4 * j + 2], ak[4 * j + 3])};
 				*reinterpret_cast<u32x2*>(vdst + (j << 4))         = u32x2{pack_bf16x2(av[4 * j], av[4 * j + 1]), pack_bf16x2(av[4 * j + 2], av[4 * j + 3])};
 			}
+			if(sb == qb_last - NW) {
+				project_q_gate(xf);
+#pragma unroll
+				for(int c = 0; c < NC; c++) q_next[c] = qf[c];
+				gate_next[0] = gate_pk[0], gate_next[1] = gate_pk[1];
+				qb_next = sb;
+			}
 			sb_last = sb;
 		}
-		// This wavefront's query blocks are walked from the last one down: its rows of x are the ones just used
-		// (unless the last key block was padding past L), so q and the gate of that block come for free.
-		qb_f = n_qblocks_all - 1 - (n_qblocks_all - 1 - wave + NW * 64) % NW;  // largest block index congruent to wave (negative: none)
+		qb_f = qb_last;
 		if(qb_f >= 0) {
 			if(sb_last != qb_f) load_x_frags(qb_f * 32 + n, xf);
 			project_q_gate(xf);
@@ -913,7 +926,11 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 				}
 		}
 		if constexpr(FUSED) {  // q and gate of this wavefront's next block
-			if(qb_f - NW >= 0) {
+			if(qb_f - NW == qb_next) {  // (wave-uniform) already projected
+#pragma unroll
+				for(int c = 0; c < NC; c++) qf[c] = q_next[c];
+				gate_pk[0] = gate_next[0], gate_pk[1] = gate_next[1];
+			} else if(qb_f - NW >= 0) {
 				u32x4 xf[NS];
 				load_x_frags((qb_f - NW) * 32 + n, xf);
 				project_q_gate(xf);

@@ -998,7 +998,6 @@ template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT = false>
 static int launch_one(const af3_dpa_params& p, hipStream_t s) {
 	constexpr int QT       = SPLIT ? 32 : NW * 32;
 	const int     n_qtiles = (int)((p.L + QT - 1) / QT);
-	const int     n_ktiles = (int)((p.L + KT - 1) / KT);
 	const int64_t n_groups = p.B * p.H;
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;

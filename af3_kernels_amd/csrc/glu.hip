@@ -33,45 +33,68 @@ namespace {
 
 constexpr int GLU_MAX_WAVES = 16;
 
-template <int KS>  // contraction steps of 16 channels: K = 16 * KS
-__global__ void __launch_bounds__(GLU_MAX_WAVES * 64) glu_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ wt, uint16_t* __restrict__ out, int64_t M, int64_t N) {
+// KS: contraction steps of 16 channels (K = 16 * KS).  WAVES: wavefronts per workgroup = 32-column tiles it owns.
+// GATED: out = silu(x . Wa) * (x . Wb) with wt = [Wa | Wb]^T; otherwise the plain product out = x . W with wt = W^T.
+template <int KS, int WAVES, bool GATED>
+// (four wavefronts per SIMD whatever the workgroup size: 128 registers each)
+__global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4))) glu_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ wt, uint16_t* __restrict__ out, int64_t M, int64_t N) {
 	constexpr int K          = 16 * KS;
 	constexpr int ROW_BYTES  = K * 2;
 	constexpr int TILE_BYTES = 32 * ROW_BYTES;
-	constexpr int TPB        = TILE_BYTES / (GLU_MAX_WAVES * 64);  // bytes of a block per thread: 8 (K = 128) or 4 (K = 64)
+	constexpr int TPB        = TILE_BYTES / (WAVES * 64);  // bytes of a block per thread: 4 .. 32
+	constexpr int PIECE      = TPB < 16 ? TPB : 16;         // moved in pieces of at most 16 bytes
+	constexpr int PPT        = TPB / PIECE;
 	constexpr int OUT_STRIDE = 80;  // bytes per row of the output patch: 64 of data, padded so that rows start in different banks
+	static_assert(TILE_BYTES % (WAVES * 64) == 0 && TPB >= 4 && TPB % PIECE == 0, "every thread moves whole pieces of a block");
 	__shared__ __attribute__((aligned(16))) unsigned char xs[2][TILE_BYTES];
-	__shared__ __attribute__((aligned(16))) unsigned char os[GLU_MAX_WAVES][32 * OUT_STRIDE];
+	__shared__ __attribute__((aligned(16))) unsigned char os[WAVES][32 * OUT_STRIDE];
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int n = lane & 31, half = lane >> 5;
-	const int64_t col0   = ((int64_t)blockIdx.y * GLU_MAX_WAVES + wave) * 32;  // first gate column of this wavefront
+	const int64_t col0   = ((int64_t)blockIdx.y * WAVES + wave) * 32;  // first (gate) column of this wavefront
 	const bool    active = col0 < N;  // wavefronts past the last column only help to move x
 
-	// weight fragments (A operand): lane (column n, g = half), step s: W^T[col][16s + 8g .. +7]; wt is [2N, K] row-major
-	u32x4 wa[KS], wb[KS];
+	// weight fragments (A operand): lane (column n, g = half), step s: W^T[col][16s + 8g .. +7]; wt is [2N, K] ([N, K]) row-major
+	u32x4 wa[KS], wb[GATED ? KS : 1];
 #pragma unroll
 	for(int s = 0; s < KS; s++) {
-		wa[s] = wb[s] = u32x4{0u, 0u, 0u, 0u};
+		wa[s] = u32x4{0u, 0u, 0u, 0u};
+		if(GATED) wb[s] = u32x4{0u, 0u, 0u, 0u};
 		if(active) {
 			wa[s] = *reinterpret_cast<const u32x4*>(wt + (col0 + n) * K + 16 * s + 8 * half);
-			wb[s] = *reinterpret_cast<const u32x4*>(wt + (N + col0 + n) * K + 16 * s + 8 * half);
+			if(GATED) wb[s] = *reinterpret_cast<const u32x4*>(wt + (N + col0 + n) * K + 16 * s + 8 * half);
 		}
 	}
 
 	const int64_t n_blocks = (M + 31) / 32;
 	auto rows_in = [&](int64_t blk) -> int { return (int)(M - blk * 32 < 32 ? M - blk * 32 : 32); };
-	// x block mover: thread t moves bytes [TPB*t, TPB*t + TPB) of the block.  In LDS the 16-byte chunk index of a row is
-	// XOR-swizzled with the row so that the operand reads below (same chunk, consecutive rows) spread over the banks.
-	typedef typename std::conditional<TPB == 8, u32x2, uint32_t>::type piece_t;
-	const int ld_off = tid * TPB;
-	const int ld_row = ld_off / ROW_BYTES, ld_col = ld_off % ROW_BYTES;
-	const int ld_dst = ld_row * ROW_BYTES + (((ld_col >> 4) ^ (ld_row & 7)) << 4) + (ld_col & 15);
-	auto fetch = [&](int64_t blk) -> piece_t {
+	// x block mover: thread t moves bytes [TPB*t, TPB*t + TPB) of the block, in pieces of at most 16 bytes.  In LDS the 16-byte
+	// chunk index of a row is XOR-swizzled with the row so that the operand reads below (same chunk, consecutive rows) spread
+	// over the banks.
+	typedef typename std::conditional<PIECE == 16, u32x4, typename std::conditional<PIECE == 8, u32x2, uint32_t>::type>::type piece_t;
+	struct staged_t {
+		piece_t v[PPT];
+	};
+	auto lds_pos = [&](int off) -> int {
+		const int r = off / ROW_BYTES, c = off % ROW_BYTES;
+		return r * ROW_BYTES + (((c >> 4) ^ (r & 7)) << 4) + (c & 15);
+	};
+	auto fetch = [&](int64_t blk) -> staged_t {
 		const __amdgpu_buffer_rsrc_t r =
 			__builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(reinterpret_cast<const unsigned char*>(x)) + blk * TILE_BYTES, 0, rows_in(blk) * ROW_BYTES, 0x00020000);
-		if constexpr(TPB == 8) return __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, ld_off, 0, 0));
-		else return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, ld_off, 0, 0);
+		staged_t st;
+#pragma unroll
+		for(int i = 0; i < PPT; i++) {
+			const int off = tid * TPB + i * PIECE;
+			if constexpr(PIECE == 16) st.v[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0));
+			else if constexpr(PIECE == 8) st.v[i] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0));
+			else st.v[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0);
+		}
+		return st;
+	};
+	auto publish = [&](int buf, const staged_t& st) {
+#pragma unroll
+		for(int i = 0; i < PPT; i++) *reinterpret_cast<piece_t*>(xs[buf] + lds_pos(tid * TPB + i * PIECE)) = st.v[i];
 	};
 	// operand reads (lane = row n, chunk 2s + half, swizzled) and the output patch
 	const int            x_rd  = n * ROW_BYTES;
@@ -83,8 +106,8 @@ __global__ void __launch_bounds__(GLU_MAX_WAVES * 64) glu_kernel(const uint16_t*
 
 	int64_t blk = blockIdx.x;
 	if(blk >= n_blocks) return;  // (whole workgroup)
-	piece_t staged = fetch(blk);
-	*reinterpret_cast<piece_t*>(xs[0] + ld_dst) = staged;
+	staged_t staged = fetch(blk);
+	publish(0, staged);
 	__syncthreads();
 	int   buf = 0;
 	u32x4 sv[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};  // the data of the two stores of a block
@@ -100,7 +123,7 @@ __global__ void __launch_bounds__(GLU_MAX_WAVES * 64) glu_kernel(const uint16_t*
 		for(int s = 0; s < KS; s++) {
 			const u32x4 xf = *reinterpret_cast<const u32x4*>(xb + (((2 * s + half) ^ sw) << 4));
 			ga = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wa[s]), __builtin_bit_cast(bf16x8, xf), ga, 0, 0, 0);
-			va = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wb[s]), __builtin_bit_cast(bf16x8, xf), va, 0, 0, 0);
+			if(GATED) va = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wb[s]), __builtin_bit_cast(bf16x8, xf), va, 0, 0, 0);
 		}
 		// silu(a) * b, rounded to bf16, into this wavefront's patch: lane (row n, half) owns columns 8*g4 + 4*half .. +3
 #pragma unroll
@@ -109,7 +132,7 @@ __global__ void __launch_bounds__(GLU_MAX_WAVES * 64) glu_kernel(const uint16_t*
 #pragma unroll
 			for(int r = 0; r < 4; r++) {
 				const float a = ga[4 * g4 + r];
-				o[r] = a * va[4 * g4 + r] * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-a * LOG2E));
+				o[r] = GATED ? a * va[4 * g4 + r] * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-a * LOG2E)) : a;
 			}
 			*reinterpret_cast<u32x2*>(patch + p_wr + g4 * 16) = u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
 		}
@@ -125,7 +148,7 @@ __global__ void __launch_bounds__(GLU_MAX_WAVES * 64) glu_kernel(const uint16_t*
 		__builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(store_t, sv[0]), orsrc, o_off, 0, 0);
 		__builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(store_t, sv[1]), orsrc, o_off + (int)(16 * N * 2), 0, 0);
 		// publish the next block (its LDS buffer was last read before the previous barrier)
-		*reinterpret_cast<piece_t*>(xs[buf ^ 1] + ld_dst) = staged;
+		publish(buf ^ 1, staged);
 		__syncthreads();
 		buf ^= 1;
 	}
@@ -137,25 +160,43 @@ __global__ void __launch_bounds__(GLU_MAX_WAVES * 64) glu_kernel(const uint16_t*
 
 using namespace af3;
 
-extern "C" int af3_gated_linear_unit(const void* x, const void* weight_t, void* out, int64_t M, int64_t K, int64_t N, int32_t dtype, void* stream) {
+namespace {
+
+// out[M, N] = x[M, K] . wt^T (GATED: silu(x . Wa) * (x . Wb), wt = [Wa | Wb]^T) -- checks shared by both entry points
+int launch_rows_times_weights(const void* x, const void* weight_t, void* out, int64_t M, int64_t K, int64_t N, int32_t dtype, bool gated, void* stream) {
 	if(!x || !weight_t || !out) return AF3_ERR_NULL_POINTER;
 	if(M <= 0 || N <= 0 || K <= 0 || M > ((int64_t)1 << 40)) return AF3_ERR_BAD_SHAPE;
 	if(dtype != AF3_BF16) return AF3_ERR_BAD_DTYPE;
 	if((K != 64 && K != 128) || N % 32 != 0 || N >= (1 << 20)) return AF3_ERR_BAD_ARGUMENT;
 	if((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(weight_t) & 15) || (reinterpret_cast<uintptr_t>(out) & 15)) return AF3_ERR_BAD_ARGUMENT;
-	const int64_t  col_tiles = N / 32;
-	const unsigned gy        = (unsigned)((col_tiles + GLU_MAX_WAVES - 1) / GLU_MAX_WAVES);
-	const int64_t  n_blocks  = (M + 31) / 32;
-	// persistent: one resident workgroup of sixteen wavefronts per compute unit
-	const int64_t  want = 256 / gy > 0 ? 256 / gy : 1;
-	const dim3     grid((unsigned)(n_blocks < want ? n_blocks : want), gy);
-	const auto     s  = static_cast<hipStream_t>(stream);
-	const auto*    xp = static_cast<const uint16_t*>(x);
-	const auto*    wp = static_cast<const uint16_t*>(weight_t);
-	auto*          op = static_cast<uint16_t*>(out);
-	if(K == 128)
-		hipLaunchKernelGGL(glu_kernel<8>, grid, dim3(GLU_MAX_WAVES * 64), 0, s, xp, wp, op, M, N);
-	else
-		hipLaunchKernelGGL(glu_kernel<4>, grid, dim3(GLU_MAX_WAVES * 64), 0, s, xp, wp, op, M, N);
+	const int64_t col_tiles = N / 32;
+	const int64_t n_blocks  = (M + 31) / 32;
+	const auto    s  = static_cast<hipStream_t>(stream);
+	const auto*   xp = static_cast<const uint16_t*>(x);
+	const auto*   wp = static_cast<const uint16_t*>(weight_t);
+	auto*         op = static_cast<uint16_t*>(out);
+	// persistent workgroups: about sixteen resident wavefronts per compute unit
+	auto go = [&](auto kern, int waves) {
+		const unsigned gy   = (unsigned)((col_tiles + waves - 1) / waves);
+		const int64_t  want = (int64_t)256 * (GLU_MAX_WAVES / waves) / gy > 0 ? (int64_t)256 * (GLU_MAX_WAVES / waves) / gy : 1;
+		hipLaunchKernelGGL(kern, dim3((unsigned)(n_blocks < want ? n_blocks : want), gy), dim3(waves * 64), 0, s, xp, wp, op, M, N);
+	};
+	if(col_tiles <= 4 && !gated) {  // narrow plain products (the attention blocks' output projection): 4-wave workgroups, four per compute unit
+		if(K == 128) go(glu_kernel<8, 4, false>, 4);
+		else go(glu_kernel<4, 4, false>, 4);
+	} else {
+		if(K == 128) gated ? go(glu_kernel<8, GLU_MAX_WAVES, true>, GLU_MAX_WAVES) : go(glu_kernel<8, GLU_MAX_WAVES, false>, GLU_MAX_WAVES);
+		else gated ? go(glu_kernel<4, GLU_MAX_WAVES, true>, GLU_MAX_WAVES) : go(glu_kernel<4, GLU_MAX_WAVES, false>, GLU_MAX_WAVES);
+	}
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+}
+
+}  // namespace
+
+extern "C" int af3_gated_linear_unit(const void* x, const void* weight_t, void* out, int64_t M, int64_t K, int64_t N, int32_t dtype, void* stream) {
+	return launch_rows_times_weights(x, weight_t, out, M, K, N, dtype, true, stream);
+}
+
+extern "C" int af3_linear(const void* x, const void* weight, void* out, int64_t M, int64_t K, int64_t N, int32_t dtype, void* stream) {
+	return launch_rows_times_weights(x, weight, out, M, K, N, dtype, false, stream);
 }

@@ -7,7 +7,7 @@ and the module that wraps the first one, GridSelfAttentionCpp (src/af3_kernels/A
 
 On the GPU the grid op in AlphaFold 3's shape (bfloat16, 128 channels, 4 heads) is ONE kernel for the projections,
 the attention and the gate (af3_grid_attention_forward: q, k, v and the gate never touch device memory) followed by
-the output projection GEMM.  Every other shape, and the diffusion op, is three launches:
+the output projection (af3_linear).  Every other shape, and the diffusion op, is three launches:
   1. ONE library GEMM for the four projections: x [rows, C] . W [C, 4C], output columns ordered
      (head, [k, v, q, gate], channel)  (hipBLASLt through torch: a plain GEMM is library territory);
   2. the attention kernel, reading q, k, v as strided views of that GEMM's output (no
@@ -214,7 +214,11 @@ def _attention_cpp(
     gated = _fused_grid_kernel(pair, mask, bias, ws, head) if B * head >= _FUSED_MIN_GROUPS else None
     if gated is None:
         gated = _attend(_project(pair.reshape(B * N, C), ws, None, head), B, N, head, mask, bias)
-    return torch.matmul(gated.view(B * N, C), out_proj.to(dtype)).view(B, N, C)
+    rows = gated.view(B * N, C)
+    if out_proj.dtype == dtype and _narrow_linear_ok(rows, C):
+        w = _cached((out_proj,), ("out_proj",), lambda: out_proj.t().contiguous())      # nn.Linear layout [out, in]
+        return _linear_rows(rows, w).view(B, N, C)
+    return torch.matmul(rows, out_proj.to(dtype)).view(B, N, C)
 
 
 def self_attention_cpp(
@@ -313,6 +317,21 @@ class GridSelfAttentionCpp(torch.nn.Module):
         return out.transpose(0, 1) if self.transpose else out
 
 
+def _narrow_linear_ok(x2: torch.Tensor, n_out: int) -> bool:
+    """Shapes for which af3_linear beats the library GEMM (measured): bfloat16, 64 or 128 input channels, at most 128 outputs."""
+    return (x2.dtype == torch.bfloat16 and x2.shape[1] in (64, 128) and n_out % 32 == 0 and n_out <= 128 and x2.shape[0] > 0 and x2.is_contiguous()
+            and x2.data_ptr() % 16 == 0)
+
+
+def _linear_rows(x2: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """x2 [M, K] . weight^T for weight [N, K] (nn.Linear layout) through af3_linear; the caller has checked the shape limits."""
+    out = torch.empty(x2.shape[0], weight.shape[0], dtype=x2.dtype, device=x2.device)
+    with ops._on_device(x2.device):
+        _lib.check(_lib.load().af3_linear(x2.data_ptr(), weight.data_ptr(), out.data_ptr(), x2.shape[0], x2.shape[1], weight.shape[0], ops._DTYPE_CODE[x2.dtype],
+                                          ops._stream_ptr(x2.device)), "af3_linear")
+    return out
+
+
 def _plain_weight(weight: torch.Tensor, vnni_repacked: bool, N_BLK: int) -> torch.Tensor:
     """[K, N] weight as the reference's callers hand it over -- plain, or VNNI panels of width N_BLK
     (vnni_repack_tensor(W, 2, N_BLK): [N/N_BLK][K/2][N_BLK][2]) -- back to plain [K, N]."""
@@ -353,7 +372,8 @@ def gated_linear_unit_cpp(x: torch.Tensor, weight: torch.Tensor, vnni_repacked: 
 
 class Linear(torch.nn.Module):
     """Bias-free linear layer with the reference's constructor (src/af3_kernels/__init__.py:138-163).  The reference repacks
-    the weight into VNNI panels for its CPU GEMM; here the product is a library GEMM (hipBLASLt) on the plain weight."""
+    the weight into VNNI panels for its CPU GEMM; here the product runs on the plain weight: af3_linear for narrow layers
+    (64 or 128 inputs, at most 128 outputs, bfloat16), a library GEMM (hipBLASLt) otherwise."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None, M_BLK: int = 128, N_BLK: int = 128) -> None:
         super().__init__()
@@ -365,4 +385,7 @@ class Linear(torch.nn.Module):
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         ops._require_device(input, self.weight)
+        x2 = input.reshape(-1, self.in_features)
+        if self.weight.dtype == input.dtype and self.weight.is_contiguous() and _narrow_linear_ok(x2, self.out_features):
+            return _linear_rows(x2, self.weight).view(*input.shape[:-1], self.out_features)
         return torch.nn.functional.linear(input, self.weight)

@@ -260,6 +260,16 @@ int af3_layernorm_pair_bias(const void* pair, const int64_t* pair_stride, const 
 int af3_gated_linear_unit(const void* x, const void* weight_t, void* out, int64_t M, int64_t K, int64_t N, int32_t dtype, void* hip_stream);
 
 /*
+ * Bias-free linear layer for narrow contractions: out[M, N] = x[M, K] . weight^T with weight in nn.Linear layout
+ * [N, K] -- the same kernel as af3_gated_linear_unit without the gate (rows of x through LDS once, weight fragments in
+ * registers, 16-byte stores).
+ * Replaces: at::Tensor linear(input, weight, M_BLK, N_BLK) -- src/csrc/gated_linear_unit.cpp:82-129, :140-147 (the reference
+ * takes the weight^T VNNI-repacked) -- and the closing output projection of _attention_impl (dot_product_attention.cpp:364-371).
+ * Supported: dtype AF3_BF16, K == 64 or 128, N % 32 == 0, 16-byte aligned pointers; AF3_ERR_BAD_ARGUMENT otherwise.
+ */
+int af3_linear(const void* x, const void* weight, void* out, int64_t M, int64_t K, int64_t N, int32_t dtype, void* hip_stream);
+
+/*
  * N-dimensional pad (ndim <= AF3_PAD_MAX_DIMS): copy src (shape src_shape, element strides
  * src_strides) into the low corner of a contiguous dst of shape dst_shape (>= src_shape in
  * every axis) and fill the rest with the 32-bit pattern `fill_bits` truncated to elem_size

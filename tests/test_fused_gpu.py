@@ -345,6 +345,16 @@ def test_gated_linear_unit_other_shapes_and_linear_module(af3, oracle):
         out = af3.gated_linear_unit_cpp(x.cuda(), w.cuda())
         want = oracle.gated_linear_unit(f32np(x), f32np(w))
         assert np.abs(f32np(out) - want).max() <= tol * max(1.0, float(np.abs(want).max()))
+    for n_out in (128, 64):                                                # narrow layers run af3_linear, bit-identical to the library GEMM here
+        g2 = torch.Generator().manual_seed(n_out)
+        lin = af3.Linear(128, n_out, False, dtype=torch.bfloat16).cuda()
+        with torch.no_grad():
+            lin.weight.copy_((torch.randn(n_out, 128, generator=g2) / 128 ** 0.5).to(torch.bfloat16))
+            x = torch.randn(5, 77, 128, generator=g2).to(torch.bfloat16)
+            y = lin(x.cuda())
+        want = f32np(x).astype(np.float64) @ f32np(lin.weight).astype(np.float64).T
+        assert y.shape == (5, 77, n_out) and np.abs(f32np(y) - want).max() <= 2e-2 * max(1.0, np.abs(want).max())
+        assert torch.equal(y, torch.nn.functional.linear(x.cuda(), lin.weight))
     lin = af3.Linear(128, 512, False, dtype=torch.bfloat16, M_BLK=128, N_BLK=128).cuda()
     with torch.no_grad():
         lin.weight.copy_((torch.randn(512, 128, generator=g) / 128 ** 0.5).to(torch.bfloat16))

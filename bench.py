@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0
 # WRITE_SIZE, KiB per dispatch) scaled by what the same counters read for a 256 MiB device copy
 # (FETCH x2.0, WRITE x1.0); the runs are summarised in profiles/dpa_mfma_bf16_cfg4_hbm_traffic.txt.
 # Counters cannot be read from inside this script, so workloads without such a run report null.
-MEASURED_TRAFFIC_BYTES = {"cfg4": 648.3e6, "grid_n768": 786.6e6}   # grid_n768: profiles/grid_attention_one_kernel_grid_n768_kernel_trace.txt
+MEASURED_TRAFFIC_BYTES = {"cfg4": 648.3e6, "grid_n768": 687.1e6}   # grid_n768: profiles/grid_attention_one_kernel_grid_n768_kernel_trace.txt
 
 
 def cpu_baseline(case, budget_s=12.0):

@@ -203,7 +203,7 @@ int af3_quantize_qkv_fp8_e4m3(const void* q, const void* k, const void* v, int32
  * Replaces: _attention_impl<bfloat16> without its closing output projection -- src/csrc/dot_product_attention.cpp:
  * 200-362 (projections :286-345, logits / bias / mask / softmax :313-333, weighted average :346-352, sigmoid gate
  * :334-361), bound as `_attention` at src/csrc/init.cpp.  The output projection (:364-371) is a plain [B*N, C] x
- * [C, C] matrix product on the result and is left to the caller's BLAS.
+ * [C, C] matrix product on the result: af3_linear below, or the caller's BLAS.
  * Supported (af3_grid_attention_supported() == 1): dtype AF3_BF16, C == 128, head == 4, N small enough for K and V
  * of one head to stay in LDS (N <= 1024); anything else returns AF3_ERR_BAD_ARGUMENT and the caller composes the
  * op from a projection product and af3_dpa_forward with its `gate` argument.

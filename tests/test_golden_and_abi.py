@@ -283,3 +283,27 @@ def test_weight_unpacking_inverts_the_panel_layout(oracle):
     wf = torch.randn(C, C, generator=g)
     panels = wf.view(C, head, K).permute(1, 0, 2).contiguous().view(C, C)
     assert torch.equal(fused._unpack_panels(panels, head), wf)
+
+
+def test_row_op_entry_points_validate_on_the_host():
+    """af3_gated_linear_unit, af3_linear and af3_layernorm_pair_bias refuse malformed calls with a status code, before any launch."""
+    from af3_kernels_amd import _lib
+    lib = _lib.load()
+    P, BF, F32 = 0x1000, _lib.AF3_BF16, _lib.AF3_F32
+    for fn in (lib.af3_gated_linear_unit, lib.af3_linear):
+        assert fn(None, P, P, 64, 128, 64, BF, None) == -1
+        assert fn(P, P, P, 0, 128, 64, BF, None) == -3
+        assert fn(P, P, P, 64, 128, 64, F32, None) == -2                  # bfloat16 only
+        assert fn(P, P, P, 64, 96, 64, BF, None) == -7                    # 64 or 128 input channels
+        assert fn(P, P, P, 64, 128, 48, BF, None) == -7                   # outputs in tiles of 32 columns
+        assert fn(P + 2, P, P, 64, 128, 64, BF, None) == -7               # rows not 16-byte aligned
+    ln = lib.af3_layernorm_pair_bias
+    ps, bs = (ctypes.c_int64 * 2)(9 * 128, 128), (ctypes.c_int64 * 2)(6 * 9, 9)
+    assert ln(None, ps, P, P, 1e-5, P, P, P, bs, 6, 9, 128, 4, BF, None) == -1
+    assert ln(P, ps, P, P, 1e-5, P, P, P, bs, 0, 9, 128, 4, BF, None) == -3
+    assert ln(P, ps, P, P, 1e-5, P, P, P, bs, 6, 9, 128, 4, F32, None) == -2
+    assert ln(P, ps, P, P, 1e-5, P, P, P, bs, 6, 9, 64, 4, BF, None) == -7      # 128 channels, 4 heads
+    assert ln(P, ps, P, P, 1e-5, P, P, P, bs, 6, 9, 128, 8, BF, None) == -7
+    assert ln(P, (ctypes.c_int64 * 2)(9 * 128, 64), P, P, 1e-5, P, P, P, bs, 6, 9, 128, 4, BF, None) == -4   # tokens overlap
+    assert ln(P, ps, P, P, 1e-5, P, P, P, (ctypes.c_int64 * 2)(6 * 9, 4), 6, 9, 128, 4, BF, None) == -4        # bias rows overlap
+    assert ln(P, ps, P, P, -1.0, P, P, P, bs, 6, 9, 128, 4, BF, None) == -7

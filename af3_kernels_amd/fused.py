@@ -1,19 +1,21 @@
-"""The two fused callers of the attention core, with the reference's names and argument lists:
+"""The callers around the attention core, with the reference's names and argument lists:
 
-    _attention_cpp      src/af3_kernels/__init__.py:55-80    -> _attention_impl      (dot_product_attention.cpp:200-378)
-    self_attention_cpp  src/af3_kernels/__init__.py:83-105   -> self_attention_impl  (dot_product_attention.cpp:380-543)
-
-and the module that wraps the first one, GridSelfAttentionCpp (src/af3_kernels/Attention.py:23-82).
+    _attention_cpp         src/af3_kernels/__init__.py:55-80    -> _attention_impl      (dot_product_attention.cpp:200-378)
+    self_attention_cpp     src/af3_kernels/__init__.py:83-105   -> self_attention_impl  (dot_product_attention.cpp:380-543)
+    GridSelfAttentionCpp   src/af3_kernels/Attention.py:23-82   (the module around _attention_cpp)
+    layernorm_pair_bias    src/af3_kernels/Attention.py:51-52   (torch ops in the reference: LayerNorm, bias projection, permute)
+    gated_linear_unit_cpp  src/af3_kernels/__init__.py:21-28    -> gated_linear_unit_impl (gated_linear_unit.cpp:20-80)
+    Linear                 src/af3_kernels/__init__.py:138-163  -> linear_impl            (gated_linear_unit.cpp:82-129)
 
 On the GPU the grid op in AlphaFold 3's shape (bfloat16, 128 channels, 4 heads) is ONE kernel for the projections,
 the attention and the gate (af3_grid_attention_forward: q, k, v and the gate never touch device memory) followed by
 the output projection (af3_linear).  Every other shape, and the diffusion op, is three launches:
   1. ONE library GEMM for the four projections: x [rows, C] . W [C, 4C], output columns ordered
      (head, [k, v, q, gate], channel)  (hipBLASLt through torch: a plain GEMM is library territory);
-  2. the attention kernel, reading q, k, v as strided views of that GEMM's output (no
+  2. the attention kernel, reading q, k, v and the gate where that GEMM left them (no
      "b n (h d) -> b h n d" copies), adding bias and mask, and applying sigmoid(gate) in its
      epilogue while writing straight into the "b n (h d)" layout;
-  3. the output projection GEMM (grid attention only).
+  3. the output projection (grid attention only).
 Weights arrive in the layout the reference's callers produce with vnni_repack_tensor(W.T, 2, C/head)
 and are unpacked once per weight set into the fused matrix (cached per live weight tensor and version).
 """

@@ -15,7 +15,12 @@
  * the bias-free case, an independent float64 numpy closed form, a pure-Python brute force on
  * tiny shapes, algebraic invariants (row-shift of the bias, key permutation, single live key,
  * uniform logits), flash == non-flash, torch's own bf16 / float8_e4m3fn casts for the
- * converters and a view/permute identity for the VNNI pack.
+ * converters and a view/permute identity for the VNNI pack.  The callers around the core (af3o_fused_attention_*,
+ * af3o_layernorm_pair_bias, af3o_gated_linear_unit) are pinned against torch library ops in float64 (linear,
+ * scaled_dot_product_attention, sigmoid, layer_norm, silu), against independent numpy forms through the golden
+ * vectors, and by special cases (zero gate weights, identity output projection, a q bias alone driving the logits,
+ * constant rows under LayerNorm, a saturated GLU gate); their reference-arithmetic variants are checked against the
+ * exact forms in fp32 (equal) and bf16 (within the bf16 budget).
  *
  * Parity unpinned: the bit pattern of the reference's bf16 pipeline (libxsmm's JIT exp
  * polynomial and BRGEMM summation order are not reproducible without libxsmm).  The oracle

@@ -159,30 +159,35 @@ __device__ __forceinline__ uint32_t lds_addr_of(const void* ptr) {
 // variant only).  SPLIT: for launches too small to fill the chip -- the NW wavefronts of a workgroup
 // share ONE block of 32 query rows and split its key tiles round robin (each with private LDS
 // buffers, no barrier in the loop); their partial (O, m, l) are merged through LDS at the end.
+// KS2: the other cure for launches too small to fill the chip, for long rows: two wavefronts share each block of 32
+// query rows AND the workgroup's K/V tiles -- wavefront 2q + s takes keys [32s, 32s + 32) of every 64-key tile for
+// query block q, so a wavefront's dependent chain is half as long and no LDS is spent on private buffers; the two
+// partial (O, m, l) are merged through LDS at the end.  Requires NW even, no SPLIT, not FUSED.
 // FUSED: the grid-attention variant.  One workgroup = one (batch, head); q, k, v and the gate are not
 // read from memory but projected in the kernel from the input rows x[b] (C channels) with the four
 // weight matrices of this head, K and V of ALL keys stay in LDS for the whole workgroup, and each
 // wavefront then walks query blocks qb = wave, wave + NW, ... on its own (no barrier after the
 // projection of K and V).  Requires DP = 32, the log2 variant, no key split.
-template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT, bool FUSED>
+template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT, bool FUSED, bool KS2>
 // (at least 2 wavefronts per SIMD: keeps the register budget at 256 so that the compiler writes MFMA
 // results to ordinary VGPRs instead of AGPRs, which every softmax operand would have to be copied out of;
 // the key-split variants are limited to fewer than 2 wavefronts per SIMD by their LDS buffers anyway)
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FUSED ? (NW <= 4 ? 3 : (NW + 3) / 4) : DP == 32 && !SPLIT ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups, fused_grid_args fa) {
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FUSED ? (NW <= 4 ? 3 : (NW + 3) / 4) : DP == 32 && !SPLIT && !KS2 ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups, fused_grid_args fa) {
 	constexpr int NC         = DP / 16;            // contraction chunks of QK^T
 	constexpr int NDB        = DP / 32;            // 32-row blocks of O^T
 	constexpr int CPR        = DP / 8;             // 16-byte chunks per K/V row
 	constexpr int TILE_BYTES = KT * DP * 2;
 	constexpr int NI         = TILE_BYTES / 1024;  // 1 KB wave loads per tile and tensor
 	constexpr int RPI        = 512 / DP;           // tile rows covered by one wave load
-	constexpr int QT         = SPLIT ? 32 : NW * 32;
+	constexpr int QT         = SPLIT ? 32 : KS2 ? NW * 16 : NW * 32;
 	constexpr int  LDS_SETS   = SPLIT ? NW : 1;  // private K/V buffer sets
 	constexpr bool BIAS_F32   = BMODE == 1;      // natural variant, bias stored as fp32, read in place
 	constexpr bool BRING      = BMODE == 2;      // natural variant, bf16 bias streamed through a per-wavefront LDS ring
-	constexpr int  RING_BYTES = BRING ? NW * 3 * 4096 : 0;
+	constexpr int  RING_BYTES = BRING ? (KS2 ? NW / 2 : NW) * 3 * 4096 : 0;  // (KS2: one ring per pair of wavefronts)
 	constexpr int  MASK_BASE  = LDS_SETS * 6 * TILE_BYTES + RING_BYTES;
 	static_assert(!(L2DOM && BMODE != 0), "the log2 variant reads its bias from the workspace");
-	static_assert(FUSED || NW <= NI, "every wavefront fetches a whole number of 1 KB pieces of each tile");
+	static_assert(FUSED || (KS2 ? (2 * NI) % NW == 0 : NW <= NI), "every wavefront fetches a whole number of 1 KB pieces of each tile");
+	static_assert(!KS2 || (!SPLIT && !FUSED && NW % 2 == 0), "the shared-tile key split pairs up the wavefronts of an unfused workgroup");
 	static_assert(!FUSED || (DP == 32 && L2DOM && !SPLIT && NW % 2 == 0), "the fused variant exists for 32-channel heads in the log2 variant");
 
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -388,7 +393,9 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	// ---- one pass per block of 32 query rows: exactly one pass unless FUSED ----
 	for(; qb_f >= 0; qb_f -= FUSED ? NW : 1) {
 		// ---- per-lane constants ----
-		const int64_t qrow   = FUSED ? (int64_t)qb_f * 32 + n : (int64_t)qtile * QT + (SPLIT ? 0 : wave * 32) + n;
+		const int     sub    = KS2 ? (wave & 1) : 0;             // KS2: which 32 keys of every 64-key tile this wavefront takes
+		const int     wblk   = SPLIT ? 0 : KS2 ? (wave >> 1) : wave;  // this wavefront's block of 32 query rows within the workgroup's QT rows
+		const int64_t qrow   = FUSED ? (int64_t)qb_f * 32 + n : (int64_t)qtile * QT + wblk * 32 + n;
 		const bool    row_ok = qrow < L;
 
 		// Q fragments (B operand of S^T = K.Q^T): lane (q = n, g = half) holds q[q][16c + 8g .. +7]
@@ -439,20 +446,20 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		const u32x4* ws_wave = nullptr;
 		if(L2DOM && has_bias) {
 			const int     n_qblocks = (int)((L + 31) / 32);
-			const int64_t qb        = FUSED ? (int64_t)qb_f : SPLIT ? (int64_t)qtile : (int64_t)qtile * NW + wave;
+			const int64_t qb        = FUSED ? (int64_t)qb_f : SPLIT ? (int64_t)qtile : (int64_t)qtile * (QT / 32) + wblk;
 			// query blocks beyond the last one only hold rows >= L; clamp so that loads stay in bounds
 			const int64_t qbc = qb < n_qblocks ? qb : n_qblocks - 1;
 			ws_wave = static_cast<const u32x4*>(p.workspace) + ((h * n_qblocks + qbc) * n_ktiles) * 256;
 		}
 		// (scalar base + per-lane 16-byte offset + scalar tile offset: no 64-bit pointer in vector registers)
 		const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(ws_wave), 0, ws_wave ? n_ktiles * 4096 : 0, 0x00020000);
-		const int                    ws_voff = lane * 16;
+		const int                    ws_voff = lane * 16 + sub * 2048;  // (KS2: fragments 2 and 3 of a tile belong to keys 32..63)
 
 		// ---- output gate: fetched into LDS now, by loads that write LDS directly and hold no registers, and read in the
 		// epilogue.  (Loading it in the epilogue exposed a full memory latency per workgroup: 8 % of the kernel's time.)
 		// The first tile wait of the prologue below also covers these loads: they are older. ----
-		unsigned char* const gate_lds = smem + gate_base + (SPLIT ? 0 : wave * (32 * DP * 2));
-		if(!FUSED && p.gate && (!SPLIT || wave == 0)) {
+		unsigned char* const gate_lds = smem + gate_base + wblk * (32 * DP * 2);
+		if(!FUSED && p.gate && (SPLIT ? wave == 0 : sub == 0)) {  // (the wavefronts that write results)
 			const u32x4   g_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.gate) + b * p.gate_stride[0] + h * p.gate_stride[1], (uint32_t)(((L - 1) * p.gate_stride[2] + D) * 2));
 			constexpr int RPL    = 512 / DP;  // rows per 1 KB wave load
 			const int     g_row  = lane / CPR, g_c = lane % CPR;
@@ -482,6 +489,18 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		const uint32_t k_lds_addr = lds_addr_of(k_lds), v_lds_addr = lds_addr_of(v_lds);
 		auto load_tile = [&](int kt, int buf) {
 			if(FUSED) return;  // K and V of every tile are already in LDS
+			if constexpr(KS2) {  // the 2 * NI pieces of K and V are dealt out over all NW wavefronts
+#pragma unroll
+				for(int t = 0; t < 2 * NI / NW; t++) {
+					const int pc = wave + NW * t;  // (wave-uniform)
+					if(pc < NI) {
+						if(k_act) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + pc * 1024, k_voff + (kt * k_tile_stride + pc * k_ld_stride));
+					} else {
+						if(v_act) lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + (pc - NI) * 1024, v_voff + (kt * v_tile_stride + (pc - NI) * v_ld_stride));
+					}
+				}
+				return;
+			}
 #pragma unroll
 			for(int t = 0; t < (SPLIT ? NI : NI / NW); t++) {
 				const int j = SPLIT ? t : wave + NW * t;  // split: this wavefront fetches whole tiles into its private buffers
@@ -499,26 +518,26 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		// entries is never read.  Whatever such lanes leave in LDS is finite: the ring starts zeroed.
 		const u32x4    b_rsrc    = raw_rsrc(BRING ? static_cast<const uint16_t*>(p.bias) + h * p.bias_stride[0] : nullptr,
 											BRING ? (uint32_t)(((L - 1) * p.bias_stride[1] + L) * 2) : 0u);
-		unsigned char* const bring = smem + LDS_SETS * 6 * TILE_BYTES + (BRING ? wave * 3 * 4096 : 0);
+		unsigned char* const bring = smem + LDS_SETS * 6 * TILE_BYTES + (BRING ? (KS2 ? wblk : wave) * 3 * 4096 : 0);
 		const uint32_t bring_addr = lds_addr_of(bring);
 		const int      b_voff     = (int)((lane >> 3) * p.bias_stride[1] * 2) + (((lane & 7) ^ (lane >> 3)) << 4);
-		const int      b_row0     = (int)((qtile * QT + (SPLIT ? 0 : wave * 32)) * p.bias_stride[1] * 2);
+		const int      b_row0     = (int)((qtile * QT + wblk * 32) * p.bias_stride[1] * 2);
 		const int      b_row8     = (int)(8 * p.bias_stride[1] * 2);
 		const int      b_key      = ((lane & 7) ^ (lane >> 3)) * 8;  // first key of this lane's chunk within a tile
 		auto load_bias_tile = [&](int kt, int slot_i) {
-			if(!BRING) return;
+			if(!BRING || (KS2 && sub != 0)) return;  // (KS2: the pair's first wavefront fetches the whole 32 x 64 tile for both)
 			const int in_row = kt * KT + b_key < (int)L ? b_voff + kt * (KT * 2) : 0x7FFF0000;
 #pragma unroll
 			for(int j = 0; j < 4; j++) lds_dma_b128(b_rsrc, bring_addr + slot_i * 4096 + j * 1024, in_row + (b_row0 + j * b_row8));
 		};
 		// fragment read: lane (n, half) takes chunk 4*sub + 2*c2 + half of row n
-		const int b_rd = n * 128 + (((n & 7) ^ half) << 4);
+		const int b_rd = (n * 128 + (((n & 7) ^ half) << 4)) ^ (sub << 6);  // (KS2: chunks 4..7 of a row hold keys 32..63)
 
 		// Natural variant: four fragments in flight, each sub-tile's pair requested two stages before its
 		// use.  Log2 variant (BIAS_LATE): one pair only -- the registers are the scarce resource at four
 		// wavefronts per SIMD -- requested inside the previous stage, right after the matrix
 		// instructions that consume the pair before it.
-		constexpr bool BIAS_LATE = L2DOM;
+		constexpr bool BIAS_LATE = L2DOM || KS2;  // (KS2: one stage per tile, so one pair one stage ahead in every variant)
 		u32x4 bfrag[4];
 		auto  load_bias_frags = [&](int kt, auto sub_c) {
 			constexpr int SUB = decltype(sub_c)::value;
@@ -529,7 +548,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 					bfrag[c2] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, ws_voff + (2 * SUB + c2) * 1024, kt * 4096, 0));
 				return;
 			}
-			const int64_t key0 = (int64_t)kt * KT + 8 * half;
+			const int64_t key0 = (int64_t)kt * KT + 8 * half + 32 * sub;
 			if(bias_vec && (int64_t)(kt + 1) * KT <= L) {  // wave-uniform: whole tile in range, aligned rows
 				const uint16_t* bp = reinterpret_cast<const uint16_t*>(bias_row) + key0;
 				if(row_ok) {
@@ -553,7 +572,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		// ---- per-lane LDS read addresses (bytes, for buffer 0 / sub-tile 0; the rest are immediates) ----
 		int k_rd[NC];
 #pragma unroll
-		for(int c = 0; c < NC; c++) k_rd[c] = n * DP * 2 + (((2 * c + half) ^ k_swizzle<DP>(n)) << 4);
+		for(int c = 0; c < NC; c++) k_rd[c] = (n + 32 * sub) * DP * 2 + (((2 * c + half) ^ k_swizzle<DP>(n)) << 4);  // (KS2: rows 32..63 of every tile)
 		// V^T fragment reads: lane l: i = l%16, G = l/16 supplies the 8-byte chunk at tile row
 		// base + 4*(G/2) + i/4, column 32*db + 16*(G%2) + 4*(i%4); it receives 4 keys of column 32*db + l%32.
 		int v_rd[NDB];
@@ -564,11 +583,11 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 			for(int db = 0; db < NDB; db++) {
 				const int col   = 32 * db + 16 * (G & 1) + 4 * (i16 & 3);
 				const int chunk = (col >> 3) ^ v_swizzle<DP>(row);
-				v_rd[db] = row * DP * 2 + chunk * 16 + (col & 7) * 2;
+				v_rd[db] = (row + 32 * sub) * DP * 2 + chunk * 16 + (col & 7) * 2;
 			}
 		}
 		// mask table read address: lanes of the upper half-wave always read the zero entries
-		const int mask_rd     = mask_base + (half == 0 ? n * 4 : (n_ktiles * KT + n) * 4);
+		const int mask_rd     = mask_base + (half == 0 ? (n + 32 * sub) * 4 : (n_ktiles * KT + n) * 4);
 		const int mask_stride = half == 0 ? KT * 4 : 0;
 
 		// ---- online-softmax state (per lane: one query row; the two halves hold disjoint keys) ----
@@ -808,7 +827,8 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 			if(BRING) read_bias_ring(0, ic<0>{});
 			sc = compute_s_plain(FUSED ? kt0 * TILE_BYTES : 0, 0, mask_rd + kt0 * mask_stride, 0);
 			rereference(sc, nullptr, true);
-			if(BIAS_LATE) load_bias_frags(kt0, ic<1>{});
+			if(KS2) load_bias_frags(__builtin_amdgcn_readfirstlane(live_at(1)), ic<0>{});  // this wavefront's next sub-tile is in the next tile
+			else if(BIAS_LATE) load_bias_frags(kt0, ic<1>{});
 			else if(my_n > 1) load_bias_frags(__builtin_amdgcn_readfirstlane(live_at(1)), ic<0>{});
 
 			int buf = 0;  // LDS buffer of tile `it` (it % 3)
@@ -820,6 +840,24 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 				const int bufn = buf == 2 ? 0 : buf + 1, bufnn = bufn == 2 ? 0 : bufn + 1;
 				// LDS offsets of tile it and of tile it+1: ring buffers, or the tiles' own places when all of K and V is resident
 				const int off_cur = (FUSED ? kt : buf) * TILE_BYTES, off_next = (FUSED ? kt1 : bufn) * TILE_BYTES;
+				if constexpr(KS2) {
+					// One stage per tile: this wavefront's 32 keys of tile `it` (exp, V fragments) and of tile it+1 (S^T).  Tile
+					// it+1 (issued one iteration ago, or in the prologue) must have landed and everyone must be done with tile
+					// it-1 before tile it+2 overwrites it; the only younger loads are the two bias fragments of the log2 variant.
+					if(L2DOM && has_bias) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+					else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+					__syncthreads();
+					if(it + 2 < my_n) {
+						load_tile(kt2, bufnn);
+						load_bias_tile(kt2, bufnn);
+					}
+					stage(ic<0>{}, off_next, mask_rd + kt1 * mask_stride, off_cur, ic<0>{}, kt2, ic<0>{}, bufn * 4096);
+					buf = bufn;
+					kt  = kt1;
+					kt1 = kt2;
+					kt2 = __builtin_amdgcn_readfirstlane(kt3_v);
+					continue;
+				}
 				// sub-tile (it, 0): next is (it, 1) in the same buffer
 				stage(ic<1>{}, off_cur, mask_rd + kt * mask_stride, off_cur, ic<0>{}, kt1, ic<0>{}, buf * 4096);
 				if(!BIAS_LATE) load_bias_frags(kt1, ic<1>{});
@@ -852,6 +890,38 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 			for(int db = 0; db < NDB; db++)
 				oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[cp][db]), __builtin_bit_cast(bf16x8, pprev[cp]), oacc[db], 0, 0, 0);
 
+		if constexpr(KS2) {
+			// ---- merge the two partial results of every pair of wavefronts (same 32 query rows, disjoint keys) ----
+			asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+			__syncthreads();  // all K/V buffers are dead: reuse the front of LDS
+			float* const mred = reinterpret_cast<float*>(smem);        // [NW][32] reference maxima
+			float* const obuf = mred + NW * 32;                        // [NW / 2][16*NDB + 1][64]
+			static_assert((NW * 32 + (NW / 2) * (16 * NDB + 1) * 64) * 4 <= 6 * TILE_BYTES, "the merge area fits in the K/V buffers");
+			if(half == 0) mred[wave * 32 + n] = m_ref;
+			__syncthreads();
+			const float mstar   = fmaxf(mred[(wave & ~1) * 32 + n], mred[(wave | 1) * 32 + n]);
+			const float scale_w = __builtin_amdgcn_exp2f((m_ref - mstar) * (L2DOM ? 1.f : LOG2E));
+			lacc[0] *= scale_w;
+#pragma unroll
+			for(int db = 0; db < NDB; db++)
+#pragma unroll
+				for(int i = 0; i < 16; i++) oacc[db][i] *= scale_w;
+			float* const slot_p = obuf + wblk * (16 * NDB + 1) * 64 + lane;
+			if(sub == 1) {
+#pragma unroll
+				for(int db = 0; db < NDB; db++)
+#pragma unroll
+					for(int i = 0; i < 16; i++) slot_p[(db * 16 + i) * 64] = oacc[db][i];
+				slot_p[16 * NDB * 64] = lacc[0];
+			}
+			__syncthreads();
+			if(sub == 1) return;
+#pragma unroll
+			for(int db = 0; db < NDB; db++)
+#pragma unroll
+				for(int i = 0; i < 16; i++) oacc[db][i] += slot_p[(db * 16 + i) * 64];
+			lacc[0] += slot_p[16 * NDB * 64];
+		}
 		if(SPLIT) {
 			// ---- merge the partial results of the NW wavefronts (same 32 query rows, disjoint keys) ----
 			asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -988,22 +1058,24 @@ static int launch_bias_prepass(const af3_dpa_params& p, hipStream_t s) {
 constexpr size_t LDS_LIMIT = 160 * 1024;  // per workgroup on gfx950
 
 // dynamic LDS of one variant: K/V buffers, bias ring, mask table, tile list, gate rows of every wavefront that writes results
-template <int DP, int NW, int BMODE, bool SPLIT>
+template <int DP, int NW, int BMODE, bool SPLIT, bool KS2 = false>
 static size_t lds_bytes(const af3_dpa_params& p) {
 	const size_t n_ktiles = (size_t)((p.L + KT - 1) / KT);
-	return (size_t)(SPLIT ? NW : 1) * 6 * KT * DP * 2 + (BMODE == 2 ? NW * 3 * 4096 : 0) + (n_ktiles * KT + 64) * 4 + n_ktiles * 2 + 16 + (p.gate ? (size_t)(SPLIT ? 1 : NW) * 32 * DP * 2 : 0);
+	const size_t writers  = SPLIT ? 1 : KS2 ? NW / 2 : NW;  // wavefronts that own a block of query rows
+	return (size_t)(SPLIT ? NW : 1) * 6 * KT * DP * 2 + (BMODE == 2 ? (KS2 ? NW / 2 : NW) * 3 * 4096 : 0) + (n_ktiles * KT + 64) * 4 + n_ktiles * 2 + 16 +
+		   (p.gate ? writers * 32 * DP * 2 : 0);
 }
 
-template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT = false>
+template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT = false, bool KS2 = false>
 static int launch_one(const af3_dpa_params& p, hipStream_t s) {
-	constexpr int QT       = SPLIT ? 32 : NW * 32;
+	constexpr int QT       = SPLIT ? 32 : KS2 ? NW * 16 : NW * 32;
 	const int     n_qtiles = (int)((p.L + QT - 1) / QT);
 	const int64_t n_groups = p.B * p.H;
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
-	const size_t smem = lds_bytes<DP, NW, BMODE, SPLIT>(p);
+	const size_t smem = lds_bytes<DP, NW, BMODE, SPLIT, KS2>(p);
 	if(smem > LDS_LIMIT) return AF3_ERR_BAD_SHAPE;  // (launch_nw only picks variants that fit)
-	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BMODE, SPLIT, false>;
+	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BMODE, SPLIT, false, KS2>;
 	if(smem > 64 * 1024) {  // beyond the default dynamic-LDS limit: raise it for this kernel (idempotent, host side)
 		if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
 	}
@@ -1054,7 +1126,7 @@ static int launch_fused_nw(const af3_dpa_params& p, const fused_grid_args& fa, h
 	const int64_t blocks   = 16 * ((p.B + 3) / 4);  // see the kernel's workgroup -> (batch row, head) map
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
 	const size_t smem = fused_lds_bytes(p.L);
-	auto         kern = dpa_mfma_bf16_kernel<32, NW, true, 0, false, true>;
+	auto         kern = dpa_mfma_bf16_kernel<32, NW, true, 0, false, true, false>;
 	if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
 	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, 1, n_groups, fa);
 	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
@@ -1095,6 +1167,13 @@ static int launch_nw(const af3_dpa_params& p, hipStream_t s) {
 		// its head from L2, which then outweighs the bias stream; from 512 query blocks on, four blocks
 		// share each K/V tile instead (measured, B=1 H=16 D=24: L=1536 25.6 us against 32.7 us with
 		// single-wave workgroups; L=768 14.0 us split in two against 14.3 / 17.8; L=384 8.5 us split in four).
+		// Long rows with too few 128-row workgroups to fill the 256 compute units: pairs of wavefronts share a query block and
+		// the workgroup's K/V tiles.  The work per SIMD is unchanged -- two wavefronts of half the length instead of one -- but
+		// the two overlap their matrix and vector phases (measured, B=1 H=16 L=1536: 26.0 against 31.1 us at head_dim 24; at
+		// head_dim 48, padded to 64, nothing is gained, so that size keeps one wavefront per query block).
+		if constexpr(DP == 32) {
+			if(blocks1 >= 512 && blocks1 <= 1024 && ktiles >= 8) return launch_one<DP, 8, L2DOM, BMODE, false, true>(p, s);
+		}
 		if(blocks1 >= 512) return launch_one<DP, 4, L2DOM, BMODE>(p, s);
 		// (the split variants' private buffers plus a long row's mask table can exceed the LDS of a compute unit: then the next one)
 		if(DP == 32 && ktiles >= 4 && blocks1 <= 256 && lds_bytes<DP, 4, BMODE, true>(p) <= LDS_LIMIT) return launch_one<DP, 4, L2DOM, BMODE, true>(p, s);

@@ -140,6 +140,41 @@ def test_small_grids_split_keys_over_wavefronts(af3, oracle, B, H, L, D, live):
     assert np.abs(f32np(out) - want).max() <= TOL[torch.bfloat16]
 
 
+@pytest.mark.parametrize("H,L,D,bias_kind,live", [
+    (16, 1536, 24, "bf16", None),          # bias through the LDS ring, one ring per pair of wavefronts
+    (16, 1536, 32, "bf16", (100, 1400)),   # dead tiles at both ends
+    (16, 1536, 48, "bf16", (100, 1400)),   # head_dim 48 (padded to 64) keeps one wavefront per query block
+    (8, 2048, 32, "f32", None),            # fp32 bias read in place
+    (16, 1000, 32, "unaligned", 900),      # bias rows that cannot take 16-byte loads: element-wise path; ragged last tile
+    (16, 1536, 16, "none_live_tail", 33),  # only the first 33 keys are live
+])
+def test_long_rows_pair_up_wavefronts_on_shared_tiles(af3, oracle, H, L, D, bias_kind, live):
+    """B = 1 with 512..1024 query blocks and at least 8 key tiles: two wavefronts share each query block and the workgroup's
+    K/V tiles, each taking 32 of every 64 keys; their partial softmax states are merged at the end."""
+    q, k, v, m, bias = rand_inputs(1, H, L, D, torch.bfloat16, seed=L + D)
+    if isinstance(live, int):
+        m[:, live:] = False
+    elif live is not None:
+        m[:] = False
+        m[:, live[0]:live[1]] = True
+    if bias_kind == "f32":                # (the drop-in casts the bias to q's dtype; the lean op hands an fp32 bias to the kernel as it is)
+        from af3_kernels_amd import ops
+        dq, dk, dv, dm = dev(q, k, v, m)
+        out = ops._dpa_forward_impl(dq, dk, dv, ops._lift_mask(dm, L), bias.float().cuda(), ops._DTYPE_CODE[torch.bfloat16], False)
+        want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), f32np(bias))
+        assert np.abs(f32np(out) - want).max() <= TOL[torch.bfloat16]
+        return
+    if bias_kind == "unaligned":
+        wide = torch.zeros(H, L, L + 3, dtype=torch.bfloat16)
+        wide[:, :, :L] = bias
+        dq, dk, dv, dm = dev(q, k, v, m)
+        out = af3.dot_product_attention_cpp(dq, dk, dv, dm, wide.cuda()[:, :, :L])       # row stride L + 3: not a multiple of 8
+        want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), f32np(bias))
+        assert np.abs(f32np(out) - want).max() <= TOL[torch.bfloat16]
+        return
+    run_case(af3, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+
+
 def test_long_rows_with_few_heads_pick_a_variant_that_fits_in_lds(af3, oracle):
     """B*H = 1 with L = 5000: the four-wave key split with the bias ring would need more LDS than a compute unit has
     (private K/V buffers + ring + a 20 KB mask table); the launcher must pick the next variant instead of failing."""

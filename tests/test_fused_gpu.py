@@ -151,6 +151,7 @@ def test_grid_attention_one_kernel_variants(af3, oracle):
 SELF_CASES = [
     # N, C, head, dtype
     (64, 768, 16, torch.bfloat16),       # the diffusion transformer's shape: 16 heads of 48 channels
+    (1536, 768, 16, torch.bfloat16),     # its longest sequence: pairs of wavefronts per query block, gate rows in LDS
     (200, 768, 16, torch.bfloat16),
     (77, 256, 8, torch.bfloat16),
     (150, 128, 4, torch.float32),

@@ -260,9 +260,10 @@ def layernorm_pair_bias(pair: torch.Tensor, ln_weight: torch.Tensor, ln_bias: to
     with 128 channels and 4 heads; the same torch ops as the reference otherwise."""
     ops._require_device(pair, ln_weight, ln_bias, proj_weight)
     head, C = proj_weight.shape
+    ln_weight, ln_bias, proj_weight = ln_weight.contiguous(), ln_bias.contiguous(), proj_weight.contiguous()
     if not (pair.dtype == torch.bfloat16 and pair.dim() == 3 and C == 128 and head == 4 and pair.shape[-1] == C and pair.numel() > 0
             and ln_weight.dtype == ln_bias.dtype == proj_weight.dtype == torch.bfloat16 and pair.stride(2) == 1 and pair.stride(0) % 8 == 0
-            and pair.stride(1) % 8 == 0 and pair.data_ptr() % 16 == 0):
+            and pair.stride(1) % 8 == 0 and all(t.data_ptr() % 16 == 0 for t in (pair, ln_weight, ln_bias, proj_weight))):
         normed = torch.nn.functional.layer_norm(pair, (C,), ln_weight, ln_bias, eps)
         return normed, torch.nn.functional.linear(normed, proj_weight).permute(2, 0, 1)
     n_i, n_j = pair.shape[:2]
@@ -270,8 +271,8 @@ def layernorm_pair_bias(pair: torch.Tensor, ln_weight: torch.Tensor, ln_bias: to
     bias = torch.empty(head, n_i, n_j, dtype=pair.dtype, device=pair.device)
     arr = ctypes.c_int64 * 2
     with ops._on_device(pair.device):
-        _lib.check(_lib.load().af3_layernorm_pair_bias(pair.data_ptr(), arr(pair.stride(0), pair.stride(1)), ln_weight.contiguous().data_ptr(), ln_bias.contiguous().data_ptr(),
-                                                       float(eps), proj_weight.contiguous().data_ptr(), normed.data_ptr(), bias.data_ptr(), arr(n_i * n_j, n_j), n_i, n_j, C, head,
+        _lib.check(_lib.load().af3_layernorm_pair_bias(pair.data_ptr(), arr(pair.stride(0), pair.stride(1)), ln_weight.data_ptr(), ln_bias.data_ptr(),
+                                                       float(eps), proj_weight.data_ptr(), normed.data_ptr(), bias.data_ptr(), arr(n_i * n_j, n_j), n_i, n_j, C, head,
                                                        ops._DTYPE_CODE[pair.dtype], ops._stream_ptr(pair.device)), "af3_layernorm_pair_bias")
     return normed, bias
 

@@ -399,3 +399,45 @@ def test_fused_callers_match_the_golden_vectors(af3):
     g = np.load(os.path.join(gdir, "glu_70x128_N64.npz"))
     out = af3.gated_linear_unit_cpp(bf(g["x"]), bf(g["weight"]))
     assert np.abs(f32np(out) - g["expected"]).max() <= 2e-2 * max(1.0, np.abs(g["expected"]).max())
+
+
+def test_fused_callers_can_be_captured_in_a_hip_graph_and_replayed(af3):
+    """Serving loops record these ops into HIP graphs: the module forward (LayerNorm + pair bias kernel, bias prepass, the one
+    attention kernel, output projection), the diffusion op and the gated linear unit are captured once and replayed with
+    fresh inputs copied into the captured buffers; every replay must reproduce the eager result bit for bit."""
+    N, C, head = 64, 128, 4
+    torch.manual_seed(5)
+    mod = af3.GridSelfAttentionCpp(C, head).cuda().to(torch.bfloat16).eval()
+    g = torch.Generator().manual_seed(8)
+    ws = [(torch.randn(768, 768, generator=g) / 768 ** 0.5).to(torch.bfloat16) for _ in range(4)]
+    packed = [pack(af3, w.cuda(), 16) for w in ws]
+    qb = torch.randn(768, generator=g).to(torch.bfloat16).cuda()
+    sbias = torch.randn(16, 96, 96, generator=g).to(torch.bfloat16).cuda()
+    smask = torch.ones(96, dtype=torch.bool, device="cuda")
+    wglu = (torch.randn(128, 512, generator=g) / 128 ** 0.5).to(torch.bfloat16).cuda()
+    pair = torch.randn(N, N, C, generator=g).to(torch.bfloat16).cuda()
+    mask = (torch.rand(N, N, generator=g) < 0.9).cuda()
+    xs = torch.randn(96, 768, generator=g).to(torch.bfloat16).cuda()
+
+    def run(p, x):
+        return mod(p, mask), af3.self_attention_cpp(x, smask, sbias, packed[0], qb, packed[1], packed[2], packed[3], 16), af3.gated_linear_unit_cpp(p, wglu)
+
+    with torch.no_grad():
+        run(pair, xs)                                  # warm-up outside the capture: library load, weight caches
+        torch.cuda.synchronize()
+        graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                outs = run(pair, xs)
+        torch.cuda.synchronize()
+        for rep in range(3):
+            g2 = torch.Generator().manual_seed(200 + rep)
+            npair = torch.randn(N, N, C, generator=g2).to(torch.bfloat16).cuda()
+            nxs = torch.randn(96, 768, generator=g2).to(torch.bfloat16).cuda()
+            pair.copy_(npair), xs.copy_(nxs)
+            graph.replay()
+            torch.cuda.synchronize()
+            eager = run(npair, nxs)
+            torch.cuda.synchronize()
+            for a, b in zip(outs, eager):
+                assert torch.equal(a, b), f"replay {rep} differs from the eager call"

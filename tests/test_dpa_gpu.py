@@ -251,6 +251,38 @@ def test_strided_inputs_and_prepadded_bias(af3, oracle):
     assert np.abs(f32np(out) - want).max() <= 2e-2
 
 
+def _sweep_shapes(n, seed, widths=(8, 16, 24, 32, 40, 48, 64)):
+    """Seeded shapes spread over what picks a kernel variant: the number of query blocks in the launch (few:
+    keys split over wavefronts; many: one wavefront per block), lengths on both sides of the 32-, 64- and
+    128-key boundaries, every padded head width, the three mask forms."""
+    rng = np.random.default_rng(seed)
+    shapes = []
+    while len(shapes) < n:
+        D = int(rng.choice(widths))
+        L = int(rng.choice([rng.integers(1, 130), 64 * rng.integers(1, 20) + rng.integers(-2, 3), rng.integers(130, 1300)]))
+        L = max(L, 1)
+        BH = int(rng.choice([1, 2, 3, 5, 8, 16, 40, 130]))
+        H = int(rng.choice([h for h in (1, 2, 4, 5, 8, 16) if BH % h == 0]))
+        B = BH // H
+        if B * H * L * L > 12_000_000:
+            continue
+        shapes.append((B, H, L, D, str(rng.choice(["none", "random", "tail"])), int(rng.choice([1, 2])), int(rng.integers(1 << 30))))
+    return shapes
+
+
+@pytest.mark.parametrize("B,H,L,D,mask,rank,seed", _sweep_shapes(24, 777, widths=(3, 5, 8, 12, 24, 32, 33, 64, 72, 128)))
+def test_fp32_seeded_shape_sweep(af3, oracle, B, H, L, D, mask, rank, seed):
+    """fp32 storage: whichever of the fp32 kernels the shape selects (matrix-core or vector-FMA)."""
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.float32, seed=seed, mask=mask, mask_rank=rank)
+    run_case(af3, oracle, q, k, v, m, bias)
+
+
+@pytest.mark.parametrize("B,H,L,D,mask,rank,seed", _sweep_shapes(48, 20241))
+def test_bf16_seeded_shape_sweep(af3, oracle, B, H, L, D, mask, rank, seed):
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=seed, mask=mask, mask_rank=rank)
+    run_case(af3, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+
+
 @pytest.mark.parametrize("B,H,L,D,mask,kernel", [
     (1, 2, 700, 40, "random", "fp32_mfma"),     # head_dim 40: padded to 64 columns
     (2, 3, 37, 20, "tail", "fp32_mfma"),        # odd length, head_dim 20

@@ -127,6 +127,24 @@ def test_grid_attention_one_kernel_matches_formula(af3, oracle, B, N):
     run_grid_case(af3, oracle, B, N, 128, 4, torch.bfloat16, one_kernel=True)
 
 
+def _one_kernel_sweep(n, seed):
+    """Seeded (B, N) over what picks the workgroup size of the one-kernel path: the number of 32-row query blocks
+    modulo 4 and modulo 12, rows short enough for three workgroups per compute unit, rows up to the LDS limit."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < n:
+        N = int(rng.choice([rng.integers(1, 140), 32 * rng.integers(1, 32) + rng.integers(-1, 2), rng.integers(140, 1024)]))
+        B = int(rng.integers(1, 7))
+        if N >= 1 and B * N * N <= 1_500_000:
+            cases.append((B, N))
+    return cases
+
+
+@pytest.mark.parametrize("B,N", _one_kernel_sweep(20, 4242))
+def test_grid_attention_one_kernel_seeded_sweep(af3, oracle, B, N):
+    run_grid_case(af3, oracle, B, N, 128, 4, torch.bfloat16, one_kernel=True)
+
+
 def test_grid_attention_one_kernel_variants(af3, oracle):
     """fp32 bias, mostly and fully dropped keys, a strided (transposed) pair view, and agreement with the three-launch path."""
     run_grid_case(af3, oracle, 4, 100, 128, 4, torch.bfloat16, one_kernel=True, bias_dtype=torch.float32)

@@ -56,6 +56,8 @@ def _cached(sources, extra, make):
         refs, versions, value = hit
         if all(r() is t for r, t in zip(refs, sources)) and versions == tuple(t._version for t in sources):
             return value
+    for k in [k for k, (refs, _, _) in _W_CACHE.items() if any(r() is None for r in refs)]:
+        del _W_CACHE[k]                      # derived matrices of weights that no longer exist
     if len(_W_CACHE) >= _W_CACHE_MAX:
         _W_CACHE.clear()
     value = make()

@@ -307,3 +307,38 @@ def test_row_op_entry_points_validate_on_the_host():
     assert ln(P, (ctypes.c_int64 * 2)(9 * 128, 64), P, P, 1e-5, P, P, P, bs, 6, 9, 128, 4, BF, None) == -4   # tokens overlap
     assert ln(P, ps, P, P, 1e-5, P, P, P, (ctypes.c_int64 * 2)(6 * 9, 4), 6, 9, 128, 4, BF, None) == -4        # bias rows overlap
     assert ln(P, ps, P, P, -1.0, P, P, P, bs, 6, 9, 128, 4, BF, None) == -7
+
+
+def test_derived_weight_cache_follows_tensor_identity_and_version():
+    """The cache of matrices derived from weights (host logic of the fused callers): same live tensor and version ->
+    same object; an in-place update or another tensor at a recycled id -> recomputed; entries of dead weights go."""
+    import gc
+    import torch
+    from af3_kernels_amd import fused
+    fused._W_CACHE.clear()
+    calls = []
+
+    def derive(t):
+        return fused._cached((t,), ("unit",), lambda: calls.append(1) or t.clone())
+
+    w = torch.arange(6.0)
+    a = derive(w)
+    assert derive(w) is a and len(calls) == 1
+    w.add_(1.0)                                  # bumps the version
+    b = derive(w)
+    assert b is not a and len(calls) == 2 and torch.equal(b, w)
+    other = torch.arange(6.0)
+    assert derive(other) is not b and len(calls) == 3
+    n_before = len(fused._W_CACHE)
+    del w, other
+    gc.collect()
+    derive(torch.zeros(3))                       # an insertion purges what belonged to tensors that no longer exist
+    assert len(fused._W_CACHE) == n_before - 2 + 1
+    # a stale entry under a recycled id must not be served: forge one
+    t = torch.ones(2)
+    key = (id(t), "unit")
+    dead = torch.ones(1)
+    import weakref
+    fused._W_CACHE[key] = ((weakref.ref(dead),), (dead._version,), "stale")
+    got = derive(t)
+    assert not isinstance(got, str) and torch.equal(got, t)

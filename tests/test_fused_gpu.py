@@ -192,6 +192,32 @@ def test_self_attention_cpp_matches_formula(af3, oracle, N, C, head, dtype):
     check(out, want, ref, dtype)
 
 
+def _self_sweep(n, seed):
+    """Seeded (N, C, head) for the diffusion op: head widths 16..64 (padded to 32 or 64 in the kernel), sequence lengths on
+    both sides of the 32- and 64-key boundaries and long enough for every key-split variant."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < n:
+        K = int(rng.choice([16, 24, 32, 48, 64]))
+        head = int(rng.choice([1, 2, 4, 8, 16]))
+        N = int(rng.choice([rng.integers(1, 100), 64 * rng.integers(1, 12) + rng.integers(-1, 2), rng.integers(100, 1200)]))
+        if N >= 1 and head * N * N <= 6_000_000 and K * head <= 1024:
+            cases.append((N, K * head, head))
+    return cases
+
+
+@pytest.mark.parametrize("N,C,head", _self_sweep(16, 99))
+def test_self_attention_cpp_seeded_sweep(af3, oracle, N, C, head):
+    x, mask, bias, wq, wk, wv, wg, _, qb = make(None, N, C, head, torch.bfloat16, seed=N * 7 + C, with_out=False, with_qbias=True)
+    print(f"self_attention_cpp N,C,head={N, C, head}", flush=True)
+    d = lambda t: t.cuda()
+    out = af3.self_attention_cpp(d(x), d(mask), d(bias), pack(af3, d(wq), head), d(qb), pack(af3, d(wk), head), pack(af3, d(wv), head),
+                                 pack(af3, d(wg), head), head, False, 64, 0)
+    torch.cuda.synchronize()
+    want = oracle.fused_attention_formula(f32np(x), mask.numpy(), f32np(bias), f32np(wq), f32np(wk), f32np(wv), f32np(wg), None, f32np(qb), head=head)
+    check(out, want, None, torch.bfloat16)
+
+
 def test_attention_cpp_mask_ranks_and_weight_cache(af3, oracle):
     """A 1-D mask is broadcast over the batch; a fully masked row set still yields finite values; changing a weight
     in place is seen by the next call (the fused weight matrix is cached per weight version)."""

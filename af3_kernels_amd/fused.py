@@ -33,6 +33,7 @@ _FUSED_MIN_GROUPS = 128
 
 _W_CACHE = {}
 _W_CACHE_MAX = 64
+_ATTEND_TEMPLATES = {}   # (B, N, head, K, dtype code) -> bytes of an af3_dpa_params block with the shape-dependent fields set
 
 
 def _unpack_panels(w: torch.Tensor, head: int) -> torch.Tensor:
@@ -126,19 +127,30 @@ def _attend(y: torch.Tensor, B: int, N: int, head: int, mask, bias) -> torch.Ten
         if bias.dim() != 3 or bias.shape[0] != head or bias.shape[1] < N or bias.shape[2] < N:
             raise ValueError(f"bias must be [head, N, N] with head={head}, N={N}, got {tuple(bias.shape)}")
     code, esz, base = ops._DTYPE_CODE[y.dtype], y.element_size(), y.data_ptr()
-    p = _lib.DpaParams()
-    p.k, p.v, p.q, p.gate = (base + i * K * esz for i in range(4))   # per token and head: (k | v | q | gate)
-    strides = (ctypes.c_int64 * 3)(N * 4 * C, 4 * K, 4 * C)
-    p.q_stride = p.k_stride = p.v_stride = p.gate_stride = strides
-    p.out, p.out_stride = out.data_ptr(), (ctypes.c_int64 * 3)(N * C, K, C)
-    p.B, p.H, p.L, p.D = B, head, N, K
+    # everything that depends on the shape alone is filled once per shape: this runs per layer of a model, and for short
+    # sequences the host side of a call costs as much as its kernels
+    shape_key = (B, N, head, K, code)
+    template = _ATTEND_TEMPLATES.get(shape_key)
+    if template is None:
+        t = _lib.DpaParams()
+        strides = (ctypes.c_int64 * 3)(N * 4 * C, 4 * K, 4 * C)
+        t.q_stride = t.k_stride = t.v_stride = t.gate_stride = strides
+        t.out_stride = (ctypes.c_int64 * 3)(N * C, K, C)
+        t.B, t.H, t.L, t.D = B, head, N, K
+        t.io_dtype = t.out_dtype = t.mma_dtype = t.bias_dtype = code
+        t.softmax_scale = float(K) ** -0.5
+        t.q_descale = t.k_descale = t.v_descale = 1.0
+        if len(_ATTEND_TEMPLATES) >= 256:
+            _ATTEND_TEMPLATES.clear()
+        template = _ATTEND_TEMPLATES[shape_key] = bytes(t)
+    p = _lib.DpaParams.from_buffer_copy(template)
+    p.k, p.v, p.q, p.gate = base, base + K * esz, base + 2 * K * esz, base + 3 * K * esz   # per token and head: (k | v | q | gate)
+    p.out = out.data_ptr()
     if bias is not None:
-        p.bias, p.bias_stride, p.bias_dtype = bias.data_ptr(), (ctypes.c_int64 * 2)(bias.stride(0), bias.stride(1)), code
+        p.bias = bias.data_ptr()
+        p.bias_stride[0], p.bias_stride[1] = bias.stride(0), bias.stride(1)
     if keep is not None:
         p.key_mask, p.key_mask_stride_b = keep.data_ptr(), (0 if keep.shape[0] == 1 else keep.stride(0))
-    p.io_dtype = p.out_dtype = p.mma_dtype = code
-    p.softmax_scale = float(K) ** -0.5
-    p.q_descale = p.k_descale = p.v_descale = 1.0
     lib = _lib.load()
     ws_bytes = lib.af3_dpa_workspace_bytes(ctypes.byref(p))
     if ws_bytes > 0 and not ops._exact_bias:

@@ -193,12 +193,19 @@ def quantize_e4m3(x):
     return out, float(scale)
 
 
-def fake_quantize_e4m3_pow2(x, pre_scale=1.0):
-    """x -> e4m3 with the shipped quantiser's power-of-two per-tensor scale -> back to float32
-    (including the pre_scale): what the fp8 kernels actually see."""
+def quantize_e4m3_pow2(x, pre_scale=1.0):
+    """Returns (bits uint8, scale) of the shipped quantiser's rule: scale = 2^floor(log2(448 / (amax * |pre_scale|)))
+    (1 when amax is 0), bits = e4m3(x * pre_scale * scale)."""
     x, xp = _f(x)
     bits = np.empty(x.shape, np.uint8)
     scale = lib().af3o_quantize_e4m3_pow2(xp, bits.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), x.size, pre_scale)
+    return bits, float(scale)
+
+
+def fake_quantize_e4m3_pow2(x, pre_scale=1.0):
+    """x -> e4m3 with the shipped quantiser's power-of-two per-tensor scale -> back to float32
+    (including the pre_scale): what the fp8 kernels actually see."""
+    bits, scale = quantize_e4m3_pow2(x, pre_scale)
     return dequantize_e4m3(bits, 1.0 / scale)
 
 

@@ -517,7 +517,9 @@ def test_fp8_mfma_matches_formula(af3, oracle, B, H, L, D, mask, rank):
     assert np.abs(comp - want_v).max() <= 4e-2, np.abs(comp - want_v).max()
     # (3) the stated fp8 budget against the formula on the un-quantised inputs: 6e-2 at diffusion-sized L.  Short
     # rows, where a single key can carry most of the weight, see the e4m3 rounding of that V row and of its
-    # probability directly (2^-4 relative each) and get a wider maximum.
+    # probability directly (2^-4 relative each): with q and k exact, those two roundings alone move these very
+    # inputs by 0.07 - 0.10 (tests/test_oracle_pins.py::test_fp8_short_row_error_budget_is_the_e4m3_rounding_of_p_and_v
+    # computes it on the CPU for the same seeds), so no e4m3 kernel meets 6e-2 there; the bound is that test's 0.15.
     want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), f32np(bias))
     err = np.abs(comp - want).max()
     assert err <= (6e-2 if L >= 1024 else 0.15), err

@@ -201,6 +201,85 @@ def test_quantize_e4m3_uses_per_tensor_amax_scale(oracle):
     assert np.abs(back - x).max() <= np.abs(x).max() / 16 + 1e-6  # 3 mantissa bits: half an ulp at the top binade
 
 
+@pytest.mark.parametrize("pre_scale", [1.0, 0.5, 32 ** -0.5, -0.17677669, 3.0])
+def test_quantize_e4m3_pow2_scale_rule_and_bits_match_torch(oracle, pre_scale):
+    """The shipped quantiser's variant: an independent scale (numpy float64 log2 / floor) and torch's own
+    float8_e4m3fn cast of x * pre_scale * scale, for tensors whose largest magnitude sits just below, at and just
+    above a power of two (the scale rule's break points), with ties and values that only saturation keeps finite."""
+    rng = np.random.default_rng(14)
+    for amax in (1.0, 0.999, 1.001, 3.7, 448.0, 447.0, 449.0, 1e-3, 6.1e4, 7.0 / 8.0):
+        x = rng.standard_normal(2048).astype(np.float32)
+        x = (x / np.abs(x).max() * amax).astype(np.float32)
+        x[5] = np.float32(amax)        # the maximum itself, exactly
+        x[6] = np.float32(-amax)
+        a = float(np.float32(np.abs(x).max()) * np.float32(abs(pre_scale)))
+        want_scale = 2.0 ** np.floor(np.log2(448.0 / a))
+        bits, scale = oracle.quantize_e4m3_pow2(x, pre_scale)
+        assert scale == want_scale, (amax, pre_scale, scale, want_scale)
+        prod = torch.from_numpy(x) * np.float32(pre_scale) * np.float32(want_scale)
+        assert prod.abs().max().item() <= 448.0 and prod.abs().max().item() > 224.0 * 0.999   # the top binade is used, nothing saturates
+        want = prod.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+        assert np.array_equal(bits, want)
+        back = oracle.fake_quantize_e4m3_pow2(x, pre_scale)
+        assert np.array_equal(back, torch.from_numpy(want).view(torch.float8_e4m3fn).float().numpy() / np.float32(want_scale))
+    # round-to-nearest-even ties of e4m3 (3 mantissa bits) at scale 1: amax 448 keeps scale = 1
+    ties = np.array([448.0, 1.0625, 1.1875, 17.0, 19.0, 2 ** -9 * 0.5, 2 ** -9 * 1.5, -1.0625, 0.0], np.float32)
+    bits, scale = oracle.quantize_e4m3_pow2(ties, 1.0)
+    assert scale == 1.0
+    assert np.array_equal(bits, torch.from_numpy(ties).to(torch.float8_e4m3fn).view(torch.uint8).numpy())
+    # an all-zero tensor keeps scale 1; a non-finite maximum does too (nothing sensible to scale to)
+    bits, scale = oracle.quantize_e4m3_pow2(np.zeros(16, np.float32), 0.5)
+    assert scale == 1.0 and not bits.any()
+    # values beyond the range saturate at +-448 (0x7E / 0xFE) instead of becoming NaN (0x7F)
+    lib = oracle.lib()
+    assert lib.af3o_f32_to_e4m3_bits(449.0) == 0x7E and lib.af3o_f32_to_e4m3_bits(-1e9) == 0xFE
+
+
+def _softmax_rows(logits):
+    logits = logits - logits.max(axis=-1, keepdims=True)
+    p = np.exp(logits)
+    return p / p.sum(axis=-1, keepdims=True)
+
+
+@pytest.mark.parametrize("B,H,L,D,mask,rank,seed", [
+    (2, 4, 128, 32, "none", 2, 3 * 128 + 32), (2, 16, 256, 24, "tail", 1, 3 * 256 + 24), (3, 4, 200, 32, "random", 2, 3 * 200 + 32),
+    (1, 2, 37, 24, "random", 1, 3 * 37 + 24), (2, 2, 130, 48, "tail", 2, 3 * 130 + 48), (1, 16, 1536, 24, "tail", 1, 3 * 1536 + 24)])
+def test_fp8_short_row_error_budget_is_the_e4m3_rounding_of_p_and_v(oracle, B, H, L, D, mask, rank, seed):
+    """Where the 0.15 max-abs bound of the fp8 GPU test on short rows (L < 1024) comes from: with q and k exact, rounding
+    only V (per-tensor power-of-two scale) and the probabilities (P * 2^8, as the fp8 kernel feeds them to its second
+    product) to e4m3 already moves the result by more than the 6e-2 of the diffusion-sized case on each of these short
+    inputs (0.07 - 0.10; rounding V alone: 0.064 - 0.107), and by less than 0.15; at L = 1536, where many keys share the
+    weight, the same two roundings stay inside 6e-2.  Same seeds and shapes as
+    tests/test_dpa_gpu.py::test_fp8_mfma_matches_formula."""
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = [torch.randn(B, H, L, D, generator=g).to(torch.bfloat16).float().numpy() for _ in range(3)]
+    bias = torch.randn(H, L, L, generator=g).to(torch.bfloat16).float().numpy()
+    if mask == "none":
+        m = torch.ones(B, L, dtype=torch.bool)
+    elif mask == "random":
+        m = torch.rand(B, L, generator=g) < 0.7
+        m[:, 0] = True
+    else:
+        m = torch.ones(B, L, dtype=torch.bool)
+        m[:, L - max(1, L // 10):] = False
+    m = m.numpy()
+    if rank == 1:
+        m = np.broadcast_to(m[0], (B, L))
+    logits = np.einsum("bhqd,bhkd->bhqk", q.astype(np.float64) * D ** -0.5, k.astype(np.float64)) + bias[None]
+    logits = np.where(m[:, None, None, :], logits, -1e9)
+    p = _softmax_rows(logits)
+    exact = np.einsum("bhqk,bhkd->bhqd", p, v.astype(np.float64))
+    assert np.abs(exact - oracle.dpa_formula(q, k, v, m, bias)).max() < 1e-5     # this restatement is the pinned formula
+    v8 = oracle.fake_quantize_e4m3_pow2(v).astype(np.float64)
+    p8 = torch.from_numpy((p * 256.0).astype(np.float32)).to(torch.float8_e4m3fn).float().numpy().astype(np.float64)
+    sim = np.einsum("bhqk,bhkd->bhqd", p8, v8) / p8.sum(axis=-1, keepdims=True)
+    err = np.abs(sim - exact).max()
+    if L < 1024:
+        assert 6e-2 < err <= 0.15, err      # no e4m3 kernel can meet 6e-2 here: the format's rounding of V alone exceeds it
+    else:
+        assert err <= 6e-2, err
+
+
 def test_vnni_repack_is_a_view_permute_per_panel(oracle):
     rng = np.random.default_rng(14)
     M, N, blk = 16, 24, 8

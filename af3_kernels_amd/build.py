@@ -1,5 +1,4 @@
-"""Builds libaf3_dpa.so (hand-written HIP for gfx950) in-tree with hipcc, and beside it libaf3_microbench.so
-(the microbenchmarks of af3_kernels_amd/microbench.py; nothing in the product library depends on it).
+"""Builds libaf3_dpa.so (hand-written HIP for gfx950) in-tree with hipcc.
 
     python -m af3_kernels_amd.build [--force]
 
@@ -14,7 +13,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJDIR = os.path.join(CSRC, "_obj")
 LIB = os.path.join(HERE, "libaf3_dpa.so")
-MICROBENCH_LIB = os.path.join(HERE, "libaf3_microbench.so")
 SOURCES = ["api.hip", "dpa_generic.hip", "dpa_mfma.hip", "dpa_mfma_f32.hip", "dpa_mfma_fp8.hip", "elementwise.hip", "pair_bias.hip", "glu.hip"]
 HEADERS = [os.path.join(CSRC, "common.hpp"), os.path.join(HERE, "..", "include", "af3_dpa.h")]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -47,14 +45,13 @@ def _compile(src, force):
 def build(force=False, verbose=False):
     os.makedirs(OBJDIR, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES) + 1)) as ex:
-        objs = list(ex.map(lambda s: _compile(s, force), SOURCES + ["microbench.hip"]))
-    for lib, members in ((LIB, objs[:-1]), (MICROBENCH_LIB, objs[-1:])):
-        if force or _stale(lib, members):
-            r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + members, capture_output=True, text=True)
-            if r.returncode != 0:
-                raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
-        if verbose:
-            print("built", lib)
+        objs = list(ex.map(lambda s: _compile(s, force), SOURCES))
+    if force or _stale(LIB, objs):
+        r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
+    if verbose:
+        print("built", LIB)
     return LIB
 
 

@@ -2,7 +2,32 @@
 // Declared in include/af3_dpa.h.  Nothing here allocates, synchronises or exits.
 #include "common.hpp"
 
+#include <atomic>
+#include <string.h>
+
 using namespace af3;
+
+int af3::current_device_status() {
+	constexpr int       MAX_DEV = 64;
+	static std::atomic<signed char> known[MAX_DEV];  // 0 = not asked yet, 1 = gfx950, -1 = anything else
+	int dev = -1;
+	if(hipGetDevice(&dev) != hipSuccess) {
+		(void)hipGetLastError();
+		return AF3_ERR_NO_DEVICE_CODE;  // no usable device at all
+	}
+	if(dev >= 0 && dev < MAX_DEV) {
+		const signed char c = known[dev].load(std::memory_order_relaxed);
+		if(c != 0) return c > 0 ? AF3_OK : AF3_ERR_NO_DEVICE_CODE;
+	}
+	hipDeviceProp_t prop;
+	if(hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+		(void)hipGetLastError();
+		return AF3_ERR_NO_DEVICE_CODE;
+	}
+	const bool ok = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+	if(dev >= 0 && dev < MAX_DEV) known[dev].store(ok ? 1 : -1, std::memory_order_relaxed);
+	return ok ? AF3_OK : AF3_ERR_NO_DEVICE_CODE;
+}
 
 namespace {
 
@@ -73,6 +98,7 @@ extern "C" int af3_dpa_select_kernel(const af3_dpa_params* params) {
 extern "C" int af3_dpa_forward(const af3_dpa_params* params, void* hip_stream) {
 	const int rc = validate(params);
 	if(rc != AF3_OK) return rc;
+	if(const int dc = current_device_status(); dc != AF3_OK) return dc;
 	hipStream_t s = static_cast<hipStream_t>(hip_stream);
 	switch(select_kernel(*params)) {
 		case 0: return launch_dpa_generic(*params, s);
@@ -103,6 +129,8 @@ extern "C" int af3_grid_attention_forward(const af3_grid_attention_params* g, vo
 	const int rc = validate_grid(g);
 	if(rc != AF3_OK) return rc;
 	if(!grid_fused_eligible(*g)) return AF3_ERR_BAD_ARGUMENT;
+	if(g->bias && (!g->workspace || g->workspace_bytes < grid_fused_workspace_bytes(*g) || (reinterpret_cast<uintptr_t>(g->workspace) & 15))) return AF3_ERR_BAD_ARGUMENT;
+	if(const int dc = current_device_status(); dc != AF3_OK) return dc;
 	return launch_grid_fused(*g, static_cast<hipStream_t>(hip_stream));
 }
 
@@ -116,7 +144,7 @@ extern "C" const char* af3_status_string(int status) {
 		case AF3_ERR_UNSUPPORTED_D: return "head_dim exceeds the supported maximum (128)";
 		case AF3_ERR_LAUNCH: return "kernel launch failed";
 		case AF3_ERR_BAD_ARGUMENT: return "invalid argument";
-		case AF3_ERR_NO_DEVICE_CODE: return "this library only carries gfx950 code";
+		case AF3_ERR_NO_DEVICE_CODE: return "the current device is not a gfx950 (MI355X); this library carries code for nothing else";
 		default: return "unknown status";
 	}
 }

@@ -51,6 +51,17 @@ struct fused_grid_args {
 	const void *    wq, *wk, *wv, *wg;
 };
 
+// Status of the launch just enqueued.  A device this library carries no code for (anything but gfx950) shows up
+// here as "no binary for this GPU" / "invalid device function" and is reported as such, not as a generic launch failure.
+inline int launch_status() {
+	const hipError_t e = hipGetLastError();
+	if(e == hipSuccess) return AF3_OK;
+	return (e == hipErrorNoBinaryForGpu || e == hipErrorInvalidDeviceFunction || e == hipErrorSharedObjectInitFailed || e == hipErrorNoDevice) ? AF3_ERR_NO_DEVICE_CODE : AF3_ERR_LAUNCH;
+}
+// AF3_OK when the calling thread's current device is a gfx950, AF3_ERR_NO_DEVICE_CODE otherwise (api.hip; one
+// property query per device and process, then a table lookup).
+int current_device_status();
+
 // Launchers implemented in the .hip files; all validated by api.hip before the call.
 int launch_dpa_generic(const af3_dpa_params& p, hipStream_t s);
 int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s);

@@ -58,7 +58,7 @@ __global__ void __launch_bounds__(GEN_WAVES * 64) dpa_generic_kernel(af3_dpa_par
 			const int64_t kr  = koff + key * p.k_stride[2];
 			float s = 0.f;
 			for(int d = 0; d < D; d++) s = fmaf(qs[wave][d], load_as_f32(p.k, kr + d, p.io_dtype), s);
-			if(p.bias) s += load_as_f32(p.bias, boff + key, p.bias_dtype);
+			if(p.bias) s = fmaxf(s + load_as_f32(p.bias, boff + key, p.bias_dtype), -3.0e38f);  // (-inf in the bias: finite, so that a chunk of such keys leaves a finite maximum)
 			if(keep && !keep[key]) s = MASK_DROPPED;  // masked_fill semantics: the logit is replaced
 			pbuf[wave][j] = s;
 			cmax = fmaxf(cmax, s);
@@ -106,7 +106,7 @@ int launch_dpa_generic(const af3_dpa_params& p, hipStream_t s) {
 	const int64_t blocks      = p.B * p.H * rows_per_bh;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
 	hipLaunchKernelGGL(dpa_generic_kernel, dim3((unsigned)blocks), dim3(GEN_WAVES * 64), 0, s, p);
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 }  // namespace af3

@@ -86,6 +86,20 @@ __device__ __forceinline__ void load_bias8_guarded(const void* bias_row, int64_t
 	}
 }
 
+// A bias fragment that rides the identity MFMA meets 0 in every other contraction slot, and 0 * -inf is NaN: an
+// additive -inf (a mask folded into the bias) is therefore replaced by -2^126 before the product (every bias below
+// that, and the -NaN patterns, likewise), which gives that key weight exactly 0 like the reference's add-then-softmax;
+// -2^126 rather than the most negative finite value so that the product with log2 e stays finite when a row's first
+// keys all carry it and it becomes the softmax reference for a while.  +inf and +NaN pass through and yield NaN, as
+// they do in the reference.  One packed unsigned minimum per dword.
+typedef __attribute__((ext_vector_type(2))) unsigned short u16x2;
+__device__ __forceinline__ u32x4 bias_frag_finite(u32x4 w) {
+	const u16x2 lim = {(unsigned short)0xFE80, (unsigned short)0xFE80};
+#pragma unroll
+	for(int j = 0; j < 4; j++) w[j] = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, w[j]), lim));
+	return w;
+}
+
 __device__ __forceinline__ float half_swap_max(float x) {
 	// lanes l and l^32 exchange; v_permlane32_swap swaps the upper half of one operand with the
 	// lower half of the other, so (x, x) yields {low|low} and {high|high}.
@@ -139,9 +153,10 @@ __global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restric
 // (explicit s_waitcnt vmcnt before the barrier that publishes a tile).  rsrc and lds_addr must be
 // wave-uniform.  The whole byte offset travels in the vector operand, which the hardware range-checks
 // against the buffer size: a lane whose offset is past the end fetches nothing from memory.
-// M0 (the LDS base of the load) is written behind the compiler's back: nothing else in this file
-// makes it use M0 -- no LDS-direct builtins, no indirect register indexing -- and gfx950's LDS
-// instructions do not read it.
+// M0 (the LDS base of the load) is written behind the compiler's back.  It cannot be declared: the compiler treats
+// M0 as a reserved register and answers an "m0" clobber with a warning that it is ignored.  What keeps this safe is
+// that nothing else in this file makes the compiler use M0 -- no LDS-direct builtins, no indirect register indexing,
+// no message or GWS instructions -- and gfx950's LDS instructions do not read it.
 __device__ __forceinline__ void lds_dma_b128(const u32x4& rsrc, uint32_t lds_addr, int voff) {
 	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
 }
@@ -553,7 +568,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 				const uint16_t* bp = reinterpret_cast<const uint16_t*>(bias_row) + key0;
 				if(row_ok) {
 #pragma unroll
-					for(int f = 2 * SUB; f < 2 * SUB + 2; f++) bfrag[f] = *reinterpret_cast<const u32x4*>(bp + 16 * f);
+					for(int f = 2 * SUB; f < 2 * SUB + 2; f++) bfrag[f] = bias_frag_finite(*reinterpret_cast<const u32x4*>(bp + 16 * f));
 				} else {
 #pragma unroll
 					for(int f = 2 * SUB; f < 2 * SUB + 2; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
@@ -565,6 +580,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 					load_bias8_guarded<BIAS_F32>(bias_row, key0 + 16 * f, L, row_ok, v8);
 #pragma unroll
 					for(int j = 0; j < 4; j++) bfrag[f][j] = pack_bf16x2(v8[2 * j], v8[2 * j + 1]);
+					bfrag[f] = bias_frag_finite(bfrag[f]);
 				}
 			}
 		};
@@ -731,7 +747,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		auto read_bias_ring = [&](int slot_off, auto sub_c) {
 			constexpr int SUB = decltype(sub_c)::value;
 #pragma unroll
-			for(int c2 = 0; c2 < 2; c2++) bfrag[2 * SUB + c2] = *reinterpret_cast<const u32x4*>(bring + slot_off + (b_rd ^ ((4 * SUB + 2 * c2) << 4)));
+			for(int c2 = 0; c2 < 2; c2++) bfrag[2 * SUB + c2] = bias_frag_finite(*reinterpret_cast<const u32x4*>(bring + slot_off + (b_rd ^ ((4 * SUB + 2 * c2) << 4))));
 		};
 		// ring_off (BRING): byte offset of the ring slot that holds the bias tile of sub-tile j+1
 		auto stage = [&](auto subn_c, int k_off, int mask_addr_next, int v_off, auto subc_c, int bias_kt, auto bias_sub_c, int ring_off) {
@@ -1052,7 +1068,7 @@ static int launch_bias_prepass(const af3_dpa_params& p, hipStream_t s) {
 	else
 		hipLaunchKernelGGL(bias_prepass_kernel<false>, dim3(g), dim3(256), 0, s, p.bias, static_cast<u32x4*>(p.workspace), p.H, p.L, p.bias_stride[0], p.bias_stride[1], n_qblocks,
 						   n_ktiles, vec_ok);
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 constexpr size_t LDS_LIMIT = 160 * 1024;  // per workgroup on gfx950
@@ -1080,7 +1096,7 @@ static int launch_one(const af3_dpa_params& p, hipStream_t s) {
 		if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
 	}
 	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, n_qtiles, n_groups, fused_grid_args{});
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 // ---- fused grid attention: projections + attention + gate in one kernel ----
@@ -1129,7 +1145,7 @@ static int launch_fused_nw(const af3_dpa_params& p, const fused_grid_args& fa, h
 	auto         kern = dpa_mfma_bf16_kernel<32, NW, true, 0, false, true, false>;
 	if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
 	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, 1, n_groups, fa);
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 int launch_grid_fused(const af3_grid_attention_params& g, hipStream_t s) {

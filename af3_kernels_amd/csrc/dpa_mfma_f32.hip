@@ -192,7 +192,8 @@ __global__ void __launch_bounds__(F32_NW * 64) dpa_mfma_f32_kernel(af3_dpa_param
 #pragma unroll
 			for(int e = 0; e < 4; e++) {
 				const uint32_t v = (st >> (8 * e)) & 0xffu;
-				const float    x = v == 1u ? s[4 * r4 + e] : (v == 0u ? -1.0e9f : -INFINITY);
+				// (a live key whose bias is -inf keeps a finite logit, so that a tile of such keys leaves a finite maximum)
+				const float    x = v == 1u ? fmaxf(s[4 * r4 + e], -3.0e38f) : (v == 0u ? -1.0e9f : -INFINITY);
 				s[4 * r4 + e]    = x;
 				mx               = fmaxf(mx, x);
 			}
@@ -259,7 +260,7 @@ int launch(const af3_dpa_params& p, hipStream_t s) {
 	if(grid > 0x7fffffff) return AF3_ERR_BAD_SHAPE;
 	const size_t smem = (size_t)4 * F32_KT * (DP + 4) * 4 + (size_t)n_tiles * F32_KT + (size_t)n_tiles * 2 + 16;
 	hipLaunchKernelGGL(dpa_mfma_f32_kernel<DP>, dim3((unsigned)grid), dim3(F32_NW * 64), smem, s, p, n_qtiles, groups);
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 }  // namespace

@@ -356,7 +356,7 @@ int launch8(const af3_dpa_params& p, hipStream_t s) {
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
 	const size_t smem = (size_t)(COMP ? 6 : 4) * KT8 * DP + ((size_t)n_ktiles * KT8 + 64) * 4 + (size_t)n_ktiles * 2 + 16;
 	hipLaunchKernelGGL((dpa_mfma_fp8_kernel<DP, COMP>), dim3((unsigned)blocks), dim3(NW8 * 64), smem, s, p, n_qtiles, n_groups);
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 }  // namespace

@@ -286,7 +286,7 @@ extern "C" int af3_convert(const void* src, int32_t sd, void* dst, int32_t dd, i
 		hipLaunchKernelGGL(cvt_e4m3_kernel<true>, dim3(ew_blocks((n + 3) / 4)), dim3(EW_THREADS), 0, s, static_cast<const uint8_t*>(src), dst, n);
 	else
 		return AF3_ERR_BAD_DTYPE;
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 extern "C" int af3_amax(const void* src, int32_t sd, int64_t n, float* amax_out, void* stream) {
@@ -297,7 +297,7 @@ extern "C" int af3_amax(const void* src, int32_t sd, int64_t n, float* amax_out,
 	if(sd == AF3_F32) hipLaunchKernelGGL(amax_kernel<false>, dim3(ew_blocks((n + 7) / 8, 512)), dim3(EW_THREADS), 0, s, src, n, amax_out);
 	else if(sd == AF3_BF16) hipLaunchKernelGGL(amax_kernel<true>, dim3(ew_blocks((n + 7) / 8, 512)), dim3(EW_THREADS), 0, s, src, n, amax_out);
 	else return AF3_ERR_BAD_DTYPE;
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 extern "C" int af3_quantize_fp8_e4m3(const void* src, int32_t sd, void* dst, int64_t rows, int64_t cols, int64_t src_row_stride, int32_t transpose_last2,
@@ -326,7 +326,7 @@ extern "C" int af3_quantize_fp8_e4m3(const void* src, int32_t sd, void* dst, int
 						   rows_per_matrix, dst_row_stride, pre_scale, amax, descale_out, static_cast<uint8_t*>(dst_residual));
 	else
 		return AF3_ERR_BAD_DTYPE;
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 extern "C" int af3_quantize_qkv_fp8_e4m3(const void* q, const void* k, const void* v, int32_t sd, int64_t B, int64_t H, int64_t L, int64_t D, float q_pre_scale, void* q8,
@@ -357,7 +357,7 @@ extern "C" int af3_quantize_qkv_fp8_e4m3(const void* q, const void* k, const voi
 		hipLaunchKernelGGL(amax3_kernel<true>, ga, dim3(EW_THREADS), 0, s, aa, scratch);
 		hipLaunchKernelGGL(quantize3_kernel<true>, gq, dim3(EW_THREADS), 0, s, qa, scratch, descales);
 	}
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 extern "C" int af3_pad_nd(const void* src, void* dst, int32_t ndim, const int64_t* src_shape, const int64_t* src_strides, const int64_t* dst_shape,
@@ -386,7 +386,7 @@ extern "C" int af3_pad_nd(const void* src, void* dst, int32_t ndim, const int64_
 		hipLaunchKernelGGL(pad_nd_kernel<uint8_t>, dim3(g), dim3(EW_THREADS), 0, s, static_cast<const uint8_t*>(src), static_cast<uint8_t*>(dst), d, total, (uint8_t)fill_bits);
 	else
 		return AF3_ERR_BAD_DTYPE;
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 extern "C" int af3_vnni_repack_bf16(const void* src, void* dst, int64_t M, int64_t N, int64_t blk, void* stream) {
@@ -397,5 +397,5 @@ extern "C" int af3_vnni_repack_bf16(const void* src, void* dst, int64_t M, int64
 	if(blk < 0 || N % blk != 0 || (M & 1)) return AF3_ERR_BAD_ARGUMENT;
 	hipLaunchKernelGGL(vnni_repack_kernel, dim3(ew_blocks(M * N)), dim3(EW_THREADS), 0, static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(src),
 					   static_cast<uint16_t*>(dst), M, N, blk);
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }

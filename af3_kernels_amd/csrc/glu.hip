@@ -190,7 +190,7 @@ int launch_rows_times_weights(const void* x, const void* weight_t, void* out, in
 		if(K == 128) gated ? go(glu_kernel<8, GLU_MAX_WAVES, true>, GLU_MAX_WAVES) : go(glu_kernel<8, GLU_MAX_WAVES, false>, GLU_MAX_WAVES);
 		else gated ? go(glu_kernel<4, GLU_MAX_WAVES, true>, GLU_MAX_WAVES) : go(glu_kernel<4, GLU_MAX_WAVES, false>, GLU_MAX_WAVES);
 	}
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }
 
 }  // namespace

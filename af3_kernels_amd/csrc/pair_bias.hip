@@ -125,5 +125,5 @@ extern "C" int af3_layernorm_pair_bias(const void* pair, const int64_t* pair_str
 	hipLaunchKernelGGL(layernorm_pair_bias_kernel, dim3((unsigned)blocks), dim3(PB_WAVES * 64), 0, static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(pair), pair_stride[0],
 					   pair_stride[1], static_cast<const uint16_t*>(ln_weight), static_cast<const uint16_t*>(ln_bias), static_cast<const uint16_t*>(proj_weight), eps,
 					   static_cast<uint16_t*>(normed), static_cast<uint16_t*>(bias), n_i, n_j, bias_stride[0], bias_stride[1]);
-	return hipGetLastError() == hipSuccess ? AF3_OK : AF3_ERR_LAUNCH;
+	return launch_status();
 }

@@ -47,23 +47,38 @@ def _unpack_panels(w: torch.Tensor, head: int) -> torch.Tensor:
     return w.reshape(head, C, K).permute(1, 0, 2).reshape(C, C)
 
 
+def _layout(t: torch.Tensor):
+    return (t.data_ptr(), t.storage_offset(), tuple(t.shape), tuple(t.stride()), t.dtype)
+
+
 def _cached(sources, extra, make):
     """make()'s result, remembered for as long as the source tensors are the same live objects at the same
-    version (an in-place update bumps the version; a freed tensor's address or id may be reused by another
-    tensor, which the weak references tell apart)."""
+    version, address and layout (an in-place update bumps the version; set_() or a resize moves the address or
+    layout; a freed tensor's id may be reused by another tensor, which the weak references tell apart).
+    Writes that bypass the version counter -- `weight.data.copy_(...)`, a foreign kernel writing the storage --
+    cannot be seen from here: call clear_weight_cache() after them."""
     key = tuple(id(t) for t in sources) + extra
     hit = _W_CACHE.get(key)
+    state = tuple((t._version,) + _layout(t) for t in sources)
     if hit is not None:
-        refs, versions, value = hit
-        if all(r() is t for r, t in zip(refs, sources)) and versions == tuple(t._version for t in sources):
+        refs, seen, value = hit
+        if all(r() is t for r, t in zip(refs, sources)) and seen == state:
             return value
-    for k in [k for k, (refs, _, _) in _W_CACHE.items() if any(r() is None for r in refs)]:
-        del _W_CACHE[k]                      # derived matrices of weights that no longer exist
+    for k in [k for k, (refs, _, _) in list(_W_CACHE.items()) if any(r() is None for r in refs)]:
+        _W_CACHE.pop(k, None)                # derived matrices of weights that no longer exist
     if len(_W_CACHE) >= _W_CACHE_MAX:
         _W_CACHE.clear()
     value = make()
-    _W_CACHE[key] = (tuple(weakref.ref(t) for t in sources), tuple(t._version for t in sources), value)
+    _W_CACHE[key] = (tuple(weakref.ref(t) for t in sources), state, value)
     return value
+
+
+def clear_weight_cache() -> None:
+    """Forgets every matrix derived from a weight tensor (the fused [4C, C] projection, the transposed output
+    projection, the gated linear unit's weight^T).  Needed only after weights were overwritten in a way that
+    does not bump the tensor's version counter, e.g. `module.weight.data.copy_(new)`; ordinary in-place
+    updates (`copy_`, `load_state_dict`, optimiser steps) are noticed without it."""
+    _W_CACHE.clear()
 
 
 def _fused_weight(ws, head: int, dtype: torch.dtype) -> torch.Tensor:

@@ -29,7 +29,8 @@ typedef enum af3_status {
 	AF3_ERR_UNSUPPORTED_D  = -5, /* head_dim above the supported maximum */
 	AF3_ERR_LAUNCH         = -6, /* hipGetLastError() reported a launch failure */
 	AF3_ERR_BAD_ARGUMENT   = -7, /* any other invalid argument (e.g. N % BLK_SZ != 0) */
-	AF3_ERR_NO_DEVICE_CODE = -8  /* the GPU in use is not gfx950 */
+	AF3_ERR_NO_DEVICE_CODE = -8  /* the current device is not a gfx950 (host-side check before the launch, or the
+	                                 runtime reporting that it has no code object for the device) */
 } af3_status;
 
 typedef enum af3_dtype {

@@ -368,6 +368,28 @@ def test_logits_far_above_the_first_tile_move_the_reference(af3, oracle):
         af3.set_exact_bias(prev)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+def test_minus_infinity_in_the_bias_gives_that_key_weight_zero(af3, oracle, dtype):
+    """An additive -inf (a mask folded into the bias) must act like the reference's add-then-softmax: weight 0 for that
+    (query, key), every other key of the row unaffected, no NaN.  Covers the in-place bias (B = 1, and B >= 2 with
+    set_exact_bias) and the rewritten-bias workspace (B >= 2), at entries spread over several tiles."""
+    B, H, L, D = 3, 2, 200, 32
+    q, k, v, m, bias = rand_inputs(B, H, L, D, dtype, seed=77, mask="random")
+    g = torch.Generator().manual_seed(78)
+    hole = torch.rand(H, L, L, generator=g) < 0.2
+    hole[:, :, 0] = False                       # key 0 is live in every batch row: no row loses all its keys
+    hole[0, 3, 1:] = True                       # a query row left with key 0 alone
+    hole[1, 5, :40] = True                      # a query row whose first tile is all -inf (key 0 included: only here)
+    bias = bias.masked_fill(hole, float("-inf"))
+    run_case(af3, oracle, q, k, v, m, bias)                                  # B >= 2: bias workspace
+    run_case(af3, oracle, q[:1], k[:1], v[:1], m[:1], bias)                  # B = 1: bias read in place
+    prev = af3.set_exact_bias(True)
+    try:
+        run_case(af3, oracle, q, k, v, m, bias)                              # B >= 2, in place
+    finally:
+        af3.set_exact_bias(prev)
+
+
 def test_length_beyond_the_matrix_core_limit_uses_the_fma_kernel(af3):
     """L > 8192 is outside the matrix-core kernel's mask table; the call must still work (fp32-FMA
     kernel) -- checked through rows summing to one and against a torch reference on a slice."""

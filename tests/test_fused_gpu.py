@@ -486,16 +486,3 @@ def test_fused_callers_can_be_captured_in_a_hip_graph_and_replayed(af3):
             torch.cuda.synchronize()
             for a, b in zip(outs, eager):
                 assert torch.equal(a, b), f"replay {rep} differs from the eager call"
-
-
-def test_microbenchmarks_run(af3, capsys):
-    """The design notes' microbenchmarks (separate library) load and run; their timings are not asserted."""
-    from af3_kernels_amd import microbench
-    r = microbench.Runner()
-    n_cu = torch.cuda.get_device_properties(0).multi_processor_count
-    for which, variant, grid, threads in ((0, 0, n_cu, 1024), (0, 2, n_cu, 1024), (1, 0, 4 * n_cu, 256), (1, 7, 4 * n_cu, 256), (1, 16, 2 * n_cu, 256), (2, 0, 512, 256)):
-        assert r.ns_per_trip(which, variant, grid, threads, 20, reps=1) > 0
-    with pytest.raises(RuntimeError):
-        r.ns_per_trip(1, 5, 8, 256, 20)           # not a built variant
-    with pytest.raises(RuntimeError):
-        r.ns_per_trip(1, 0, 8, 256, 21)           # odd trip count

@@ -342,3 +342,29 @@ def test_derived_weight_cache_follows_tensor_identity_and_version():
     fused._W_CACHE[key] = ((weakref.ref(dead),), (dead._version,), "stale")
     got = derive(t)
     assert not isinstance(got, str) and torch.equal(got, t)
+    # a tensor whose storage was swapped under the same object and version (set_) is seen through its address
+    u = torch.arange(4.0)
+    first = derive(u)
+    u.set_(torch.arange(4.0) + 10.0)
+    second = derive(u)
+    assert second is not first and torch.equal(second, u)
+    # a write that bypasses the version counter cannot be seen; clear_weight_cache() is the documented remedy
+    n = len(calls)
+    u.data.copy_(torch.zeros(4))
+    assert derive(u) is second and len(calls) == n
+    fused.clear_weight_cache()
+    third = derive(u)
+    assert len(calls) == n + 1 and torch.equal(third, torch.zeros(4))
+
+
+def test_no_device_is_reported_as_such_before_anything_is_launched():
+    """Without a gfx950 as the current device (this test runs where there is no GPU at all) a well-formed call
+    returns AF3_ERR_NO_DEVICE_CODE from the host-side check; nothing is enqueued."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present: the arch check passes here")
+    from af3_kernels_amd import _lib
+    lib = _lib.load()
+    assert lib.af3_dpa_forward(ctypes.byref(_params()), None) == -8
+    with pytest.raises(RuntimeError, match="gfx950"):
+        _lib.check(-8, "af3_dpa_forward")

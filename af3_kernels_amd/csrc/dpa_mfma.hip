@@ -96,7 +96,10 @@ typedef __attribute__((ext_vector_type(2))) unsigned short u16x2;
 __device__ __forceinline__ u32x4 bias_frag_finite(u32x4 w) {
 	const u16x2 lim = {(unsigned short)0xFE80, (unsigned short)0xFE80};
 #pragma unroll
-	for(int j = 0; j < 4; j++) w[j] = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, w[j]), lim));
+	for(int j = 0; j < 4; j++) {
+		const uint32_t x = w[j];  // (a copy: __builtin_bit_cast applied to the vector element itself reads element 0 with this compiler)
+		w[j] = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, x), lim));
+	}
 	return w;
 }
 

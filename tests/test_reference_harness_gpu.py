@@ -63,4 +63,4 @@ def test_reference_harness_preset(oracle, set_size):
     diff, ref_diff = num / den, ref_num / den               # the harness's "Diff" (as a fraction)
     print(f"  Diff {100 * diff:.5f} %   (reference arithmetic restated on the CPU: {100 * ref_diff:.5f} %)", flush=True)
     assert diff <= 2.0 * ref_diff + 1e-6, (diff, ref_diff)
-XX
+    assert diff <= 5e-3                                      # measured 0.17 - 0.21 %; the reference's bf16 logits alone cost 1.3 - 2.4 % here

@@ -9,7 +9,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libaf3_dpa.so")
 
 AF3_F32, AF3_BF16, AF3_FP8_E4M3 = 0, 1, 2
-ABI_VERSION = 3
+ABI_VERSION = 4
+STATIC_SCRATCH_BYTES = 16 * 1024 * 1024   # AF3_STATIC_SCRATCH_BYTES
 
 i64, i32, f32, vp = ctypes.c_int64, ctypes.c_int32, ctypes.c_float, ctypes.c_void_p
 
@@ -49,6 +50,7 @@ QKV_SCRATCH_FLOATS = 768   # AF3_QKV_SCRATCH_FLOATS
 # name -> (restype, argtypes); every symbol include/af3_dpa.h declares
 SYMBOLS = {
     "af3_dpa_forward": (ctypes.c_int, [ctypes.POINTER(DpaParams), vp]),
+    "af3_dpa_forward_static_scratch": (ctypes.c_int, [ctypes.POINTER(DpaParams), vp]),
     "af3_dpa_select_kernel": (ctypes.c_int, [ctypes.POINTER(DpaParams)]),
     "af3_dpa_workspace_bytes": (ctypes.c_int64, [ctypes.POINTER(DpaParams)]),
     "af3_grid_attention_forward": (ctypes.c_int, [ctypes.POINTER(GridAttentionParams), vp]),
@@ -90,5 +92,5 @@ def load():
 def check(status: int, what: str):
     if status != 0:
         msg = load().af3_status_string(status).decode()
-        exc = ValueError if status in (-2, -3, -4, -5, -7) else RuntimeError
+        exc = ValueError if status in (-2, -3, -4, -5, -7, -9) else RuntimeError
         raise exc(f"{what}: {msg} (af3_status {status})")

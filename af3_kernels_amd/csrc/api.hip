@@ -95,6 +95,53 @@ extern "C" int af3_dpa_select_kernel(const af3_dpa_params* params) {
 	return select_kernel(*params);
 }
 
+// ---- the allocation-free entry point's scratch: a device array inside the code object, one copy per GPU ----
+// In host code the array's name is only a handle for hipGetSymbolAddress; the address that kernels and copies may use
+// is looked up once per device (with that device current) and kept here.
+static __device__ __align__(256) unsigned char scratch[AF3_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int        SCRATCH_MAX_DEV = 64;
+std::atomic<void*>   scratch_ptr[SCRATCH_MAX_DEV];
+
+// device address of `scratch` on the current device, or nullptr with *status set
+void* static_scratch_address(int* status) {
+	int dev = -1;
+	if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SCRATCH_MAX_DEV) {
+		(void)hipGetLastError();
+		*status = AF3_ERR_NO_DEVICE_CODE;
+		return nullptr;
+	}
+	void* ptr = scratch_ptr[dev].load(std::memory_order_acquire);
+	if(ptr) return ptr;
+	const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));  // (two threads may both ask: they get the same answer)
+	if(e != hipSuccess || !ptr) {
+		(void)hipGetLastError();
+		*status = (e == hipErrorNoBinaryForGpu || e == hipErrorInvalidDeviceFunction || e == hipErrorSharedObjectInitFailed) ? AF3_ERR_NO_DEVICE_CODE : AF3_ERR_LAUNCH;
+		return nullptr;
+	}
+	scratch_ptr[dev].store(ptr, std::memory_order_release);
+	return ptr;
+}
+}  // namespace
+
+extern "C" int af3_dpa_forward_static_scratch(const af3_dpa_params* params, void* hip_stream) {
+	const int rc = validate(params);
+	if(rc != AF3_OK) return rc;
+	af3_dpa_params p = *params;
+	p.workspace = nullptr, p.workspace_bytes = 0;
+	const int64_t need = select_kernel(p) == 1 ? mfma_bf16_workspace_bytes(p) : 0;
+	if(need > (int64_t)AF3_STATIC_SCRATCH_BYTES) return AF3_ERR_SCRATCH_LIMIT;
+	if(const int dc = current_device_status(); dc != AF3_OK) return dc;
+	if(need > 0) {
+		int   st  = AF3_OK;
+		void* ptr = static_scratch_address(&st);
+		if(!ptr) return st;
+		p.workspace = ptr, p.workspace_bytes = AF3_STATIC_SCRATCH_BYTES;
+	}
+	return af3_dpa_forward(&p, hip_stream);
+}
+
 extern "C" int af3_dpa_forward(const af3_dpa_params* params, void* hip_stream) {
 	const int rc = validate(params);
 	if(rc != AF3_OK) return rc;
@@ -144,9 +191,10 @@ extern "C" const char* af3_status_string(int status) {
 		case AF3_ERR_UNSUPPORTED_D: return "head_dim exceeds the supported maximum (128)";
 		case AF3_ERR_LAUNCH: return "kernel launch failed";
 		case AF3_ERR_BAD_ARGUMENT: return "invalid argument";
+		case AF3_ERR_SCRATCH_LIMIT: return "the call needs more scratch than the library's static scratch array holds (use af3_dpa_forward with a workspace)";
 		case AF3_ERR_NO_DEVICE_CODE: return "the current device is not a gfx950 (MI355X); this library carries code for nothing else";
 		default: return "unknown status";
 	}
 }
 
-extern "C" int af3_abi_version(void) { return 3; }
+extern "C" int af3_abi_version(void) { return 4; }

@@ -29,8 +29,10 @@ typedef enum af3_status {
 	AF3_ERR_UNSUPPORTED_D  = -5, /* head_dim above the supported maximum */
 	AF3_ERR_LAUNCH         = -6, /* hipGetLastError() reported a launch failure */
 	AF3_ERR_BAD_ARGUMENT   = -7, /* any other invalid argument (e.g. N % BLK_SZ != 0) */
-	AF3_ERR_NO_DEVICE_CODE = -8  /* the current device is not a gfx950 (host-side check before the launch, or the
+	AF3_ERR_NO_DEVICE_CODE = -8, /* the current device is not a gfx950 (host-side check before the launch, or the
 	                                 runtime reporting that it has no code object for the device) */
+	AF3_ERR_SCRATCH_LIMIT  = -9  /* af3_dpa_forward_static_scratch: the call needs more scratch than the library's
+	                                 built-in AF3_STATIC_SCRATCH_BYTES */
 } af3_status;
 
 typedef enum af3_dtype {
@@ -141,6 +143,22 @@ int af3_dpa_forward(const af3_dpa_params* params, void* hip_stream);
 /* Bytes of workspace the call would use (0 when a workspace would not help, e.g. B == 1,
  * no bias, or a kernel that does not take one); negative = af3_status error.  Host only. */
 int64_t af3_dpa_workspace_bytes(const af3_dpa_params* params);
+
+/*
+ * af3_dpa_forward for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and results as
+ * af3_dpa_forward called with a workspace of af3_dpa_workspace_bytes() bytes, except that params->workspace and
+ * params->workspace_bytes are ignored: the scratch (the rewritten bias of the bf16 kernel) lives in a device array of
+ * AF3_STATIC_SCRATCH_BYTES that is part of the library's code object, one copy per GPU for the life of the process.
+ * The call allocates and frees nothing.  A call that needs more scratch than that returns AF3_ERR_SCRATCH_LIMIT and
+ * enqueues nothing (H * ceil(L/32)^2 * 4 KiB must fit: e.g. 4 heads up to L = 1024, 16 heads up to L = 512); a call
+ * that needs none (one batch row, no bias, float32 or fp8 arithmetic) is af3_dpa_forward.  Every call on one GPU shares
+ * that GPU's array and overwrites all of it that it reads, so nothing needs clearing between calls, but calls that
+ * overlap in time on one GPU (two streams, two threads) race on it: serialise them, or give af3_dpa_forward separate
+ * workspaces instead.
+ */
+#define AF3_STATIC_SCRATCH_BYTES (16 * 1024 * 1024)
+int af3_dpa_forward_static_scratch(const af3_dpa_params* params, void* hip_stream);
 
 /* Which kernel af3_dpa_forward would run for these arguments: 0 = fp32 vector-FMA kernel,
  * 1 = bf16 MFMA kernel, 2 = fp8 MFMA kernel, 3 = fp32 MFMA kernel; negative = af3_status error.

@@ -30,17 +30,19 @@ struct Case {
 	const char* name;
 	int64_t     B, H, L, D;
 	int         dtype;      // AF3_F32 or AF3_BF16
-	bool        workspace;  // hand the library its optional scratch buffer
+	int         workspace;  // 0: none; 1: hand the library its optional scratch buffer; 2: af3_dpa_forward_static_scratch (the library's own array)
 	int         drop_tail;  // keys dropped at the end of every row of the last batch entry
 	double      tol;
 };
 
 const Case CASES[] = {
-	{"fp32 2x4x128x32 (fp32-FMA kernel)", 2, 4, 128, 32, AF3_F32, false, 16, 1e-4},
-	{"bf16 3x4x200x32 with workspace", 3, 4, 200, 32, AF3_BF16, true, 20, 2e-2},
-	{"bf16 3x4x200x32 without workspace", 3, 4, 200, 32, AF3_BF16, false, 20, 2e-2},
-	{"bf16 1x16x256x24 in-place bias", 1, 16, 256, 24, AF3_BF16, false, 13, 2e-2},
-	{"bf16 2x2x96x64", 2, 2, 96, 64, AF3_BF16, true, 0, 2e-2},
+	{"fp32 2x4x128x32 (fp32-FMA kernel)", 2, 4, 128, 32, AF3_F32, 0, 16, 1e-4},
+	{"bf16 3x4x200x32 with workspace", 3, 4, 200, 32, AF3_BF16, 1, 20, 2e-2},
+	{"bf16 3x4x200x32 without workspace", 3, 4, 200, 32, AF3_BF16, 0, 20, 2e-2},
+	{"bf16 1x16x256x24 in-place bias", 1, 16, 256, 24, AF3_BF16, 0, 13, 2e-2},
+	{"bf16 2x2x96x64", 2, 2, 96, 64, AF3_BF16, 1, 0, 2e-2},
+	{"bf16 5x4x300x32 static scratch", 5, 4, 300, 32, AF3_BF16, 2, 9, 2e-2},
+	{"bf16 3x4x200x32 static scratch (smaller call on the same array)", 3, 4, 200, 32, AF3_BF16, 2, 20, 2e-2},
 };
 
 // splitmix64 -> approximately normal values (sum of 4 uniforms), reproducible without <random>
@@ -116,12 +118,12 @@ int run(const Case& c, hipStream_t stream) {
 	p.softmax_scale = 1.0f / std::sqrt((float)c.D);
 	p.q_descale = p.k_descale = p.v_descale = 1.0f;
 	const int64_t ws = af3_dpa_workspace_bytes(&p);
-	if(c.workspace && ws > 0) {
+	if(c.workspace == 1 && ws > 0) {
 		HIP_OK(hipMalloc(&dws, (size_t)ws));
 		p.workspace = dws, p.workspace_bytes = ws;
 	}
 	const int kernel = af3_dpa_select_kernel(&p);
-	const int rc     = af3_dpa_forward(&p, stream);
+	const int rc     = c.workspace == 2 ? af3_dpa_forward_static_scratch(&p, stream) : af3_dpa_forward(&p, stream);
 	if(rc != AF3_OK) {
 		std::fprintf(stderr, "af3_dpa_forward: %s\n", af3_status_string(rc));
 		return 1;

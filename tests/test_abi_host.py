@@ -28,7 +28,7 @@ def test_host_program_links_the_library_and_lists_its_cases():
     r = subprocess.run([BIN, "--list"], capture_output=True, text=True, timeout=60)
     assert r.returncode == 0, r.stderr
     lines = r.stdout.strip().splitlines()
-    assert lines[0] == "abi version 3" and len(lines) >= 5
+    assert lines[0] == "abi version 4" and len(lines) >= 5
 
 
 @pytest.mark.gpu
@@ -38,4 +38,4 @@ def test_c_callers_get_the_formula_through_the_abi_alone():
     r = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr, flush=True)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count(" ok") >= 7 and "FAIL" not in r.stdout
+    assert r.stdout.count(" ok") >= 9 and "FAIL" not in r.stdout

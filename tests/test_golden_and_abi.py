@@ -368,3 +368,21 @@ def test_no_device_is_reported_as_such_before_anything_is_launched():
     assert lib.af3_dpa_forward(ctypes.byref(_params()), None) == -8
     with pytest.raises(RuntimeError, match="gfx950"):
         _lib.check(-8, "af3_dpa_forward")
+
+
+def test_static_scratch_entry_point_rejects_calls_beyond_its_limit_on_the_host():
+    """af3_dpa_forward_static_scratch: a call whose scratch need exceeds the library's built-in array returns
+    AF3_ERR_SCRATCH_LIMIT before anything touches a device; malformed calls return the usual codes."""
+    from af3_kernels_amd import _lib
+    lib = _lib.load()
+    fwd, need = lib.af3_dpa_forward_static_scratch, lib.af3_dpa_workspace_bytes
+    assert fwd(None, None) == -1
+    assert fwd(ctypes.byref(_params(L=0)), None) == -3
+    L = 2048
+    st = (ctypes.c_int64 * 3)(4 * L * 32, L * 32, 32)
+    big = _params(B=2, H=4, L=L, bias=0x1000, bias_stride=(ctypes.c_int64 * 2)(L * L, L), q_stride=st, k_stride=st, v_stride=st, out_stride=st)
+    assert need(ctypes.byref(big)) > _lib.STATIC_SCRATCH_BYTES
+    assert fwd(ctypes.byref(big), None) == -9
+    assert b"scratch" in lib.af3_status_string(-9)
+    with pytest.raises(ValueError):
+        _lib.check(-9, "x")

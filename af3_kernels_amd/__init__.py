@@ -27,11 +27,12 @@ from .ops import (  # noqa: F401
     reset_debug_timers,
     selected_kernel,
     set_exact_bias,
+    set_rows_kernel,
     vnni_repack_tensor,
 )
 
 __all__ = [
     "dot_product_attention_cpp", "dot_product_attention_fp8", "pad_and_align_tensor", "vnni_repack_tensor",
     "reset_debug_timers", "print_debug_timers", "print_debug_thread_imbalance", "convert", "quantize_fp8_e4m3",
-    "selected_kernel", "set_exact_bias", "_attention_cpp", "self_attention_cpp", "GridSelfAttentionCpp", "layernorm_pair_bias", "gated_linear_unit_cpp", "Linear", "clear_weight_cache",
+    "selected_kernel", "set_exact_bias", "set_rows_kernel", "_attention_cpp", "self_attention_cpp", "GridSelfAttentionCpp", "layernorm_pair_bias", "gated_linear_unit_cpp", "Linear", "clear_weight_cache",
 ]

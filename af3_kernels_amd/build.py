@@ -13,8 +13,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJDIR = os.path.join(CSRC, "_obj")
 LIB = os.path.join(HERE, "libaf3_dpa.so")
-SOURCES = ["api.hip", "dpa_generic.hip", "dpa_mfma.hip", "dpa_mfma_f32.hip", "dpa_mfma_fp8.hip", "elementwise.hip", "pair_bias.hip", "glu.hip"]
-HEADERS = [os.path.join(CSRC, "common.hpp"), os.path.join(HERE, "..", "include", "af3_dpa.h")]
+SOURCES = ["api.hip", "dpa_generic.hip", "dpa_mfma.hip", "dpa_mfma_rows.hip", "dpa_mfma_f32.hip", "dpa_mfma_fp8.hip", "elementwise.hip", "pair_bias.hip", "glu.hip"]
+HEADERS = [os.path.join(CSRC, "common.hpp"), os.path.join(CSRC, "mfma_helpers.hpp"), os.path.join(HERE, "..", "include", "af3_dpa.h")]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed-fp32 ops are switched off for device code; the host pass warns that it does not know
 # the feature, which is harmless.

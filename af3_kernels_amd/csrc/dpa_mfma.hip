@@ -44,37 +44,9 @@
 // :148-191 (the running max / sum recurrence); the harness formula
 // examples/dot_product_attention.py:20-43 for masking (dropped keys get weight 0, an all-dropped
 // row yields the mean of V).
-#include <type_traits>
-
-#include "common.hpp"
+#include "mfma_helpers.hpp"
 
 namespace af3 {
-
-constexpr int   KT         = 64;       // keys per tile
-constexpr int   MAX_L_MFMA = 8192;     // mask table (4 B/key) and tile list live in LDS
-constexpr float REF_SLACK  = 12.f;     // log2 units: a moved reference sits this close to the row maximum
-constexpr float PSUM_LIMIT = 0x1p30f;  // per-lane row-sum bound that triggers the rare path
-
-typedef __attribute__((ext_vector_type(2))) __bf16   bf16x2;
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
-typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
-template <int V>
-using ic = std::integral_constant<int, V>;
-
-// ---- LDS layout -----------------------------------------------------------------------------
-// K tile: [KT rows][DP cols] bf16; the 16-byte chunks of a row are XOR-swizzled so that the 8
-// lanes served in one LDS cycle of a ds_read_b128 (8 consecutive rows, same logical chunk) hit
-// distinct banks.  The swizzle only depends on row % 8.
-template <int DP>
-__device__ __forceinline__ int k_swizzle(int row) {
-	return (DP == 32) ? ((row >> 1) & 3) : (row & 7);
-}
-// V tile: [KT rows][DP cols] bf16 row-major; for DP = 64 the two 64-byte halves of a row are
-// swapped on odd rows (keeps the transposed reads of 8 rows x 64 B spread over all banks).
-template <int DP>
-__device__ __forceinline__ int v_swizzle(int row) {  // in 16-byte chunks
-	return (DP == 64) ? ((row & 1) << 2) : 0;
-}
 
 // 8 consecutive bias values bias[row][key .. key+7], guarded: elements at key >= L read as zero.
 template <bool BIAS_F32>
@@ -101,13 +73,6 @@ __device__ __forceinline__ u32x4 bias_frag_finite(u32x4 w) {
 		w[j] = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, x), lim));
 	}
 	return w;
-}
-
-__device__ __forceinline__ float half_swap_max(float x) {
-	// lanes l and l^32 exchange; v_permlane32_swap swaps the upper half of one operand with the
-	// lower half of the other, so (x, x) yields {low|low} and {high|high}.
-	auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-	return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
 // ---- bias prepass (log2 variant) ---------------------------------------------------------------
@@ -147,29 +112,6 @@ __global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restric
 		}
 		ws[i] = o;
 	}
-}
-
-// 16 bytes per lane from a raw buffer straight into LDS (lane i lands at lds_addr + 16*i).  Written as
-// inline assembly on purpose: the compiler makes every LDS read that follows an LDS-direct load it
-// knows about wait for vmcnt(0), which exposes the whole latency of every tile load when only one or
-// two wavefronts share a SIMD.  Loads issued here are invisible to it; the kernel orders them itself
-// (explicit s_waitcnt vmcnt before the barrier that publishes a tile).  rsrc and lds_addr must be
-// wave-uniform.  The whole byte offset travels in the vector operand, which the hardware range-checks
-// against the buffer size: a lane whose offset is past the end fetches nothing from memory.
-// M0 (the LDS base of the load) is written behind the compiler's back.  It cannot be declared: the compiler treats
-// M0 as a reserved register and answers an "m0" clobber with a warning that it is ignored.  What keeps this safe is
-// that nothing else in this file makes the compiler use M0 -- no LDS-direct builtins, no indirect register indexing,
-// no message or GWS instructions -- and gfx950's LDS instructions do not read it.
-__device__ __forceinline__ void lds_dma_b128(const u32x4& rsrc, uint32_t lds_addr, int voff) {
-	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
-}
-__device__ __forceinline__ u32x4 raw_rsrc(const void* base, uint32_t bytes) {
-	const uint64_t a = reinterpret_cast<uint64_t>(base);
-	return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a), (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xFFFFu)),
-				 (uint32_t)__builtin_amdgcn_readfirstlane((int)bytes), 0x00020000u};
-}
-__device__ __forceinline__ uint32_t lds_addr_of(const void* ptr) {
-	return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const void*)ptr);
 }
 
 // DP: head_dim padded to a multiple of 32 (32 or 64).  NW: wavefronts per workgroup.  L2DOM: log2
@@ -1052,9 +994,19 @@ static int64_t ws_bytes_needed(const af3_dpa_params& p) {
 	return p.H * n_qblocks * n_ktiles * 256 * 16;
 }
 
+// Whether the call goes to the kernel of dpa_mfma_rows.hip (four batch rows per wavefront sharing each bias tile): its
+// shape limits, enough workgroups to give every compute unit one (smaller launches do better with this file's key-split
+// variants), and the caller's hint (af3_dpa_params.reserved: 1 = take it whenever the shape allows, 2 = never).
+static bool rows_kernel_wanted(const af3_dpa_params& p) {
+	if(p.reserved == 2 || !mfma_rows_eligible(p)) return false;
+	if(p.reserved == 1) return true;
+	return ((p.B + 3) / 4) * p.H * ((p.L + 127) / 128) >= 256;
+}
+
 // The rewrite costs one extra pass over the bias; it pays off as soon as two batch rows share it.
 int64_t mfma_bf16_workspace_bytes(const af3_dpa_params& p) {
 	if(!mfma_bf16_eligible(p) || !p.bias || p.B < 2) return 0;
+	if(rows_kernel_wanted(p)) return mfma_rows_workspace_bytes(p);
 	return ws_bytes_needed(p);
 }
 
@@ -1205,6 +1157,8 @@ static int launch_nw(const af3_dpa_params& p, hipStream_t s) {
 }
 
 int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s) {
+	if(rows_kernel_wanted(p) && (!p.bias || (p.workspace && p.workspace_bytes >= mfma_rows_workspace_bytes(p) && (reinterpret_cast<uintptr_t>(p.workspace) & 15) == 0)))
+		return launch_dpa_mfma_rows(p, s);
 	const bool bf32   = p.bias && p.bias_dtype == AF3_F32;
 	const bool use_ws = p.bias && p.workspace && mfma_bf16_workspace_bytes(p) > 0 && p.workspace_bytes >= ws_bytes_needed(p) &&
 						(reinterpret_cast<uintptr_t>(p.workspace) & 15) == 0;

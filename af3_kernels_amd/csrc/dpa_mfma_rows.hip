@@ -1,0 +1,535 @@
+// bf16 matrix-core attention kernel for batched calls whose batch rows share one bias (triangle / grid attention):
+// out[b] = softmax(q[b].k[b]^T*scale + bias, mask[b]).v[b] with bias [H, L, L] common to all b.
+//
+// The reference walks (batch, head, query tile) tasks and re-reads the bias tile for every batch row
+// (src/csrc/dot_product_attention.cpp:88-110).  Here a wavefront owns one block of 32 query rows of one head for FOUR
+// batch rows at once and walks the key axis once for all four: a 32 x 32 bias tile is loaded once, as fp32 already
+// laid out like the matrix core's accumulator, and is the C operand of the first K.Q^T instruction of each of the
+// four rows -- the bias add costs no instruction at all and a quarter of the loads.  The four rows are four
+// independent dependence chains: while the vector ALU exponentiates the logits of one row, the matrix pipe computes
+// the logits of the next row and the P.V product of the previous one.
+//
+// Per 32 x 32 block of logits: 2 MFMA K.Q^T (+ bias through C), 1 MFMA key mask and softmax reference, 2 MFMA
+// V^T.P^T, 2 half-size MFMA row sums; 16 v_exp_f32 and 8 v_cvt_pk_bf16_f32 -- the arithmetic of dpa_mfma.hip's log2
+// variant (same transposed layout, same optimistic softmax reference, same mask constants) without its two bias
+// MFMAs.
+//
+// Work split.  Workgroup = NW wavefronts = NW blocks of 32 query rows of one (group of 4 batch rows, head).  K and V
+// tiles (32 keys x 4 batch rows) are staged in LDS by loads that write LDS directly, four buffers deep, and shared
+// by the NW wavefronts; one workgroup barrier per tile, i.e. per four blocks of logits of every wavefront.
+#include "mfma_helpers.hpp"
+
+namespace af3 {
+
+namespace {
+
+constexpr int ROWS   = 4;                  // batch rows per wavefront
+constexpr int KT_R   = 32;                 // keys per tile
+constexpr int NBUF_R = 3;                  // tile buffers
+constexpr int TILE_R = KT_R * 32 * 2;      // bytes of one tensor's tile of one batch row (head_dim padded to 32)
+constexpr int BUF_R  = ROWS * 2 * TILE_R;  // one buffer: [row][K tile | V tile]
+constexpr int MAX_L_ROWS = 4096;           // mask table: 8 bytes per key for the four rows
+
+// ---- bias prepass ---------------------------------------------------------------------------------------------------
+// Workspace layout: [H][query block of 32][key tile of 32][load 4][lane 64] x 16 bytes = the accumulator layout of
+// v_mfma_f32_32x32x16: lane (q = lane%32, g = lane/32), register 4*ld + e  <->  key 32*t + 8*ld + 4*g + e.
+// Values are fp32 bias * log2 e; zero outside the L x L corner; -inf, NaN and anything below -2^100 become -2^100
+// (weight exactly 0, like a dropped key).
+template <bool BIAS_F32>
+__global__ void __launch_bounds__(256) bias_rows_prepass_kernel(const void* __restrict__ bias, f32x4* __restrict__ ws, int64_t H, int64_t L, int64_t stride_h, int64_t stride_q,
+																  int n_qblocks, int n_tiles, bool vec_ok) {
+	const int64_t total = H * n_qblocks * (int64_t)n_tiles * 256;
+	for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+		const int     lane = (int)(i & 63), ld = (int)((i >> 6) & 3);
+		const int64_t t1   = i >> 8;
+		const int     t    = (int)(t1 % n_tiles);
+		const int64_t t2   = t1 / n_tiles;
+		const int     qb   = (int)(t2 % n_qblocks);
+		const int64_t h    = t2 / n_qblocks;
+		const int64_t row  = (int64_t)qb * 32 + (lane & 31);
+		const int64_t key  = (int64_t)t * KT_R + 8 * ld + 4 * (lane >> 5);
+		float         f[4] = {0.f, 0.f, 0.f, 0.f};
+		if(row < L) {
+			const int64_t off = h * stride_h + row * stride_q + key;
+			if(BIAS_F32) {
+				const float* bp = static_cast<const float*>(bias) + off;
+				if(vec_ok && key + 4 <= L) {
+					const f32x4 raw = *reinterpret_cast<const f32x4*>(bp);
+					f[0] = raw[0], f[1] = raw[1], f[2] = raw[2], f[3] = raw[3];
+				} else {
+#pragma unroll
+					for(int e = 0; e < 4; e++)
+						if(key + e < L) f[e] = bp[e];
+				}
+			} else {
+				const uint16_t* bp = static_cast<const uint16_t*>(bias) + off;
+				if(vec_ok && key + 4 <= L) {
+					const u32x2 raw = *reinterpret_cast<const u32x2*>(bp);
+					f[0] = bf16_bits_to_f32(raw[0] & 0xffffu), f[1] = bf16_bits_to_f32(raw[0] >> 16);
+					f[2] = bf16_bits_to_f32(raw[1] & 0xffffu), f[3] = bf16_bits_to_f32(raw[1] >> 16);
+				} else {
+#pragma unroll
+					for(int e = 0; e < 4; e++)
+						if(key + e < L) f[e] = bf16_bits_to_f32(bp[e]);
+				}
+			}
+		}
+		f32x4 o;
+#pragma unroll
+		for(int e = 0; e < 4; e++) o[e] = fmaxf(f[e] * LOG2E, MASK_DROPPED);  // (fmaxf returns the other operand for NaN)
+		ws[i] = o;
+	}
+}
+
+// NW: wavefronts per workgroup (= ROWS: wavefront w fetches the tiles of batch row w).  HAS_BIAS: false = no bias at all.
+template <int NW, bool HAS_BIAS>
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) dpa_rows_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups) {
+	static_assert(NW == ROWS, "wavefront w fetches the K and V tiles of batch row w");
+	constexpr int SLOT_BASE = NBUF_R * BUF_R;                       // per-wavefront bias slots (4 KB each)
+	constexpr int MASK_BASE = SLOT_BASE + (HAS_BIAS ? NW * 4096 : 0);
+	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+	// [buffer 3][batch row 4][K tile 2 KB | V tile 2 KB] [bias slot 4 KB per wavefront] [mask table: (tiles + 1) x 4 rows x 32 keys, bf16 bits]
+	const int64_t L        = p.L;
+	const int     D        = (int)p.D;
+	const int     n_t_all  = (int)((L + KT_R - 1) / KT_R);
+	uint16_t* const mask_tab = reinterpret_cast<uint16_t*>(smem + MASK_BASE);
+	__shared__ int  s_last[ROWS];  // index of the last live key + 1 of each batch row (0: every key dropped)
+
+	// ---- workgroup -> (group of batch rows, head, query tile): all query tiles of one (group, head) get ids congruent
+	// mod 8, i.e. the same XCD (they share that XCD's L2 copy of K and V), and an XCD only sees heads xcd % H (for H | 8),
+	// so its share of the bias workspace stays L2-resident across the whole batch.
+	const int64_t wg    = blockIdx.x;
+	const int     xcd   = (int)(wg & 7);
+	const int64_t slot  = wg >> 3;
+	const int64_t group = (slot / n_qtiles) * 8 + xcd;
+	const int     qtile = (int)(slot % n_qtiles);
+	if(group >= n_groups) return;
+	const int64_t g = group / p.H, h = group % p.H;
+	const int64_t b0 = g * ROWS;
+
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int n = lane & 31, half = lane >> 5;
+
+	// ---- zero the tile buffers when a load can leave parts of them unwritten (padded head columns, rows past L):
+	// stale LDS contents there must be finite ----
+	if(D != 32 || L % KT_R != 0)
+		for(int i = tid; i < NBUF_R * BUF_R / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
+
+	// ---- key-mask table: entry = additive mask value of (tile, batch row, key) as bf16 bits; wavefront w fills row w ----
+	{
+		const int      r    = wave;
+		const int64_t  br   = b0 + r < p.B ? b0 + r : p.B - 1;
+		const uint8_t* keep = p.key_mask ? p.key_mask + br * p.key_mask_stride_b : nullptr;
+		int            last = 0;
+		for(int base = 0; base < (n_t_all + 1) * KT_R; base += 64) {
+			const int  key  = base + lane;
+			const bool in   = key < L;
+			const bool live = in && (keep ? keep[key] != 0 : true);
+			if(key < (n_t_all + 1) * KT_R) mask_tab[((key >> 5) * ROWS + r) * 32 + (key & 31)] = live ? (uint16_t)0 : (in ? MASK_DROPPED_BF16 : MASK_OUT_OF_RANGE_BF16);
+			const unsigned long long bal = __ballot(live);
+			if(bal) last = base + 64 - __builtin_clzll(bal);
+		}
+		// A batch row without any live key yields the mean over all L keys (masked_fill(-1e9) + softmax in
+		// examples/dot_product_attention.py:37-39): its keys count as live, and q and the bias are dropped for it
+		// below, so that all its logits are exactly equal.
+		if(last == 0)
+			for(int key = lane; key < (n_t_all + 1) * KT_R; key += 64) mask_tab[((key >> 5) * ROWS + r) * 32 + (key & 31)] = key < L ? (uint16_t)0 : MASK_OUT_OF_RANGE_BF16;
+		if(lane == 0) s_last[r] = last;
+	}
+	__syncthreads();
+	// keys behind the last live key of every row carry weight 0 and are not walked; a row without live keys needs them all
+	int  l_eff = 0;
+	bool dropped[ROWS];
+#pragma unroll
+	for(int r = 0; r < ROWS; r++) {
+		const int last = __builtin_amdgcn_readfirstlane(s_last[r]);
+		dropped[r]     = last == 0;
+		const int need = dropped[r] ? (int)L : last;
+		l_eff          = need > l_eff ? need : l_eff;
+	}
+	const int n_t = (l_eff + KT_R - 1) / KT_R;
+
+	// ---- per-lane constants ----
+	const int64_t qrow   = (int64_t)qtile * (NW * 32) + wave * 32 + n;
+	const bool    row_ok = qrow < L;
+	// Q fragments (B operand of S^T = K.Q^T): lane (q = n, g = half) holds q[q][16c + 8g .. +7], scaled by
+	// softmax_scale * log2 e in fp32 and rounded once to bf16 (the reference rounds the scaled q too,
+	// src/csrc/dot_product_attention.cpp:95-98).  A batch row without live keys gets q = 0.
+	bf16x8 qf[ROWS][2];
+#pragma unroll
+	for(int r = 0; r < ROWS; r++) {
+		const int64_t   br   = b0 + r < p.B ? b0 + r : p.B - 1;
+		const float     qmul = dropped[r] ? 0.f : p.softmax_scale * LOG2E;
+		const uint16_t* qp   = static_cast<const uint16_t*>(p.q) + br * p.q_stride[0] + h * p.q_stride[1] + qrow * p.q_stride[2];
+#pragma unroll
+		for(int c = 0; c < 2; c++) {
+			const int d0  = 16 * c + 8 * half;
+			u32x4     raw = {0u, 0u, 0u, 0u};
+			if(row_ok && d0 < D) raw = *reinterpret_cast<const u32x4*>(qp + d0);
+			u32x4 sc4;
+#pragma unroll
+			for(int j = 0; j < 4; j++) {
+				const uint32_t w = raw[j];
+				sc4[j] = pack_bf16x2(bf16_bits_to_f32(w & 0xffffu) * qmul, bf16_bits_to_f32(w >> 16) * qmul);
+			}
+			qf[r][c] = __builtin_bit_cast(bf16x8, sc4);
+		}
+	}
+	// Operands of the mask MFMA (v_mfma_f32_32x32x8_bf16: four contraction slots per half-wave, two registers per operand).
+	// A (per key): slot 0 = the key's mask value (from the table, zero-extended), slots 2 and 3 = 1.0.
+	// B (per query): slot 0 = 1.0, slots 2 and 3 = -m_hi and -m_lo, the softmax reference of this lane's query row as two
+	// bf16 terms (16 significant bits).  Lanes of the upper half-wave supply slots 4..7: their B is zero, so whatever
+	// finite value their A holds contributes nothing.
+	u32x2 maskA = {0u, 0x3F803F80u};
+	u32x2 maskB[ROWS];
+#pragma unroll
+	for(int r = 0; r < ROWS; r++) maskB[r] = u32x2{half == 0 ? 0x3F80u : 0u, 0u};
+
+	// ---- tile and bias loaders: loads that write LDS directly (no registers, invisible to the compiler's wait counting;
+	// every wait for them below is explicit).  This wavefront fetches K and V of batch row `wave`: four 1 KB pieces per
+	// tile (K rows 0-15, 16-31, V rows 0-15, 16-31; lane i -> tile row i/4, 16-byte chunk i%4, K chunks swizzled), and
+	// the four 1 KB pieces of its own bias fragment.  Lanes of padded head columns carry an offset beyond the buffer's
+	// range: the hardware fetches nothing for them. ----
+	const int64_t b_ld   = b0 + wave < p.B ? b0 + wave : p.B - 1;
+	const u32x4   k_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.k) + b_ld * p.k_stride[0] + h * p.k_stride[1], (uint32_t)(((L - 1) * p.k_stride[2] + D) * 2));
+	const u32x4   v_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.v) + b_ld * p.v_stride[0] + h * p.v_stride[1], (uint32_t)(((L - 1) * p.v_stride[2] + D) * 2));
+	const int     ld_row = lane >> 2, ld_pc = lane & 3;
+	const int     k_chunk = ld_pc ^ k_swizzle<32>(ld_row);
+	const int     k_voff  = k_chunk * 8 < D ? (int)(ld_row * p.k_stride[2] * 2) + k_chunk * 16 : 0x40000000;
+	const int     v_voff  = ld_pc * 8 < D ? (int)(ld_row * p.v_stride[2] * 2) + ld_pc * 16 : 0x40000000;
+	const int     k_tile_stride = (int)(KT_R * p.k_stride[2] * 2), v_tile_stride = (int)(KT_R * p.v_stride[2] * 2);
+	const int     k_pc_stride = (int)(16 * p.k_stride[2] * 2), v_pc_stride = (int)(16 * p.v_stride[2] * 2);
+	const uint32_t lds_tiles = lds_addr_of(smem) + wave * (2 * TILE_R);
+	auto load_tile = [&](int t, int buf_off) {
+		lds_dma_b128(k_rsrc, lds_tiles + buf_off, k_voff + t * k_tile_stride);
+		lds_dma_b128(k_rsrc, lds_tiles + buf_off + 1024, k_voff + (t * k_tile_stride + k_pc_stride));
+		lds_dma_b128(v_rsrc, lds_tiles + buf_off + TILE_R, v_voff + t * v_tile_stride);
+		lds_dma_b128(v_rsrc, lds_tiles + buf_off + TILE_R + 1024, v_voff + (t * v_tile_stride + v_pc_stride));
+	};
+	// bias fragment of key tile t: 4 KB of this (head, query block)'s slab of the workspace -> this wavefront's slot
+	const int     n_qblocks = (int)((L + 31) / 32);
+	const int64_t qb        = (int64_t)qtile * NW + wave;
+	const int64_t qbc       = qb < n_qblocks ? qb : n_qblocks - 1;  // (blocks past the end only hold rows >= L)
+	const u32x4   ws_rsrc   = raw_rsrc(HAS_BIAS ? static_cast<const unsigned char*>(p.workspace) + ((h * n_qblocks + qbc) * n_t_all) * 4096 : nullptr, HAS_BIAS ? (uint32_t)(n_t_all * 4096) : 0u);
+	const int      ws_voff  = lane * 16;
+	const uint32_t lds_slot = lds_addr_of(smem) + SLOT_BASE + wave * 4096;
+	auto load_bias = [&](int t) {
+		if(!HAS_BIAS) return;
+#pragma unroll
+		for(int ld = 0; ld < 4; ld++) lds_dma_b128(ws_rsrc, lds_slot + ld * 1024, ws_voff + (t * 4096 + ld * 1024));  // (past the last tile: nothing is fetched)
+	};
+	constexpr int LOADS_PER_TILE = 4 + (HAS_BIAS ? 4 : 0);
+
+	// ---- per-lane LDS read offsets inside a (buffer, batch row) block ----
+	int k_rd[2];
+#pragma unroll
+	for(int c = 0; c < 2; c++) k_rd[c] = n * 64 + (((2 * c + half) ^ k_swizzle<32>(n)) << 4);
+	// V^T fragment reads (ds_read_b64_tr_b16): lane l: i = l%16, G = l/16 supplies the 8-byte chunk at tile row
+	// base + 4*(G/2) + i/4, column 16*(G%2) + 4*(i%4); it receives 4 keys of column l%32.
+	int v_rd;
+	{
+		const int i16 = lane & 15, G = lane >> 4;
+		const int row = 4 * (G >> 1) + (i16 >> 2), col = 16 * (G & 1) + 4 * (i16 & 3);
+		v_rd = TILE_R + row * 64 + (col >> 3) * 16 + (col & 7) * 2;
+	}
+	const int mask_rd = MASK_BASE + n * 2;               // + ((tile * ROWS + row) * 32) * 2
+	const int slot_rd = SLOT_BASE + wave * 4096 + lane * 16;  // + 1024 per group of four accumulator registers
+
+	// ---- online-softmax state: one query row per lane and batch row (the two half-waves hold disjoint keys) ----
+	float  m_ref[ROWS];   // reference maximum, log2 units, exactly m_hi + m_lo of two bf16 values
+	float  lsum[ROWS];    // the row sum (complete: the same value in both half-waves)
+	f32x16 oacc[ROWS];
+#pragma unroll
+	for(int r = 0; r < ROWS; r++) {
+		m_ref[r] = 0.f;
+		lsum[r]  = 0.f;
+#pragma unroll
+		for(int i = 0; i < 16; i++) oacc[r][i] = 0.f;
+	}
+
+	// Row sums on the matrix pipe (see dpa_mfma.hip): a 16x16x32 MFMA whose A operand is this 0/1 pattern leaves, in
+	// register 0 of every lane, the sum of the 16 packed probabilities of that lane's own query row over both half-waves.
+	u32x4 ones_a;
+	{
+		const int      i16 = lane & 15, kg = lane >> 4;
+		const bool     on  = ((i16 == 0 || i16 == 8) && (kg & 1) == 0) || ((i16 == 4 || i16 == 12) && (kg & 1) == 1);
+		const uint32_t w   = on ? 0x3F803F80u : 0u;
+		ones_a = u32x4{w, w, w, w};
+	}
+
+	// Move the reference of batch row R for every query whose maximum is not within REF_SLACK of it (all queries when
+	// `force`), rescale what has been accumulated and re-express s relative to the new reference.
+	auto rereference = [&](auto r_c, f32x16& s, bool force) {
+		constexpr int R = decltype(r_c)::value;
+		float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+		for(int i = 3; i < 15; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
+		mx = half_swap_max(fmaxf(mx, s[15]));
+		// s already has m_ref subtracted (by the mask MFMA)
+		const bool  need   = force || mx > REF_SLACK;
+		const float m_want = m_ref[R] + mx;
+		const float m_hi   = bf16_bits_to_f32(f32_to_bf16_bits(need ? m_want : m_ref[R]));
+		const float m_lo   = bf16_bits_to_f32(f32_to_bf16_bits((need ? m_want : m_ref[R]) - m_hi));
+		const float m_new  = m_hi + m_lo;  // exactly what the mask MFMA will subtract (unchanged when !need)
+		const float delta  = m_new - m_ref[R];
+		const float alpha  = force ? 1.f : __builtin_amdgcn_exp2f(-delta);  // nothing is accumulated yet when forced
+#pragma unroll
+		for(int i = 0; i < 16; i++) s[i] -= delta;
+		m_ref[R] = m_new;
+		if(half == 0) maskB[R][1] = f32_to_bf16_bits(-m_hi) | (f32_to_bf16_bits(-m_lo) << 16);
+		lsum[R] *= alpha;
+#pragma unroll
+		for(int i = 0; i < 16; i++) oacc[R][i] *= alpha;
+	};
+	auto exp_part = [&](const f32x16& s, u32x4 (&pf)[2], auto i0_c, auto n_c) {
+		constexpr int I0 = decltype(i0_c)::value, N = decltype(n_c)::value;
+#pragma unroll
+		for(int i = I0; i < I0 + N; i += 2) pf[i >> 3][(i & 7) >> 1] = pack_bf16x2(__builtin_amdgcn_exp2f(s[i]), __builtin_amdgcn_exp2f(s[i + 1]));
+	};
+	auto read_kfrag = [&](int addr) -> u32x4 { return *reinterpret_cast<const u32x4*>(smem + addr); };
+	auto rowsum     = [&](const f32x4& c, const u32x4& pf) -> f32x4 { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ones_a), __builtin_bit_cast(bf16x8, pf), c, 0, 0, 0); };
+	auto mask_mfma  = [&](const f32x16& c, const u32x2& b) -> f32x16 {
+		return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(s16x4, maskA), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+	};
+
+	// Pipeline registers: S^T of the current step, P^T and V^T fragments of the previous one, K fragments of the next
+	// one, and the bias fragment of the tile the next step belongs to (accumulator order: the C operand of that step's
+	// first K.Q^T instruction).
+	f32x16 sc, bias_frag;
+	u32x4  kf[2];
+	u32x4  pprev[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
+	u32x4  vprev[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
+#pragma unroll
+	for(int i = 0; i < 16; i++) bias_frag[i] = 0.f;
+	auto read_bias_slot = [&] {
+		if(!HAS_BIAS) return;
+#pragma unroll
+		for(int ld = 0; ld < 4; ld++) {
+			const f32x4 v = *reinterpret_cast<const f32x4*>(smem + slot_rd + ld * 1024);
+			bias_frag[4 * ld] = v[0], bias_frag[4 * ld + 1] = v[1], bias_frag[4 * ld + 2] = v[2], bias_frag[4 * ld + 3] = v[3];
+		}
+	};
+
+	// One step = one 32 x 32 block of logits of batch row R.  On entry `sc` holds its finished S^T, `pprev` / `vprev`
+	// belong to the previous step (batch row R-1, or row 3 of the previous tile) and `kf` holds the K fragments of the
+	// next step.  The step alternates matrix instructions of three independent chains with slices of its vector work
+	//     matrix pipe                                            vector ALU
+	//     O^T[R-1] += V^T . P^T (previous step, 2 instructions)   exp2 / pack of this step, two logits per slice
+	//     S^T of the next step (K.Q^T + bias, mask: 3)
+	//     row sum of this step (2 half-size instructions)
+	// so that no instruction waits for the one issued just before it, and leaves S^T(next) in `sc`, P^T in `pprev`, this
+	// step's V^T fragments in `vprev`, the K fragments of the step after the next in `kf`.
+	// k_addr2: LDS byte address of the K tile of the step after the next; m_addr: (per lane) of the next step's mask
+	// entries; v_addr: of this step's V tile; mid: hook run once the first K.Q^T instruction of the next step is issued.
+	// FIRST: the very first tile, which fixes every row's softmax reference.  ANYDROP: some batch row of this group has no
+	// live key (it then takes no bias: a wave-uniform branch the common instantiation does not carry).
+	auto step = [&](auto r_c, auto first_c, auto anydrop_c, int k_addr2, int m_addr, int v_addr, auto&& mid) {
+		constexpr int  R = decltype(r_c)::value, RN = (R + 1) % ROWS, RP = (R + ROWS - 1) % ROWS;
+		constexpr bool FIRST = decltype(first_c)::value != 0, ANYDROP = decltype(anydrop_c)::value != 0;
+		if constexpr(FIRST) rereference(r_c, sc, true);
+		maskA[0] = *reinterpret_cast<const uint16_t*>(smem + m_addr);
+		u32x4  pcur[2];
+		f32x16 sn;
+		f32x4  rs = {0.f, 0.f, 0.f, 0.f};
+#define AF3_CHUNK_END() __builtin_amdgcn_sched_barrier(0)
+		AF3_CHUNK_END();
+		oacc[RP] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[0]), __builtin_bit_cast(bf16x8, pprev[0]), oacc[RP], 0, 0, 0);
+		exp_part(sc, pcur, ic<0>{}, ic<2>{});
+		AF3_CHUNK_END();
+		{
+			f32x16 z;
+#pragma unroll
+			for(int i = 0; i < 16; i++) z[i] = 0.f;
+			bool with_bias = HAS_BIAS;
+			if constexpr(ANYDROP) with_bias = HAS_BIAS && !dropped[RN];  // (wave-uniform)
+			if(with_bias) sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[0]), qf[RN][0], bias_frag, 0, 0, 0);
+			else sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[0]), qf[RN][0], z, 0, 0, 0);
+		}
+		mid();
+		exp_part(sc, pcur, ic<2>{}, ic<2>{});
+		AF3_CHUNK_END();
+		oacc[RP] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[1]), __builtin_bit_cast(bf16x8, pprev[1]), oacc[RP], 0, 0, 0);
+		// V^T fragments of this step for the next step's P.V, now that the previous ones are consumed
+#pragma unroll
+		for(int cp = 0; cp < 2; cp++)
+#pragma unroll
+			for(int t = 0; t < 2; t++) {
+				const s16x4 rr = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(smem + v_addr + v_rd + (16 * cp + 8 * t) * 64));
+				const u32x2 r2 = __builtin_bit_cast(u32x2, rr);
+				vprev[cp][2 * t] = r2[0], vprev[cp][2 * t + 1] = r2[1];
+			}
+		exp_part(sc, pcur, ic<4>{}, ic<2>{});
+		AF3_CHUNK_END();
+		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[1]), qf[RN][1], sn, 0, 0, 0);
+		// K fragments of the step after the next, now that the next step's are consumed
+		kf[0] = read_kfrag(k_addr2 + k_rd[0]);
+		kf[1] = read_kfrag(k_addr2 + k_rd[1]);
+		exp_part(sc, pcur, ic<6>{}, ic<2>{});
+		AF3_CHUNK_END();
+		rs = rowsum(rs, pcur[0]);
+		exp_part(sc, pcur, ic<8>{}, ic<4>{});
+		AF3_CHUNK_END();
+		sn = mask_mfma(sn, maskB[RN]);
+		exp_part(sc, pcur, ic<12>{}, ic<4>{});
+		AF3_CHUNK_END();
+#undef AF3_CHUNK_END
+		rs = rowsum(rs, pcur[1]);
+		// This step's sum stays below 32 * 2^REF_SLACK while every probability respects the reference, so the test also
+		// catches a single probability near or beyond the limit (inf, NaN).
+		if(__ballot(!(rs[0] < PSUM_LIMIT))) {  // rare
+			rereference(r_c, sc, false);
+			exp_part(sc, pcur, ic<0>{}, ic<16>{});
+			rs = rowsum(f32x4{0.f, 0.f, 0.f, 0.f}, pcur[0]);
+			rs = rowsum(rs, pcur[1]);
+		}
+		lsum[R] += rs[0];
+		sc       = sn;
+		pprev[0] = pcur[0];
+		pprev[1] = pcur[1];
+	};
+
+	// One tile: four steps.  Tile t sits in buffer t % 3.  In front of the third step the loads issued one tile earlier
+	// (tile t + 1 and its bias fragment: the youngest loads this wavefront has in flight) are awaited and a barrier
+	// publishes tile t + 1 -- the third step fetches K fragments from it -- and tells that every wavefront is done with
+	// tile t - 1, whose buffer tile t + 2 then overwrites.  The third step's first matrix instruction is the last reader
+	// of bias fragment t: behind it the fragment registers are refilled from the slot, and the slot, once those reads
+	// have returned (the last step's first matrix instruction waits for them), with fragment t + 2.
+	auto tile = [&](auto first_c, auto anydrop_c, int t, int buf, int bufn, int bufnn) {
+		const int m0 = mask_rd + t * (ROWS * 64);
+		auto none = [] {};
+		step(ic<0>{}, first_c, anydrop_c, buf + 2 * (2 * TILE_R), m0 + 1 * 64, buf + 0 * (2 * TILE_R), none);
+		step(ic<1>{}, first_c, anydrop_c, buf + 3 * (2 * TILE_R), m0 + 2 * 64, buf + 1 * (2 * TILE_R), none);
+		asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+		step(ic<2>{}, first_c, anydrop_c, bufn + 0 * (2 * TILE_R), m0 + 3 * 64, buf + 2 * (2 * TILE_R), [&] {
+			load_tile(t + 2, bufnn);  // (past the end of the rows: nothing is fetched)
+			read_bias_slot();
+		});
+		step(ic<3>{}, first_c, anydrop_c, bufn + 1 * (2 * TILE_R), m0 + ROWS * 64, buf + 3 * (2 * TILE_R), [&] { load_bias(t + 2); });
+	};
+	auto run = [&](auto anydrop_c) {
+		constexpr bool ANYDROP = decltype(anydrop_c)::value != 0;
+		// ---- prologue: the first two tiles, the first two bias fragments, S^T of the first step, K fragments of the second ----
+		load_tile(0, 0);
+		load_bias(0);
+		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+		read_bias_slot();  // fragment 0 -> registers
+		asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+		load_tile(1, BUF_R);
+		load_bias(1);
+		__syncthreads();   // tile 0 is complete (every wavefront has waited for its own pieces)
+		{
+			f32x16 s0;
+#pragma unroll
+			for(int i = 0; i < 16; i++) s0[i] = (HAS_BIAS && !(ANYDROP && dropped[0])) ? bias_frag[i] : 0.f;
+#pragma unroll
+			for(int c = 0; c < 2; c++) s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, read_kfrag(k_rd[c])), qf[0][c], s0, 0, 0, 0);
+			maskA[0] = *reinterpret_cast<const uint16_t*>(smem + mask_rd);
+			sc = mask_mfma(s0, maskB[0]);
+			kf[0] = read_kfrag(2 * TILE_R + k_rd[0]);
+			kf[1] = read_kfrag(2 * TILE_R + k_rd[1]);
+		}
+		tile(ic<1>{}, anydrop_c, 0, 0, BUF_R, 2 * BUF_R);
+		int buf = BUF_R;
+		for(int t = 1; t < n_t; t++) {
+			const int bufn = buf == (NBUF_R - 1) * BUF_R ? 0 : buf + BUF_R, bufnn = bufn == (NBUF_R - 1) * BUF_R ? 0 : bufn + BUF_R;
+			tile(ic<0>{}, anydrop_c, t, buf, bufn, bufnn);
+			buf = bufn;
+		}
+	};
+	if(n_t > 0) {
+		bool any_dropped = false;
+#pragma unroll
+		for(int r = 0; r < ROWS; r++) any_dropped = any_dropped || dropped[r];
+		if(any_dropped) run(ic<1>{});
+		else run(ic<0>{});
+	}
+	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may still be writing LDS when the workgroup's allocation is released
+	// the last step's P.V product (batch row 3)
+	oacc[ROWS - 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[0]), __builtin_bit_cast(bf16x8, pprev[0]), oacc[ROWS - 1], 0, 0, 0);
+	oacc[ROWS - 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[1]), __builtin_bit_cast(bf16x8, pprev[1]), oacc[ROWS - 1], 0, 0, 0);
+
+	// ---- epilogue: O^T register i is head column 8*(i/4) + 4*half + i%4 ----
+	if(row_ok) {
+#pragma unroll
+		for(int r = 0; r < ROWS; r++) {
+			if(b0 + r >= p.B) break;
+			const float   inv  = 1.f / lsum[r];
+			const int64_t ooff = (b0 + r) * p.out_stride[0] + h * p.out_stride[1] + qrow * p.out_stride[2];
+#pragma unroll
+			for(int g4 = 0; g4 < 4; g4++) {
+				const int d0 = 8 * g4 + 4 * half;
+				if(d0 >= D) continue;
+				const float o0 = oacc[r][4 * g4] * inv, o1 = oacc[r][4 * g4 + 1] * inv, o2 = oacc[r][4 * g4 + 2] * inv, o3 = oacc[r][4 * g4 + 3] * inv;
+				if(p.out_dtype == AF3_BF16) {
+					const u32x2 w = {pack_bf16x2(o0, o1), pack_bf16x2(o2, o3)};
+					*reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.out) + ooff + d0) = w;
+				} else {
+					const float4 w = {o0, o1, o2, o3};
+					*reinterpret_cast<float4*>(static_cast<float*>(p.out) + ooff + d0) = w;
+				}
+			}
+		}
+	}
+}
+
+size_t rows_lds_bytes(const af3_dpa_params& p) {
+	const size_t n_t_all = (size_t)((p.L + KT_R - 1) / KT_R);
+	return (size_t)NBUF_R * BUF_R + (p.bias ? ROWS * 4096 : 0) + (n_t_all + 1) * ROWS * 32 * 2;
+}
+
+int64_t rows_ws_bytes(const af3_dpa_params& p) {
+	const int64_t n_qblocks = (p.L + 31) / 32, n_t_all = (p.L + KT_R - 1) / KT_R;
+	return p.H * n_qblocks * n_t_all * 4096;
+}
+
+template <int NW, bool HAS_BIAS>
+int launch_rows(const af3_dpa_params& p, hipStream_t s) {
+	const int     n_qtiles = (int)((p.L + NW * 32 - 1) / (NW * 32));
+	const int64_t n_groups = ((p.B + ROWS - 1) / ROWS) * p.H;
+	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
+	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
+	const size_t smem = rows_lds_bytes(p);
+	auto         kern = dpa_rows_bf16_kernel<NW, HAS_BIAS>;
+	if(smem > 64 * 1024) {
+		if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
+	}
+	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, n_qtiles, n_groups);
+	return launch_status();
+}
+
+}  // namespace
+
+// Shapes the kernel takes: what dpa_mfma.hip's kernel takes (mfma_bf16_eligible, checked by the caller), and in addition
+// head_dim <= 32, at least four batch rows, no output gate, and a length whose mask table fits beside the tile buffers.
+bool mfma_rows_eligible(const af3_dpa_params& p) {
+	if(p.D > 32 || p.B < ROWS || p.gate || p.L > MAX_L_ROWS) return false;
+	// buffer addressing of the bias workspace of one (head, query block) uses 32-bit byte offsets
+	if(((p.L + KT_R - 1) / KT_R) * 4096 >= 0x7fffffffLL) return false;
+	return true;
+}
+
+int64_t mfma_rows_workspace_bytes(const af3_dpa_params& p) { return p.bias ? rows_ws_bytes(p) : 0; }
+
+int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
+	if(p.bias) {
+		const bool     bf32      = p.bias_dtype == AF3_F32;
+		const int      n_qblocks = (int)((p.L + 31) / 32), n_t_all = (int)((p.L + KT_R - 1) / KT_R);
+		const int64_t  total     = p.H * n_qblocks * (int64_t)n_t_all * 256;
+		const unsigned g         = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
+		const int64_t  esz       = bf32 ? 4 : 2;
+		const bool     vec_ok    = ((reinterpret_cast<uintptr_t>(p.bias) & (4 * esz - 1)) == 0) && (p.bias_stride[0] % 4 == 0) && (p.bias_stride[1] % 4 == 0);
+		if(bf32)
+			hipLaunchKernelGGL(bias_rows_prepass_kernel<true>, dim3(g), dim3(256), 0, s, p.bias, static_cast<f32x4*>(p.workspace), p.H, p.L, p.bias_stride[0], p.bias_stride[1],
+							   n_qblocks, n_t_all, vec_ok);
+		else
+			hipLaunchKernelGGL(bias_rows_prepass_kernel<false>, dim3(g), dim3(256), 0, s, p.bias, static_cast<f32x4*>(p.workspace), p.H, p.L, p.bias_stride[0], p.bias_stride[1],
+							   n_qblocks, n_t_all, vec_ok);
+		const int rc = launch_status();
+		if(rc != AF3_OK) return rc;
+		return launch_rows<4, true>(p, s);
+	}
+	return launch_rows<4, false>(p, s);
+}
+
+}  // namespace af3

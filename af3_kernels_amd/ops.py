@@ -135,6 +135,7 @@ def _fill_params(q, k, v, keep, bias, out, mma_dtype, force_generic, descales=No
     p.softmax_scale = float(D) ** -0.5 if softmax_scale is None else softmax_scale
     p.q_descale = p.k_descale = p.v_descale = 1.0
     p.force_generic = int(bool(force_generic))
+    p.reserved = _rows_kernel_hint
     if descales is not None:
         p.device_descales = descales.data_ptr()
     if gate is not None:
@@ -159,6 +160,17 @@ def _check_shapes(q, k, v, keep, bias, v_transposed=False):
 
 
 _exact_bias = False
+_rows_kernel_hint = 0
+
+
+def set_rows_kernel(mode: str) -> str:
+    """Kernel choice for batched bf16 calls whose shape suits the four-batch-rows-per-wavefront kernel (head_dim <= 32,
+    at least four batch rows): "auto" (default: taken when the launch is large enough to fill the GPU), "always" or
+    "never" (testing aids).  Returns the previous mode."""
+    global _rows_kernel_hint
+    names = ("auto", "always", "never")
+    prev, _rows_kernel_hint = names[_rows_kernel_hint], names.index(mode)
+    return prev
 
 
 def set_exact_bias(flag: bool) -> bool:

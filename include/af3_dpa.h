@@ -97,7 +97,8 @@ typedef struct af3_dpa_params {
 	float          k_descale;
 	float          v_descale;
 	int32_t        force_generic; /* non-zero: always take the fp32-FMA kernel (testing aid) */
-	int32_t        reserved;
+	int32_t        reserved;      /* kernel hint for batched bf16 calls that suit the four-batch-rows-per-wavefront kernel
+	                                 (head_dim <= 32, B >= 4): 0 = chosen by launch size, 1 = always, 2 = never (testing aids) */
 	/* Optional: 3 device floats {q_descale, k_descale, v_descale} as written by
 	 * af3_quantize_fp8_e4m3; when non-NULL they override the three host values above, so a
 	 * quantise -> attend sequence needs no device-to-host copy. */

@@ -572,7 +572,9 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 			float alpha;
 			if(L2DOM) {
 				// s already has m_ref subtracted (by the mask MFMA)
-				const bool  need  = force || mx > REF_SLACK;
+				// (a first sub-tile whose keys are all dropped says nothing about the row: the reference stays at 0, its
+				// probabilities are exactly 0, and the first live logits keep their own bits)
+				const bool  need  = (force && (all_dropped || mx > -0x1p99f)) || mx > REF_SLACK;  // (a row without any live key keeps the mask constant as its reference)
 				const float m_want = m_ref + mx;
 				const float m_hi   = bf16_bits_to_f32(f32_to_bf16_bits(need ? m_want : m_ref));
 				const float m_lo   = bf16_bits_to_f32(f32_to_bf16_bits((need ? m_want : m_ref) - m_hi));

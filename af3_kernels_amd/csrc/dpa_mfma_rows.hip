@@ -29,12 +29,15 @@ constexpr int NBUF_R = 3;                  // tile buffers
 constexpr int TILE_R = KT_R * 32 * 2;      // bytes of one tensor's tile of one batch row (head_dim padded to 32)
 constexpr int BUF_R  = ROWS * 2 * TILE_R;  // one buffer: [row][K tile | V tile]
 constexpr int MAX_L_ROWS = 4096;           // mask table: 8 bytes per key for the four rows
+constexpr float BIAS_FLOOR = -0x1p17f;     // lowest value the rewritten bias holds (log2 units)
 
 // ---- bias prepass ---------------------------------------------------------------------------------------------------
 // Workspace layout: [H][query block of 32][key tile of 32][load 4][lane 64] x 16 bytes = the accumulator layout of
 // v_mfma_f32_32x32x16: lane (q = lane%32, g = lane/32), register 4*ld + e  <->  key 32*t + 8*ld + 4*g + e.
-// Values are fp32 bias * log2 e; zero outside the L x L corner; -inf, NaN and anything below -2^100 become -2^100
-// (weight exactly 0, like a dropped key).
+// Values are fp32 bias * log2 e; zero outside the L x L corner; -inf, NaN and anything below -2^17 become -2^17: such an
+// entry still gets weight exactly 0 beside any ordinary logit, a row made of nothing else still comes out uniform, and a
+// softmax reference that starts there (a row whose first keys are all masked through the bias) leaves the logits that
+// follow their fp32 precision to within 2^-6.
 template <bool BIAS_F32>
 __global__ void __launch_bounds__(256) bias_rows_prepass_kernel(const void* __restrict__ bias, f32x4* __restrict__ ws, int64_t H, int64_t L, int64_t stride_h, int64_t stride_q,
 																  int n_qblocks, int n_tiles, bool vec_ok) {
@@ -76,7 +79,7 @@ __global__ void __launch_bounds__(256) bias_rows_prepass_kernel(const void* __re
 		}
 		f32x4 o;
 #pragma unroll
-		for(int e = 0; e < 4; e++) o[e] = fmaxf(f[e] * LOG2E, MASK_DROPPED);  // (fmaxf returns the other operand for NaN)
+		for(int e = 0; e < 4; e++) o[e] = fmaxf(f[e] * LOG2E, BIAS_FLOOR);  // (fmaxf returns the other operand for NaN)
 		ws[i] = o;
 	}
 }
@@ -267,7 +270,10 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 		for(int i = 3; i < 15; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
 		mx = half_swap_max(fmaxf(mx, s[15]));
 		// s already has m_ref subtracted (by the mask MFMA)
-		const bool  need   = force || mx > REF_SLACK;
+		// (a first tile whose keys are all dropped says nothing about the row: the reference stays where it is, the tile's
+		// probabilities are exactly 0, and the first live logits are measured against a reference they can be subtracted
+		// from without losing their own bits)
+		const bool  need   = (force && mx > -0x1p99f) || mx > REF_SLACK;
 		const float m_want = m_ref[R] + mx;
 		const float m_hi   = bf16_bits_to_f32(f32_to_bf16_bits(need ? m_want : m_ref[R]));
 		const float m_lo   = bf16_bits_to_f32(f32_to_bf16_bits((need ? m_want : m_ref[R]) - m_hi));
@@ -332,11 +338,32 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 		u32x4  pcur[2];
 		f32x16 sn;
 		f32x4  rs = {0.f, 0.f, 0.f, 0.f};
-#define AF3_CHUNK_END() __builtin_amdgcn_sched_barrier(0)
-		AF3_CHUNK_END();
+		// The order below is the order the instructions are meant to issue in: one matrix instruction, then a slice of the
+		// vector work, so that consecutive matrix instructions belong to different chains.  Matrix intrinsics are pure
+		// values to the compiler and would drift to wherever their consumers are; each slice therefore ends with an empty
+		// asm statement that names what the slice produced and the operand the next slice's matrix instruction waits for
+		// (asm statements keep their order, and so does everything that feeds or reads them), followed by a scheduling barrier.
+#define AF3_PIN2(a, b)                                \
+	{                                                 \
+		auto pa_ = a;                                 \
+		auto pb_ = b;                                 \
+		asm volatile("" : "+v"(pa_), "+v"(pb_));      \
+		a = pa_, b = pb_;                             \
+	}                                                 \
+	__builtin_amdgcn_sched_barrier(0)
+#define AF3_PIN3(a, b, c)                                        \
+	{                                                            \
+		auto pa_ = a;                                            \
+		auto pb_ = b;                                            \
+		auto pc_ = c;                                            \
+		asm volatile("" : "+v"(pa_), "+v"(pb_), "+v"(pc_));      \
+		a = pa_, b = pb_, c = pc_;                               \
+	}                                                            \
+	__builtin_amdgcn_sched_barrier(0)
+		__builtin_amdgcn_sched_barrier(0);
 		oacc[RP] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[0]), __builtin_bit_cast(bf16x8, pprev[0]), oacc[RP], 0, 0, 0);
 		exp_part(sc, pcur, ic<0>{}, ic<2>{});
-		AF3_CHUNK_END();
+		AF3_PIN3(oacc[RP][0], pcur[0][0], kf[0][0]);
 		{
 			f32x16 z;
 #pragma unroll
@@ -348,7 +375,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 		}
 		mid();
 		exp_part(sc, pcur, ic<2>{}, ic<2>{});
-		AF3_CHUNK_END();
+		AF3_PIN3(sn[0], pcur[0][1], pprev[1][0]);
 		oacc[RP] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[1]), __builtin_bit_cast(bf16x8, pprev[1]), oacc[RP], 0, 0, 0);
 		// V^T fragments of this step for the next step's P.V, now that the previous ones are consumed
 #pragma unroll
@@ -360,20 +387,26 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 				vprev[cp][2 * t] = r2[0], vprev[cp][2 * t + 1] = r2[1];
 			}
 		exp_part(sc, pcur, ic<4>{}, ic<2>{});
-		AF3_CHUNK_END();
+		AF3_PIN3(oacc[RP][0], pcur[0][2], kf[1][0]);
 		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[1]), qf[RN][1], sn, 0, 0, 0);
 		// K fragments of the step after the next, now that the next step's are consumed
 		kf[0] = read_kfrag(k_addr2 + k_rd[0]);
 		kf[1] = read_kfrag(k_addr2 + k_rd[1]);
 		exp_part(sc, pcur, ic<6>{}, ic<2>{});
-		AF3_CHUNK_END();
+		AF3_PIN2(sn[0], pcur[0][3]);
 		rs = rowsum(rs, pcur[0]);
 		exp_part(sc, pcur, ic<8>{}, ic<4>{});
-		AF3_CHUNK_END();
+		AF3_PIN3(rs[0], pcur[1][0], pcur[1][1]);
+		{
+			uint32_t ma_ = maskA[0];
+			asm volatile("" : "+v"(ma_));
+			maskA[0] = ma_;
+		}
 		sn = mask_mfma(sn, maskB[RN]);
 		exp_part(sc, pcur, ic<12>{}, ic<4>{});
-		AF3_CHUNK_END();
-#undef AF3_CHUNK_END
+		AF3_PIN3(sn[0], pcur[1][2], pcur[1][3]);
+#undef AF3_PIN2
+#undef AF3_PIN3
 		rs = rowsum(rs, pcur[1]);
 		// This step's sum stays below 32 * 2^REF_SLACK while every probability respects the reference, so the test also
 		// catches a single probability near or beyond the limit (inf, NaN).

@@ -443,6 +443,100 @@ def test_named_configs_full_size(af3, oracle, name, sample_rows):
     assert (out.float() <= vmax + 1e-2).all() and (out.float() >= vmin - 1e-2).all()
 
 
+# ---- the kernel for batches that share a bias (four batch rows per wavefront) -----------------------------------------
+# Large launches take it by themselves (the named configs above do); here it is forced on small and awkward shapes.
+
+@pytest.fixture
+def rows_kernel(af3):
+    prev = af3.set_rows_kernel("always")
+    yield af3
+    af3.set_rows_kernel(prev)
+
+
+@pytest.mark.parametrize("B,H,L,D,mask,rank", [
+    (4, 4, 128, 32, "none", 2), (5, 2, 200, 32, "random", 2), (8, 4, 384, 32, "tail", 2), (7, 3, 37, 24, "random", 2),
+    (4, 1, 65, 16, "tail", 1), (9, 4, 1000, 32, "random", 2), (4, 2, 96, 8, "none", 1), (6, 16, 256, 24, "tail", 1),
+    (13, 1, 1, 32, "none", 2), (4, 5, 33, 32, "random", 2), (12, 4, 1491, 32, "random", 2),
+])
+def test_shared_bias_kernel_matches_formula(rows_kernel, oracle, B, H, L, D, mask, rank):
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=5 * L + D + B, mask=mask, mask_rank=rank)
+    run_case(rows_kernel, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+
+
+def test_shared_bias_kernel_agrees_with_the_one_row_kernel(af3):
+    """Same arithmetic in both kernels (bf16 products, fp32 accumulation, bf16 probabilities); they differ in the rounding of
+    the bias (fp32 here, fp16 in the one-row kernel's workspace) and in summation order."""
+    q, k, v, m, bias = dev(*rand_inputs(8, 4, 300, 32, torch.bfloat16, seed=31, mask="random"))
+    af3.set_rows_kernel("always")
+    a = af3.dot_product_attention_cpp(q, k, v, m, bias).float()
+    af3.set_rows_kernel("never")
+    b = af3.dot_product_attention_cpp(q, k, v, m, bias).float()
+    af3.set_rows_kernel("auto")
+    assert (a - b).abs().max().item() <= 1.6e-2 and (a - b).abs().mean().item() <= 1e-3
+
+
+def test_shared_bias_kernel_edge_cases(rows_kernel, oracle):
+    af3 = rows_kernel
+    B, H, L, D = 9, 2, 150, 32
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=41, mask="random")
+    m[1, :] = False                       # a batch row without live keys: mean of V, whatever the bias says
+    m[2, :] = False
+    m[2, 77] = True                       # a single live key: that V row
+    m[5, :64] = False                     # the first tiles of a row are dead: its reference starts at the mask constant
+    m[6, 100:] = False                    # keys behind the last live key of every row of a group are not walked
+    m[7, 100:] = False
+    m[4, 100:] = False
+    out = af3.dot_product_attention_cpp(*dev(q, k, v, m, bias)).float().cpu()
+    assert torch.isfinite(out).all()
+    want = torch.from_numpy(oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), f32np(bias)))
+    assert (out - want).abs().max().item() <= 2e-2
+    mean = v[1].float().mean(dim=1, keepdim=True).expand(H, L, D)
+    assert (out[1] - mean).abs().max().item() <= 1.6e-2
+    one = v[2][:, 77:78, :].expand(H, L, D).float()
+    assert (out[2] - one).abs().max().item() <= 2 ** -7 * one.abs().max().item()
+    # values at dropped keys do not matter, NaN and infinity included in K and V... as long as they are finite in K (0 * inf)
+    k2, v2 = k.clone(), v.clone()
+    for b in range(B):
+        k2[b][:, ~m[b], :] = 50.0
+        v2[b][:, ~m[b], :] = -1e4
+    again = af3.dot_product_attention_cpp(*dev(q, k2, v2, m, bias)).float().cpu()
+    live_rows = [b for b in range(B) if m[b].any()]
+    assert torch.equal(again[live_rows], out[live_rows])
+    # fp32 bias (exact in this kernel's workspace), fp32 output through the lean op, no bias at all, strided inputs
+    run_case(af3, oracle, q, k, v, m, bias.float())
+    dq, dk, dv, dm = dev(q, k, v, m)
+    nob = af3.dot_product_attention_cpp(dq, dk, dv, dm, None)
+    want0 = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), np.zeros((H, L, L), np.float32))
+    assert np.abs(f32np(nob) - want0).max() <= 2e-2
+    big = torch.randn(B, H, L, 3 * D, generator=torch.Generator().manual_seed(42)).to(torch.bfloat16)
+    qs, ks, vs = big[..., :D], big[..., D:2 * D], big[..., 2 * D:]
+    run_case(af3, oracle, qs, ks, vs, m, bias)
+
+
+def test_shared_bias_kernel_moves_its_reference(rows_kernel, oracle):
+    """Logits that grow along the row, isolated spikes, rows of hugely negative biases, masking expressed through the bias,
+    the reference harness's large-mean recipe and -inf entries: the rare path of every one of the four row chains."""
+    af3 = rows_kernel
+    B, H, L, D = 6, 2, 512, 32
+    q, k, v, m, bias0 = rand_inputs(B, H, L, D, torch.bfloat16, seed=99)
+    bias = (bias0.float() + torch.linspace(-40.0, 60.0, L)[None, None, :]).to(torch.bfloat16)
+    bias[:, 5, 300] = 120.0
+    bias[:, 7, :] = -3.0e4
+    bias[:, 9, :40] = -1.0e9
+    bias[:, 11, 1:] = float("-inf")
+    run_case(af3, oracle, q, k, v, m, bias)
+    g = torch.Generator().manual_seed(1896)
+    q, k, v = [(torch.randn(B, H, L, D, generator=g) * 2 + 3).to(torch.bfloat16) for _ in range(3)]
+    bias = (torch.randn(H, L, L, generator=g) * 2 + 3).to(torch.bfloat16)
+    # outputs are 3 +- 2 here and logits 50 +- 20, so the softmax is nearly one-hot and the bf16 rounding of the scaled q alone
+    # moves single weights by percents: judged by the harness's own relative-L1 measure (examples/dot_product_attention.py:129-134)
+    out = f32np(af3.dot_product_attention_cpp(*dev(q, k, v, m, bias)))
+    want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), f32np(bias))
+    assert np.isfinite(out).all()
+    assert np.abs(out - want).sum() / np.abs(want).sum() <= 5e-3
+    assert np.abs(out - want).max() <= 0.25
+
+
 # ---- element-wise kernels -------------------------------------------------------------------
 
 def test_convert_matches_torch_casts(af3):

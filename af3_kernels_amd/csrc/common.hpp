@@ -68,6 +68,7 @@ int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s);
 int launch_dpa_mfma_fp8(const af3_dpa_params& p, hipStream_t s);
 // dpa_mfma_rows.hip: the bf16 kernel for batches that share a bias (four batch rows per wavefront); the caller has checked mfma_bf16_eligible
 bool mfma_rows_eligible(const af3_dpa_params& p);
+bool mfma_rows_can_serve(const af3_dpa_params& p);   // eligible, and its bias can be served (workspace given, or readable in place)
 int64_t mfma_rows_workspace_bytes(const af3_dpa_params& p);
 int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s);
 bool mfma_bf16_eligible(const af3_dpa_params& p);

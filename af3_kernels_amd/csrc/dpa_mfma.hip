@@ -997,12 +997,12 @@ static int64_t ws_bytes_needed(const af3_dpa_params& p) {
 }
 
 // Whether the call goes to the kernel of dpa_mfma_rows.hip (four batch rows per wavefront sharing each bias tile): its
-// shape limits, enough workgroups to give every compute unit one (smaller launches do better with this file's key-split
-// variants), and the caller's hint (af3_dpa_params.reserved: 1 = take it whenever the shape allows, 2 = never).
+// shape limits, enough workgroups of four-row groups to give every compute unit one (smaller launches do better with this
+// file's variants: measured on 5 x 16 x 1536 x 24, 72 us here against 109 us there), and the caller's hint (af3_dpa_params.reserved: 1 = take it whenever the shape allows, 2 = never).
 static bool rows_kernel_wanted(const af3_dpa_params& p) {
 	if(p.reserved == 2 || !mfma_rows_eligible(p)) return false;
 	if(p.reserved == 1) return true;
-	return ((p.B + 3) / 4) * p.H * ((p.L + 127) / 128) >= 256;
+	return (p.B / 4) * p.H * ((p.L + 127) / 128) >= 256;  // (workgroups of the launch that takes the groups of four rows)
 }
 
 // The rewrite costs one extra pass over the bias; it pays off as soon as two batch rows share it.
@@ -1159,8 +1159,7 @@ static int launch_nw(const af3_dpa_params& p, hipStream_t s) {
 }
 
 int launch_dpa_mfma_bf16(const af3_dpa_params& p, hipStream_t s) {
-	if(rows_kernel_wanted(p) && (!p.bias || (p.workspace && p.workspace_bytes >= mfma_rows_workspace_bytes(p) && (reinterpret_cast<uintptr_t>(p.workspace) & 15) == 0)))
-		return launch_dpa_mfma_rows(p, s);
+	if(rows_kernel_wanted(p) && mfma_rows_can_serve(p)) return launch_dpa_mfma_rows(p, s);
 	const bool bf32   = p.bias && p.bias_dtype == AF3_F32;
 	const bool use_ws = p.bias && p.workspace && mfma_bf16_workspace_bytes(p) > 0 && p.workspace_bytes >= ws_bytes_needed(p) &&
 						(reinterpret_cast<uintptr_t>(p.workspace) & 15) == 0;

@@ -23,11 +23,9 @@ namespace af3 {
 
 namespace {
 
-constexpr int ROWS   = 4;                  // batch rows per wavefront
 constexpr int KT_R   = 32;                 // keys per tile
 constexpr int NBUF_R = 3;                  // tile buffers
 constexpr int TILE_R = KT_R * 32 * 2;      // bytes of one tensor's tile of one batch row (head_dim padded to 32)
-constexpr int BUF_R  = ROWS * 2 * TILE_R;  // one buffer: [row][K tile | V tile]
 constexpr int MAX_L_ROWS = 4096;           // mask table: 8 bytes per key for the four rows
 constexpr float BIAS_FLOOR = -0x1p17f;     // lowest value the rewritten bias holds (log2 units)
 
@@ -84,19 +82,27 @@ __global__ void __launch_bounds__(256) bias_rows_prepass_kernel(const void* __re
 	}
 }
 
-// NW: wavefronts per workgroup (= ROWS: wavefront w fetches the tiles of batch row w).  HAS_BIAS: false = no bias at all.
-template <int NW, bool HAS_BIAS>
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) dpa_rows_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups) {
-	static_assert(NW == ROWS, "wavefront w fetches the K and V tiles of batch row w");
-	constexpr int SLOT_BASE = NBUF_R * BUF_R;                       // per-wavefront bias slots (4 KB each)
-	constexpr int MASK_BASE = SLOT_BASE + (HAS_BIAS ? NW * 4096 : 0);
+// ROWS: batch rows per wavefront (2, 3 or 4); a workgroup is always four wavefronts = 128 query rows, and wavefront w < ROWS
+// fetches the K and V tiles of batch row w.
+// BMODE: 0 = no bias (C operand zero); 1 = bias from the rewritten fp32 workspace, one 4 KB fragment per tile through this
+// wavefront's LDS slot; 2 = bf16 bias read in place (no workspace: for batches too small to pay for the rewrite), four
+// 8-byte loads per lane and tile, converted to the accumulator layout in registers.
+// The launch covers batch rows [b_first, b_first + b_count) in groups of ROWS.
+template <int ROWS, int BMODE>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) dpa_rows_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups, int64_t b_first, int64_t b_count) {
+	static_assert(ROWS >= 2 && ROWS <= 4, "two to four row chains per wavefront");
+	constexpr int  NW       = 4;
+	constexpr bool HAS_BIAS = BMODE != 0, SLOT = BMODE == 1, DIRECT = BMODE == 2;
+	constexpr int  BUF_R    = ROWS * 2 * TILE_R;                    // one buffer: [row][K tile | V tile]
+	constexpr int  SLOT_BASE = NBUF_R * BUF_R;                      // per-wavefront bias slots (4 KB each)
+	constexpr int  MASK_BASE = SLOT_BASE + (SLOT ? NW * 4096 : 0);
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 	// [buffer 3][batch row 4][K tile 2 KB | V tile 2 KB] [bias slot 4 KB per wavefront] [mask table: (tiles + 1) x 4 rows x 32 keys, bf16 bits]
 	const int64_t L        = p.L;
 	const int     D        = (int)p.D;
 	const int     n_t_all  = (int)((L + KT_R - 1) / KT_R);
 	uint16_t* const mask_tab = reinterpret_cast<uint16_t*>(smem + MASK_BASE);
-	__shared__ int  s_last[ROWS];  // index of the last live key + 1 of each batch row (0: every key dropped)
+	__shared__ int  s_last[4];  // index of the last live key + 1 of each batch row (0: every key dropped)
 
 	// ---- workgroup -> (group of batch rows, head, query tile): all query tiles of one (group, head) get ids congruent
 	// mod 8, i.e. the same XCD (they share that XCD's L2 copy of K and V), and an XCD only sees heads xcd % H (for H | 8),
@@ -108,7 +114,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 	const int     qtile = (int)(slot % n_qtiles);
 	if(group >= n_groups) return;
 	const int64_t g = group / p.H, h = group % p.H;
-	const int64_t b0 = g * ROWS;
+	const int64_t b0 = b_first + g * ROWS, b_end = b_first + b_count;   // (rows past b_end repeat the last one and are not stored)
 
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -120,9 +126,9 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 		for(int i = tid; i < NBUF_R * BUF_R / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
 
 	// ---- key-mask table: entry = additive mask value of (tile, batch row, key) as bf16 bits; wavefront w fills row w ----
-	{
+	if(wave < ROWS) {
 		const int      r    = wave;
-		const int64_t  br   = b0 + r < p.B ? b0 + r : p.B - 1;
+		const int64_t  br   = b0 + r < b_end ? b0 + r : b_end - 1;
 		const uint8_t* keep = p.key_mask ? p.key_mask + br * p.key_mask_stride_b : nullptr;
 		int            last = 0;
 		for(int base = 0; base < (n_t_all + 1) * KT_R; base += 64) {
@@ -162,7 +168,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 	bf16x8 qf[ROWS][2];
 #pragma unroll
 	for(int r = 0; r < ROWS; r++) {
-		const int64_t   br   = b0 + r < p.B ? b0 + r : p.B - 1;
+		const int64_t   br   = b0 + r < b_end ? b0 + r : b_end - 1;
 		const float     qmul = dropped[r] ? 0.f : p.softmax_scale * LOG2E;
 		const uint16_t* qp   = static_cast<const uint16_t*>(p.q) + br * p.q_stride[0] + h * p.q_stride[1] + qrow * p.q_stride[2];
 #pragma unroll
@@ -194,7 +200,8 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 	// tile (K rows 0-15, 16-31, V rows 0-15, 16-31; lane i -> tile row i/4, 16-byte chunk i%4, K chunks swizzled), and
 	// the four 1 KB pieces of its own bias fragment.  Lanes of padded head columns carry an offset beyond the buffer's
 	// range: the hardware fetches nothing for them. ----
-	const int64_t b_ld   = b0 + wave < p.B ? b0 + wave : p.B - 1;
+	const int64_t b_ld   = b0 + wave < b_end ? b0 + wave : b_end - 1;
+	const bool    loader = wave < ROWS;  // (wave-uniform)
 	const u32x4   k_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.k) + b_ld * p.k_stride[0] + h * p.k_stride[1], (uint32_t)(((L - 1) * p.k_stride[2] + D) * 2));
 	const u32x4   v_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.v) + b_ld * p.v_stride[0] + h * p.v_stride[1], (uint32_t)(((L - 1) * p.v_stride[2] + D) * 2));
 	const int     ld_row = lane >> 2, ld_pc = lane & 3;
@@ -205,6 +212,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 	const int     k_pc_stride = (int)(16 * p.k_stride[2] * 2), v_pc_stride = (int)(16 * p.v_stride[2] * 2);
 	const uint32_t lds_tiles = lds_addr_of(smem) + wave * (2 * TILE_R);
 	auto load_tile = [&](int t, int buf_off) {
+		if(!loader) return;
 		lds_dma_b128(k_rsrc, lds_tiles + buf_off, k_voff + t * k_tile_stride);
 		lds_dma_b128(k_rsrc, lds_tiles + buf_off + 1024, k_voff + (t * k_tile_stride + k_pc_stride));
 		lds_dma_b128(v_rsrc, lds_tiles + buf_off + TILE_R, v_voff + t * v_tile_stride);
@@ -214,15 +222,29 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 	const int     n_qblocks = (int)((L + 31) / 32);
 	const int64_t qb        = (int64_t)qtile * NW + wave;
 	const int64_t qbc       = qb < n_qblocks ? qb : n_qblocks - 1;  // (blocks past the end only hold rows >= L)
-	const u32x4   ws_rsrc   = raw_rsrc(HAS_BIAS ? static_cast<const unsigned char*>(p.workspace) + ((h * n_qblocks + qbc) * n_t_all) * 4096 : nullptr, HAS_BIAS ? (uint32_t)(n_t_all * 4096) : 0u);
+	const u32x4   ws_rsrc   = raw_rsrc(SLOT ? static_cast<const unsigned char*>(p.workspace) + ((h * n_qblocks + qbc) * n_t_all) * 4096 : nullptr, SLOT ? (uint32_t)(n_t_all * 4096) : 0u);
 	const int      ws_voff  = lane * 16;
 	const uint32_t lds_slot = lds_addr_of(smem) + SLOT_BASE + wave * 4096;
 	auto load_bias = [&](int t) {
-		if(!HAS_BIAS) return;
+		if(!SLOT) return;
 #pragma unroll
 		for(int ld = 0; ld < 4; ld++) lds_dma_b128(ws_rsrc, lds_slot + ld * 1024, ws_voff + (t * 4096 + ld * 1024));  // (past the last tile: nothing is fetched)
 	};
-	constexpr int LOADS_PER_TILE = 4 + (HAS_BIAS ? 4 : 0);
+	// direct mode: this lane's four 8-byte pieces of a tile's bias, bias[h][q][32 t + 8 ld + 4 half .. + 3] (bf16), through a
+	// range-checked buffer over the head's slab; pieces whose keys lie at or beyond L are sent out of range and read as zero
+	[[maybe_unused]] u32x2 braw[4] = {u32x2{0u, 0u}, u32x2{0u, 0u}, u32x2{0u, 0u}, u32x2{0u, 0u}};
+	const int64_t qrow_b = qrow < L ? qrow : L - 1;
+	const __amdgpu_buffer_rsrc_t bd_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+		DIRECT ? const_cast<uint16_t*>(static_cast<const uint16_t*>(p.bias)) + h * p.bias_stride[0] : nullptr, 0, DIRECT ? (int)(((L - 1) * p.bias_stride[1] + L) * 2) : 0, 0x00020000);
+	const int bd_voff = (int)((qrow_b * p.bias_stride[1] + 4 * half) * 2);
+	auto load_bias_direct = [&](int t) {
+		if(!DIRECT) return;
+#pragma unroll
+		for(int ld = 0; ld < 4; ld++) {
+			const bool in = t * KT_R + 8 * ld + 4 * half < L;
+			braw[ld] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(bd_rsrc, in ? bd_voff + ld * 16 : 0x40000000, t * (KT_R * 2), 0));
+		}
+	};
 
 	// ---- per-lane LDS read offsets inside a (buffer, batch row) block ----
 	int k_rd[2];
@@ -308,12 +330,28 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 	u32x4  vprev[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
 #pragma unroll
 	for(int i = 0; i < 16; i++) bias_frag[i] = 0.f;
-	auto read_bias_slot = [&] {
-		if(!HAS_BIAS) return;
+	// the next tile's bias fragment -> registers: from the slot, or (direct mode) from the raw bf16 pieces loaded a tile ago:
+	// clamped from below like the workspace's values (packed unsigned minimum: -2^16 and everything beyond it, -inf and
+	// -NaN patterns included), widened to fp32 and scaled by log2 e
+	auto next_bias_fragment = [&] {
+		if constexpr(SLOT) {
 #pragma unroll
-		for(int ld = 0; ld < 4; ld++) {
-			const f32x4 v = *reinterpret_cast<const f32x4*>(smem + slot_rd + ld * 1024);
-			bias_frag[4 * ld] = v[0], bias_frag[4 * ld + 1] = v[1], bias_frag[4 * ld + 2] = v[2], bias_frag[4 * ld + 3] = v[3];
+			for(int ld = 0; ld < 4; ld++) {
+				const f32x4 v = *reinterpret_cast<const f32x4*>(smem + slot_rd + ld * 1024);
+				bias_frag[4 * ld] = v[0], bias_frag[4 * ld + 1] = v[1], bias_frag[4 * ld + 2] = v[2], bias_frag[4 * ld + 3] = v[3];
+			}
+		} else if constexpr(DIRECT) {
+			typedef __attribute__((ext_vector_type(2))) unsigned short u16x2;
+			const u16x2 lim = {(unsigned short)0xC780, (unsigned short)0xC780};
+#pragma unroll
+			for(int ld = 0; ld < 4; ld++)
+#pragma unroll
+				for(int j = 0; j < 2; j++) {
+					const uint32_t raw = braw[ld][j];
+					const uint32_t w   = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2, raw), lim));
+					bias_frag[4 * ld + 2 * j]     = __uint_as_float(w << 16) * LOG2E;
+					bias_frag[4 * ld + 2 * j + 1] = __uint_as_float(w & 0xffff0000u) * LOG2E;
+				}
 		}
 	};
 
@@ -422,34 +460,49 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 		pprev[1] = pcur[1];
 	};
 
-	// One tile: four steps.  Tile t sits in buffer t % 3.  In front of the third step the loads issued one tile earlier
-	// (tile t + 1 and its bias fragment: the youngest loads this wavefront has in flight) are awaited and a barrier
-	// publishes tile t + 1 -- the third step fetches K fragments from it -- and tells that every wavefront is done with
-	// tile t - 1, whose buffer tile t + 2 then overwrites.  The third step's first matrix instruction is the last reader
-	// of bias fragment t: behind it the fragment registers are refilled from the slot, and the slot, once those reads
-	// have returned (the last step's first matrix instruction waits for them), with fragment t + 2.
+	// One tile: ROWS steps.  Tile t sits in buffer t % 3.  In front of the last-but-one step the loads issued one tile
+	// earlier (tile t + 1 and its bias fragment: the youngest loads this wavefront has in flight) are awaited and a barrier
+	// publishes tile t + 1 -- that step fetches K fragments from it -- and tells that every wavefront is done with tile
+	// t - 1, whose buffer tile t + 2 then overwrites.  That step's first matrix instruction is the last reader of bias
+	// fragment t: behind it the fragment registers take fragment t + 1, and the slot (once those reads have returned: the
+	// last step's first matrix instruction waits for them) or the raw-piece registers are refilled with fragment t + 2.
 	auto tile = [&](auto first_c, auto anydrop_c, int t, int buf, int bufn, int bufnn) {
 		const int m0 = mask_rd + t * (ROWS * 64);
-		auto none = [] {};
-		step(ic<0>{}, first_c, anydrop_c, buf + 2 * (2 * TILE_R), m0 + 1 * 64, buf + 0 * (2 * TILE_R), none);
-		step(ic<1>{}, first_c, anydrop_c, buf + 3 * (2 * TILE_R), m0 + 2 * 64, buf + 1 * (2 * TILE_R), none);
-		asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-		step(ic<2>{}, first_c, anydrop_c, bufn + 0 * (2 * TILE_R), m0 + 3 * 64, buf + 2 * (2 * TILE_R), [&] {
-			load_tile(t + 2, bufnn);  // (past the end of the rows: nothing is fetched)
-			read_bias_slot();
-		});
-		step(ic<3>{}, first_c, anydrop_c, bufn + 1 * (2 * TILE_R), m0 + ROWS * 64, buf + 3 * (2 * TILE_R), [&] { load_bias(t + 2); });
+		auto one = [&](auto r_c) {
+			constexpr int R = decltype(r_c)::value;
+			if constexpr(R < ROWS) {
+				constexpr int R1 = R + 1, R2 = R + 2;                        // the next step and the one after it ...
+				const int     k2 = (R2 >= ROWS ? bufn : buf) + (R2 % ROWS) * (2 * TILE_R);   // ... may belong to the next tile
+				const int     m1 = m0 + R1 * 64;                             // (row ROWS of tile t is row 0 of tile t + 1)
+				const int     vc = buf + R * (2 * TILE_R);
+				if constexpr(R == ROWS - 2) {
+					asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+					step(r_c, first_c, anydrop_c, k2, m1, vc, [&] {
+						load_tile(t + 2, bufnn);  // (past the end of the rows: nothing is fetched)
+						next_bias_fragment();
+						load_bias_direct(t + 2);
+					});
+				} else if constexpr(R == ROWS - 1) {
+					step(r_c, first_c, anydrop_c, k2, m1, vc, [&] { load_bias(t + 2); });
+				} else {
+					step(r_c, first_c, anydrop_c, k2, m1, vc, [] {});
+				}
+			}
+		};
+		one(ic<0>{}), one(ic<1>{}), one(ic<2>{}), one(ic<3>{});
 	};
 	auto run = [&](auto anydrop_c) {
 		constexpr bool ANYDROP = decltype(anydrop_c)::value != 0;
 		// ---- prologue: the first two tiles, the first two bias fragments, S^T of the first step, K fragments of the second ----
 		load_tile(0, 0);
 		load_bias(0);
+		load_bias_direct(0);
 		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-		read_bias_slot();  // fragment 0 -> registers
+		next_bias_fragment();  // fragment 0 -> registers
 		asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 		load_tile(1, BUF_R);
 		load_bias(1);
+		load_bias_direct(1);
 		__syncthreads();   // tile 0 is complete (every wavefront has waited for its own pieces)
 		{
 			f32x16 s0;
@@ -482,18 +535,31 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 	oacc[ROWS - 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[0]), __builtin_bit_cast(bf16x8, pprev[0]), oacc[ROWS - 1], 0, 0, 0);
 	oacc[ROWS - 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[1]), __builtin_bit_cast(bf16x8, pprev[1]), oacc[ROWS - 1], 0, 0, 0);
 
-	// ---- epilogue: O^T register i is head column 8*(i/4) + 4*half + i%4 ----
+	// ---- epilogue: O^T register i is head column 8*(i/4) + 4*half + i%4; optional output gate (out *= sigmoid(gate), the
+	// reference's "weighted_avg *= sigmoid(gating_query(pair))", src/csrc/dot_product_attention.cpp:335-349) ----
 	if(row_ok) {
 #pragma unroll
 		for(int r = 0; r < ROWS; r++) {
-			if(b0 + r >= p.B) break;
+			if(b0 + r >= b_end) break;
 			const float   inv  = 1.f / lsum[r];
 			const int64_t ooff = (b0 + r) * p.out_stride[0] + h * p.out_stride[1] + qrow * p.out_stride[2];
+			u32x2         gw[4] = {u32x2{0u, 0u}, u32x2{0u, 0u}, u32x2{0u, 0u}, u32x2{0u, 0u}};
+			if(p.gate) {
+				const uint16_t* gp = static_cast<const uint16_t*>(p.gate) + (b0 + r) * p.gate_stride[0] + h * p.gate_stride[1] + qrow * p.gate_stride[2];
+#pragma unroll
+				for(int g4 = 0; g4 < 4; g4++)
+					if(8 * g4 + 4 * half < D) gw[g4] = *reinterpret_cast<const u32x2*>(gp + 8 * g4 + 4 * half);
+			}
 #pragma unroll
 			for(int g4 = 0; g4 < 4; g4++) {
 				const int d0 = 8 * g4 + 4 * half;
 				if(d0 >= D) continue;
-				const float o0 = oacc[r][4 * g4] * inv, o1 = oacc[r][4 * g4 + 1] * inv, o2 = oacc[r][4 * g4 + 2] * inv, o3 = oacc[r][4 * g4 + 3] * inv;
+				float o0 = oacc[r][4 * g4] * inv, o1 = oacc[r][4 * g4 + 1] * inv, o2 = oacc[r][4 * g4 + 2] * inv, o3 = oacc[r][4 * g4 + 3] * inv;
+				if(p.gate) {
+					const uint32_t g0 = gw[g4][0], g1 = gw[g4][1];
+					o0 *= sigmoidf_fast(bf16_bits_to_f32(g0 & 0xffffu)), o1 *= sigmoidf_fast(bf16_bits_to_f32(g0 >> 16));
+					o2 *= sigmoidf_fast(bf16_bits_to_f32(g1 & 0xffffu)), o3 *= sigmoidf_fast(bf16_bits_to_f32(g1 >> 16));
+				}
 				if(p.out_dtype == AF3_BF16) {
 					const u32x2 w = {pack_bf16x2(o0, o1), pack_bf16x2(o2, o3)};
 					*reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.out) + ooff + d0) = w;
@@ -506,46 +572,72 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 	}
 }
 
-size_t rows_lds_bytes(const af3_dpa_params& p) {
-	const size_t n_t_all = (size_t)((p.L + KT_R - 1) / KT_R);
-	return (size_t)NBUF_R * BUF_R + (p.bias ? ROWS * 4096 : 0) + (n_t_all + 1) * ROWS * 32 * 2;
-}
-
 int64_t rows_ws_bytes(const af3_dpa_params& p) {
 	const int64_t n_qblocks = (p.L + 31) / 32, n_t_all = (p.L + KT_R - 1) / KT_R;
 	return p.H * n_qblocks * n_t_all * 4096;
 }
 
-template <int NW, bool HAS_BIAS>
-int launch_rows(const af3_dpa_params& p, hipStream_t s) {
-	const int     n_qtiles = (int)((p.L + NW * 32 - 1) / (NW * 32));
-	const int64_t n_groups = ((p.B + ROWS - 1) / ROWS) * p.H;
+// The bf16 bias can be read in place when its rows start on 8-byte boundaries, keys come in whole groups of four and the
+// slab of one head fits 32-bit byte offsets.
+bool direct_bias_ok(const af3_dpa_params& p) {
+	return p.bias && p.bias_dtype == AF3_BF16 && p.L % 4 == 0 && (reinterpret_cast<uintptr_t>(p.bias) & 7) == 0 && p.bias_stride[0] % 4 == 0 && p.bias_stride[1] % 4 == 0 &&
+		   ((p.L - 1) * p.bias_stride[1] + p.L) * 2 < 0x40000000LL;
+}
+
+// 0 = no bias, 1 = through the rewritten workspace, 2 = read in place, -1 = this kernel cannot serve the call.  The
+// rewrite costs three passes over the bias and pays off from four groups of batch rows on.
+int rows_bias_mode(const af3_dpa_params& p) {
+	if(!p.bias) return 0;
+	const bool ws_ok = p.workspace && p.workspace_bytes >= rows_ws_bytes(p) && (reinterpret_cast<uintptr_t>(p.workspace) & 15) == 0;
+	if(p.B >= 16 && ws_ok) return 1;
+	if(direct_bias_ok(p)) return 2;
+	return ws_ok ? 1 : -1;
+}
+
+template <int ROWS, int BMODE>
+int launch_rows(const af3_dpa_params& p, int64_t b_first, int64_t b_count, hipStream_t s) {
+	const int     n_qtiles = (int)((p.L + 127) / 128);
+	const int64_t n_groups = ((b_count + ROWS - 1) / ROWS) * p.H;
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
-	const size_t smem = rows_lds_bytes(p);
-	auto         kern = dpa_rows_bf16_kernel<NW, HAS_BIAS>;
+	const size_t n_t_all = (size_t)((p.L + KT_R - 1) / KT_R);
+	const size_t smem    = (size_t)NBUF_R * ROWS * 2 * TILE_R + (BMODE == 1 ? 4 * 4096 : 0) + (n_t_all + 1) * ROWS * 32 * 2;
+	auto         kern    = dpa_rows_bf16_kernel<ROWS, BMODE>;
 	if(smem > 64 * 1024) {
 		if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
 	}
-	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, n_qtiles, n_groups);
+	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), smem, s, p, n_qtiles, n_groups, b_first, b_count);
 	return launch_status();
+}
+
+template <int BMODE>
+int launch_rows_n(int rows, const af3_dpa_params& p, int64_t b_first, int64_t b_count, hipStream_t s) {
+	return rows == 4 ? launch_rows<4, BMODE>(p, b_first, b_count, s) : rows == 3 ? launch_rows<3, BMODE>(p, b_first, b_count, s) : launch_rows<2, BMODE>(p, b_first, b_count, s);
 }
 
 }  // namespace
 
 // Shapes the kernel takes: what dpa_mfma.hip's kernel takes (mfma_bf16_eligible, checked by the caller), and in addition
-// head_dim <= 32, at least four batch rows, no output gate, and a length whose mask table fits beside the tile buffers.
+// head_dim <= 32, at least two batch rows, a length whose mask table fits beside the tile buffers, 8-byte aligned gate rows.
 bool mfma_rows_eligible(const af3_dpa_params& p) {
-	if(p.D > 32 || p.B < ROWS || p.gate || p.L > MAX_L_ROWS) return false;
-	// buffer addressing of the bias workspace of one (head, query block) uses 32-bit byte offsets
-	if(((p.L + KT_R - 1) / KT_R) * 4096 >= 0x7fffffffLL) return false;
+	if(p.D > 32 || p.B < 2 || p.L > MAX_L_ROWS) return false;
+	if(p.gate && ((reinterpret_cast<uintptr_t>(p.gate) & 7) || p.gate_stride[0] % 4 || p.gate_stride[1] % 4 || p.gate_stride[2] % 4)) return false;
 	return true;
 }
 
-int64_t mfma_rows_workspace_bytes(const af3_dpa_params& p) { return p.bias ? rows_ws_bytes(p) : 0; }
+// Workspace the call would use: none when the bias is better read in place (few batch rows).
+int64_t mfma_rows_workspace_bytes(const af3_dpa_params& p) {
+	if(!p.bias) return 0;
+	if(p.B < 16 && direct_bias_ok(p)) return 0;
+	return rows_ws_bytes(p);
+}
+
+bool mfma_rows_can_serve(const af3_dpa_params& p) { return mfma_rows_eligible(p) && rows_bias_mode(p) >= 0; }
 
 int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
-	if(p.bias) {
+	const int mode = rows_bias_mode(p);
+	if(mode < 0) return AF3_ERR_BAD_ARGUMENT;
+	if(mode == 1) {
 		const bool     bf32      = p.bias_dtype == AF3_F32;
 		const int      n_qblocks = (int)((p.L + 31) / 32), n_t_all = (int)((p.L + KT_R - 1) / KT_R);
 		const int64_t  total     = p.H * n_qblocks * (int64_t)n_t_all * 256;
@@ -560,9 +652,31 @@ int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
 							   n_qblocks, n_t_all, vec_ok);
 		const int rc = launch_status();
 		if(rc != AF3_OK) return rc;
-		return launch_rows<4, true>(p, s);
 	}
-	return launch_rows<4, false>(p, s);
+	// The batch in groups of four rows, the remainder as one group of two or three (a remainder of one borrows a row:
+	// ... 4, 3, 2); every group of one launch has the same number of rows.
+	const int64_t B = p.B;
+	int64_t       n4 = B / 4, rem = B % 4;
+	int           tail[2] = {0, 0};
+	if(rem == 1) {
+		if(n4 >= 1) n4 -= 1, tail[0] = 3, tail[1] = 2;
+		else return AF3_ERR_BAD_SHAPE;  // (B == 1 is not eligible)
+	} else if(rem != 0) {
+		tail[0] = (int)rem;
+	}
+	int64_t done = 0;
+	if(n4 > 0) {
+		const int rc = mode == 0 ? launch_rows<4, 0>(p, 0, 4 * n4, s) : mode == 1 ? launch_rows<4, 1>(p, 0, 4 * n4, s) : launch_rows<4, 2>(p, 0, 4 * n4, s);
+		if(rc != AF3_OK) return rc;
+		done = 4 * n4;
+	}
+	for(int i = 0; i < 2; i++) {
+		if(tail[i] == 0) continue;
+		const int rc = mode == 0 ? launch_rows_n<0>(tail[i], p, done, tail[i], s) : mode == 1 ? launch_rows_n<1>(tail[i], p, done, tail[i], s) : launch_rows_n<2>(tail[i], p, done, tail[i], s);
+		if(rc != AF3_OK) return rc;
+		done += tail[i];
+	}
+	return AF3_OK;
 }
 
 }  // namespace af3

@@ -457,10 +457,34 @@ def rows_kernel(af3):
     (4, 4, 128, 32, "none", 2), (5, 2, 200, 32, "random", 2), (8, 4, 384, 32, "tail", 2), (7, 3, 37, 24, "random", 2),
     (4, 1, 65, 16, "tail", 1), (9, 4, 1000, 32, "random", 2), (4, 2, 96, 8, "none", 1), (6, 16, 256, 24, "tail", 1),
     (13, 1, 1, 32, "none", 2), (4, 5, 33, 32, "random", 2), (12, 4, 1491, 32, "random", 2),
+    (2, 4, 128, 32, "none", 2), (3, 2, 200, 32, "random", 2), (5, 16, 256, 24, "tail", 1), (6, 3, 36, 24, "random", 2),   # groups of two and three rows
+    (17, 2, 100, 32, "random", 2), (18, 2, 37, 32, "random", 2), (19, 1, 64, 16, "tail", 2),                          # 4 ... 4 + 3 + 2, + 2, + 3
 ])
 def test_shared_bias_kernel_matches_formula(rows_kernel, oracle, B, H, L, D, mask, rank):
+    """Every way the batch is cut into groups of four, three and two rows, with the bias through the rewritten workspace
+    (16 batch rows and more) or read in place (fewer; lengths that are not multiples of 4 then leave the call to the
+    one-row kernel), and again without a workspace at all (set_exact_bias: in place whenever the layout allows)."""
     q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=5 * L + D + B, mask=mask, mask_rank=rank)
+    if B >= 6:
+        m = m.clone() if m.dim() == 2 else m
+        if m.dim() == 2:
+            m[B - 1, :] = False                # a batch row without live keys in the last (partial) group
     run_case(rows_kernel, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+    prev = rows_kernel.set_exact_bias(True)
+    try:
+        run_case(rows_kernel, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+    finally:
+        rows_kernel.set_exact_bias(prev)
+
+
+def test_shared_bias_kernel_applies_the_output_gate(rows_kernel, oracle):
+    from af3_kernels_amd import ops, _lib
+    B, H, L, D = 6, 4, 200, 32
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=7, mask="random")
+    g = torch.randn(B, H, L, D, generator=torch.Generator().manual_seed(8)).to(torch.bfloat16)
+    out = ops._dpa_forward_impl(q.cuda(), k.cuda(), v.cuda(), ops._lift_mask(m.cuda(), L), bias.cuda(), _lib.AF3_BF16, False, gate=g.cuda())
+    want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), f32np(bias)) / (1.0 + np.exp(-f32np(g)))
+    assert np.abs(f32np(out) - want).max() <= 2e-2
 
 
 def test_shared_bias_kernel_agrees_with_the_one_row_kernel(af3):

@@ -653,28 +653,53 @@ int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
 		const int rc = launch_status();
 		if(rc != AF3_OK) return rc;
 	}
-	// The batch in groups of four rows, the remainder as one group of two or three (a remainder of one borrows a row:
-	// ... 4, 3, 2); every group of one launch has the same number of rows.
-	const int64_t B = p.B;
-	int64_t       n4 = B / 4, rem = B % 4;
-	int           tail[2] = {0, 0};
-	if(rem == 1) {
-		if(n4 >= 1) n4 -= 1, tail[0] = 3, tail[1] = 2;
-		else return AF3_ERR_BAD_SHAPE;  // (B == 1 is not eligible)
-	} else if(rem != 0) {
-		tail[0] = (int)rem;
+	// The batch is cut into groups of `rows` batch rows per wavefront, the remainder into groups of two or three (a
+	// remainder of one borrows from the last full group); every group of one launch has the same number of rows.  Four
+	// rows share a bias tile best, but what counts is how evenly the workgroups fill the GPU's 512 slots (two per
+	// compute unit): the launch time is about (rounds of 512 workgroups) x (rows per group) x (cost per row, which grows
+	// as fewer rows share a tile: measured 1 : 1.075 : 1.09 for 4 : 3 : 2 rows), and the cheapest plan is taken.
+	const int64_t B = p.B, per_row_wgs = p.H * ((p.L + 127) / 128);
+	auto plan = [&](int rows, int64_t (&count)[3], int (&rows_of)[3]) -> double {
+		static const double cost_per_row[5] = {0, 0, 1.09, 1.075, 1.0};
+		int64_t full = B / rows, rem = B % rows;
+		int     n    = 0;
+		if(rem == 1 && rows > 2) {
+			if(full >= 1) full -= 1, rem += rows;  // e.g. 4 + 1 -> 3 + 2
+			else return 1e30;
+		} else if(rem == 1) {
+			return 1e30;  // (rows == 2 and an odd batch: another plan serves it)
+		}
+		if(full > 0) count[n] = full * rows, rows_of[n] = rows, n++;
+		if(rem == 5) count[n] = 3, rows_of[n] = 3, n++, count[n] = 2, rows_of[n] = 2, n++;
+		else if(rem == 4) count[n] = 2, rows_of[n] = 2, n++, count[n] = 2, rows_of[n] = 2, n++;   // (rows == 3: 3 + 1 -> 2 + 2)
+		else if(rem > 0) count[n] = rem, rows_of[n] = (int)rem, n++;
+		for(int i = n; i < 3; i++) count[i] = 0, rows_of[i] = 0;
+		double t = 0;
+		for(int i = 0; i < n; i++) {
+			const int64_t wgs = ((count[i] + rows_of[i] - 1) / rows_of[i]) * per_row_wgs;
+			t += (double)((wgs + 511) / 512) * rows_of[i] * cost_per_row[rows_of[i]];
+		}
+		return t;
+	};
+	int64_t count[3] = {0, 0, 0};
+	int     rows_of[3] = {0, 0, 0};
+	double  best = 1e30;
+	for(int rows = 4; rows >= 2; rows--) {
+		int64_t c[3];
+		int     r[3];
+		const double t = plan(rows, c, r);
+		if(t < best * 0.999) {
+			best = t;
+			for(int i = 0; i < 3; i++) count[i] = c[i], rows_of[i] = r[i];
+		}
 	}
+	if(best >= 1e30) return AF3_ERR_BAD_SHAPE;  // (B == 1 is not eligible)
 	int64_t done = 0;
-	if(n4 > 0) {
-		const int rc = mode == 0 ? launch_rows<4, 0>(p, 0, 4 * n4, s) : mode == 1 ? launch_rows<4, 1>(p, 0, 4 * n4, s) : launch_rows<4, 2>(p, 0, 4 * n4, s);
+	for(int i = 0; i < 3; i++) {
+		if(count[i] == 0) continue;
+		const int rc = mode == 0 ? launch_rows_n<0>(rows_of[i], p, done, count[i], s) : mode == 1 ? launch_rows_n<1>(rows_of[i], p, done, count[i], s) : launch_rows_n<2>(rows_of[i], p, done, count[i], s);
 		if(rc != AF3_OK) return rc;
-		done = 4 * n4;
-	}
-	for(int i = 0; i < 2; i++) {
-		if(tail[i] == 0) continue;
-		const int rc = mode == 0 ? launch_rows_n<0>(tail[i], p, done, tail[i], s) : mode == 1 ? launch_rows_n<1>(tail[i], p, done, tail[i], s) : launch_rows_n<2>(tail[i], p, done, tail[i], s);
-		if(rc != AF3_OK) return rc;
-		done += tail[i];
+		done += count[i];
 	}
 	return AF3_OK;
 }

@@ -122,78 +122,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 
 	// ---- zero the tile buffers when a load can leave parts of them unwritten (padded head columns, rows past L):
 	// stale LDS contents there must be finite ----
-	if(D != 32 || L % KT_R != 0)
+	if(D != 32 || L % KT_R != 0) {
 		for(int i = tid; i < NBUF_R * BUF_R / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
-
-	// ---- key-mask table: entry = additive mask value of (tile, batch row, key) as bf16 bits; wavefront w fills row w ----
-	if(wave < ROWS) {
-		const int      r    = wave;
-		const int64_t  br   = b0 + r < b_end ? b0 + r : b_end - 1;
-		const uint8_t* keep = p.key_mask ? p.key_mask + br * p.key_mask_stride_b : nullptr;
-		int            last = 0;
-		for(int base = 0; base < (n_t_all + 1) * KT_R; base += 64) {
-			const int  key  = base + lane;
-			const bool in   = key < L;
-			const bool live = in && (keep ? keep[key] != 0 : true);
-			if(key < (n_t_all + 1) * KT_R) mask_tab[((key >> 5) * ROWS + r) * 32 + (key & 31)] = live ? (uint16_t)0 : (in ? MASK_DROPPED_BF16 : MASK_OUT_OF_RANGE_BF16);
-			const unsigned long long bal = __ballot(live);
-			if(bal) last = base + 64 - __builtin_clzll(bal);
-		}
-		// A batch row without any live key yields the mean over all L keys (masked_fill(-1e9) + softmax in
-		// examples/dot_product_attention.py:37-39): its keys count as live, and q and the bias are dropped for it
-		// below, so that all its logits are exactly equal.
-		if(last == 0)
-			for(int key = lane; key < (n_t_all + 1) * KT_R; key += 64) mask_tab[((key >> 5) * ROWS + r) * 32 + (key & 31)] = key < L ? (uint16_t)0 : MASK_OUT_OF_RANGE_BF16;
-		if(lane == 0) s_last[r] = last;
+		__syncthreads();
 	}
-	__syncthreads();
-	// keys behind the last live key of every row carry weight 0 and are not walked; a row without live keys needs them all
-	int  l_eff = 0;
-	bool dropped[ROWS];
-#pragma unroll
-	for(int r = 0; r < ROWS; r++) {
-		const int last = __builtin_amdgcn_readfirstlane(s_last[r]);
-		dropped[r]     = last == 0;
-		const int need = dropped[r] ? (int)L : last;
-		l_eff          = need > l_eff ? need : l_eff;
-	}
-	const int n_t = (l_eff + KT_R - 1) / KT_R;
 
 	// ---- per-lane constants ----
 	const int64_t qrow   = (int64_t)qtile * (NW * 32) + wave * 32 + n;
 	const bool    row_ok = qrow < L;
-	// Q fragments (B operand of S^T = K.Q^T): lane (q = n, g = half) holds q[q][16c + 8g .. +7], scaled by
-	// softmax_scale * log2 e in fp32 and rounded once to bf16 (the reference rounds the scaled q too,
-	// src/csrc/dot_product_attention.cpp:95-98).  A batch row without live keys gets q = 0.
-	bf16x8 qf[ROWS][2];
-#pragma unroll
-	for(int r = 0; r < ROWS; r++) {
-		const int64_t   br   = b0 + r < b_end ? b0 + r : b_end - 1;
-		const float     qmul = dropped[r] ? 0.f : p.softmax_scale * LOG2E;
-		const uint16_t* qp   = static_cast<const uint16_t*>(p.q) + br * p.q_stride[0] + h * p.q_stride[1] + qrow * p.q_stride[2];
-#pragma unroll
-		for(int c = 0; c < 2; c++) {
-			const int d0  = 16 * c + 8 * half;
-			u32x4     raw = {0u, 0u, 0u, 0u};
-			if(row_ok && d0 < D) raw = *reinterpret_cast<const u32x4*>(qp + d0);
-			u32x4 sc4;
-#pragma unroll
-			for(int j = 0; j < 4; j++) {
-				const uint32_t w = raw[j];
-				sc4[j] = pack_bf16x2(bf16_bits_to_f32(w & 0xffffu) * qmul, bf16_bits_to_f32(w >> 16) * qmul);
-			}
-			qf[r][c] = __builtin_bit_cast(bf16x8, sc4);
-		}
-	}
-	// Operands of the mask MFMA (v_mfma_f32_32x32x8_bf16: four contraction slots per half-wave, two registers per operand).
-	// A (per key): slot 0 = the key's mask value (from the table, zero-extended), slots 2 and 3 = 1.0.
-	// B (per query): slot 0 = 1.0, slots 2 and 3 = -m_hi and -m_lo, the softmax reference of this lane's query row as two
-	// bf16 terms (16 significant bits).  Lanes of the upper half-wave supply slots 4..7: their B is zero, so whatever
-	// finite value their A holds contributes nothing.
-	u32x2 maskA = {0u, 0x3F803F80u};
-	u32x2 maskB[ROWS];
-#pragma unroll
-	for(int r = 0; r < ROWS; r++) maskB[r] = u32x2{half == 0 ? 0x3F80u : 0u, 0u};
+	int n_t = 1;   // key tiles to walk: known once the key masks are read; the first tile is always walked
 
 	// ---- tile and bias loaders: loads that write LDS directly (no registers, invisible to the compiler's wait counting;
 	// every wait for them below is explicit).  This wavefront fetches K and V of batch row `wave`: four 1 KB pieces per
@@ -211,12 +148,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	const int     k_tile_stride = (int)(KT_R * p.k_stride[2] * 2), v_tile_stride = (int)(KT_R * p.v_stride[2] * 2);
 	const int     k_pc_stride = (int)(16 * p.k_stride[2] * 2), v_pc_stride = (int)(16 * p.v_stride[2] * 2);
 	const uint32_t lds_tiles = lds_addr_of(smem) + wave * (2 * TILE_R);
+	auto load_tile_piece = [&](int t, int buf_off, auto pc_c) {
+		constexpr int PC = decltype(pc_c)::value;
+		if(!loader || t >= n_t) return;   // (no request for a tile the walk stops short of: nothing is in flight when the kernel ends)
+		if constexpr(PC == 0) lds_dma_b128(k_rsrc, lds_tiles + buf_off, k_voff + t * k_tile_stride);
+		if constexpr(PC == 1) lds_dma_b128(k_rsrc, lds_tiles + buf_off + 1024, k_voff + (t * k_tile_stride + k_pc_stride));
+		if constexpr(PC == 2) lds_dma_b128(v_rsrc, lds_tiles + buf_off + TILE_R, v_voff + t * v_tile_stride);
+		if constexpr(PC == 3) lds_dma_b128(v_rsrc, lds_tiles + buf_off + TILE_R + 1024, v_voff + (t * v_tile_stride + v_pc_stride));
+	};
 	auto load_tile = [&](int t, int buf_off) {
-		if(!loader) return;
-		lds_dma_b128(k_rsrc, lds_tiles + buf_off, k_voff + t * k_tile_stride);
-		lds_dma_b128(k_rsrc, lds_tiles + buf_off + 1024, k_voff + (t * k_tile_stride + k_pc_stride));
-		lds_dma_b128(v_rsrc, lds_tiles + buf_off + TILE_R, v_voff + t * v_tile_stride);
-		lds_dma_b128(v_rsrc, lds_tiles + buf_off + TILE_R + 1024, v_voff + (t * v_tile_stride + v_pc_stride));
+		load_tile_piece(t, buf_off, ic<0>{}), load_tile_piece(t, buf_off, ic<1>{}), load_tile_piece(t, buf_off, ic<2>{}), load_tile_piece(t, buf_off, ic<3>{});
 	};
 	// bias fragment of key tile t: 4 KB of this (head, query block)'s slab of the workspace -> this wavefront's slot
 	const int     n_qblocks = (int)((L + 31) / 32);
@@ -225,11 +166,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	const u32x4   ws_rsrc   = raw_rsrc(SLOT ? static_cast<const unsigned char*>(p.workspace) + ((h * n_qblocks + qbc) * n_t_all) * 4096 : nullptr, SLOT ? (uint32_t)(n_t_all * 4096) : 0u);
 	const int      ws_voff  = lane * 16;
 	const uint32_t lds_slot = lds_addr_of(smem) + SLOT_BASE + wave * 4096;
-	auto load_bias = [&](int t) {
-		if(!SLOT) return;
-#pragma unroll
-		for(int ld = 0; ld < 4; ld++) lds_dma_b128(ws_rsrc, lds_slot + ld * 1024, ws_voff + (t * 4096 + ld * 1024));  // (past the last tile: nothing is fetched)
+	auto load_bias_piece = [&](int t, auto pc_c) {
+		constexpr int PC = decltype(pc_c)::value;
+		if(!SLOT || t >= n_t) return;
+		lds_dma_b128(ws_rsrc, lds_slot + PC * 1024, ws_voff + (t * 4096 + PC * 1024));
 	};
+	auto load_bias = [&](int t) { load_bias_piece(t, ic<0>{}), load_bias_piece(t, ic<1>{}), load_bias_piece(t, ic<2>{}), load_bias_piece(t, ic<3>{}); };
 	// direct mode: this lane's four 8-byte pieces of a tile's bias, bias[h][q][32 t + 8 ld + 4 half .. + 3] (bf16), through a
 	// range-checked buffer over the head's slab; pieces whose keys lie at or beyond L are sent out of range and read as zero
 	[[maybe_unused]] u32x2 braw[4] = {u32x2{0u, 0u}, u32x2{0u, 0u}, u32x2{0u, 0u}, u32x2{0u, 0u}};
@@ -238,13 +180,135 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 		DIRECT ? const_cast<uint16_t*>(static_cast<const uint16_t*>(p.bias)) + h * p.bias_stride[0] : nullptr, 0, DIRECT ? (int)(((L - 1) * p.bias_stride[1] + L) * 2) : 0, 0x00020000);
 	const int bd_voff = (int)((qrow_b * p.bias_stride[1] + 4 * half) * 2);
 	auto load_bias_direct = [&](int t) {
-		if(!DIRECT) return;
+		if(!DIRECT || t >= n_t) return;
 #pragma unroll
 		for(int ld = 0; ld < 4; ld++) {
 			const bool in = t * KT_R + 8 * ld + 4 * half < L;
 			braw[ld] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(bd_rsrc, in ? bd_voff + ld * 16 : 0x40000000, t * (KT_R * 2), 0));
 		}
 	};
+
+	// ---- everything the walk needs before its first step is requested here in one go, so that the workgroup pays one
+	// memory latency, not a chain of them: the first K and V tiles and the first bias fragment (straight into LDS), the raw
+	// q rows, and the key-mask bytes ----
+	load_tile(0, 0);
+	load_bias(0);
+	load_bias_direct(0);
+	u32x4 qraw[ROWS][2];
+#pragma unroll
+	for(int r = 0; r < ROWS; r++) {
+		const int64_t   br = b0 + r < b_end ? b0 + r : b_end - 1;
+		const uint16_t* qp = static_cast<const uint16_t*>(p.q) + br * p.q_stride[0] + h * p.q_stride[1] + qrow * p.q_stride[2];
+#pragma unroll
+		for(int c = 0; c < 2; c++) {
+			const int d0 = 16 * c + 8 * half;
+			qraw[r][c]   = u32x4{0u, 0u, 0u, 0u};
+			if(row_ok && d0 < D) qraw[r][c] = *reinterpret_cast<const u32x4*>(qp + d0);
+		}
+	}
+
+	// ---- key-mask table: entry = additive mask value of (tile, batch row, key) as bf16 bits; wavefront w fills row w.
+	// With 4-byte aligned mask rows a lane takes four keys per load and all loads of the row are in flight together. ----
+	const int n_keys_tab = (n_t_all + 1) * KT_R;
+	if(wave < ROWS) {
+		const int      r    = wave;
+		const int64_t  br   = b0 + r < b_end ? b0 + r : b_end - 1;
+		const uint8_t* keep = p.key_mask ? p.key_mask + br * p.key_mask_stride_b : nullptr;
+		int            last = 0;
+		const bool     vec  = !keep || (((reinterpret_cast<uintptr_t>(p.key_mask) | (uintptr_t)p.key_mask_stride_b | (uintptr_t)L) & 3) == 0);
+		if(vec) {
+			constexpr int MAXC = MAX_L_ROWS / 256 + 1;   // chunks of 256 keys (4 per lane) that cover the table
+			uint32_t      mraw[MAXC];
+#pragma unroll
+			for(int c = 0; c < MAXC; c++) {
+				const int key0 = 256 * c + 4 * lane;
+				mraw[c]        = 0u;
+				if(256 * c < L) mraw[c] = !keep ? 0x01010101u : (key0 < L ? *reinterpret_cast<const uint32_t*>(keep + key0) : 0u);
+			}
+			auto write_chunks = [&](bool all_live) {
+#pragma unroll
+				for(int c = 0; c < MAXC; c++) {
+					const int key0 = 256 * c + 4 * lane;
+					if(256 * c >= n_keys_tab) break;
+					uint32_t e[4];
+#pragma unroll
+					for(int j = 0; j < 4; j++) {
+						const bool in   = key0 + j < L;
+						const bool live = in && (all_live || ((mraw[c] >> (8 * j)) & 0xffu) != 0);
+						e[j]            = live ? 0u : (in ? (uint32_t)MASK_DROPPED_BF16 : (uint32_t)MASK_OUT_OF_RANGE_BF16);
+						if(live && !all_live) last = key0 + j + 1;
+					}
+					if(key0 < n_keys_tab) *reinterpret_cast<u32x2*>(mask_tab + ((key0 >> 5) * ROWS + r) * 32 + (key0 & 31)) = u32x2{e[0] | (e[1] << 16), e[2] | (e[3] << 16)};
+				}
+			};
+			write_chunks(false);
+#pragma unroll
+			for(int off = 32; off >= 1; off >>= 1) {
+				const int o = __shfl_xor(last, off);
+				last        = o > last ? o : last;
+			}
+			// A batch row without any live key yields the mean over all L keys (masked_fill(-1e9) + softmax in
+			// examples/dot_product_attention.py:37-39): its keys count as live, and q and the bias are dropped for it
+			// below, so that all its logits are exactly equal.
+			if(last == 0) {
+				write_chunks(true);
+				last = 0;
+			}
+		} else {
+			for(int base = 0; base < n_keys_tab; base += 64) {
+				const int  key  = base + lane;
+				const bool in   = key < L;
+				const bool live = in && keep[in ? key : 0] != 0;
+				if(key < n_keys_tab) mask_tab[((key >> 5) * ROWS + r) * 32 + (key & 31)] = live ? (uint16_t)0 : (in ? MASK_DROPPED_BF16 : MASK_OUT_OF_RANGE_BF16);
+				const unsigned long long bal = __ballot(live);
+				if(bal) last = base + 64 - __builtin_clzll(bal);
+			}
+			if(last == 0)   // (as above)
+				for(int key = lane; key < n_keys_tab; key += 64) mask_tab[((key >> 5) * ROWS + r) * 32 + (key & 31)] = key < L ? (uint16_t)0 : MASK_OUT_OF_RANGE_BF16;
+		}
+		if(lane == 0) s_last[r] = last;
+	}
+	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's pieces of the first tile and its bias fragment have landed
+	__syncthreads();                                    // the mask table and the first tile are complete
+	// keys behind the last live key of every row carry weight 0 and are not walked; a row without live keys needs them all
+	int  l_eff = 0;
+	bool dropped[ROWS];
+#pragma unroll
+	for(int r = 0; r < ROWS; r++) {
+		const int last = __builtin_amdgcn_readfirstlane(s_last[r]);
+		dropped[r]     = last == 0;
+		const int need = dropped[r] ? (int)L : last;
+		l_eff          = need > l_eff ? need : l_eff;
+	}
+	n_t = (l_eff + KT_R - 1) / KT_R;
+
+	// Q fragments (B operand of S^T = K.Q^T): lane (q = n, g = half) holds q[q][16c + 8g .. +7], scaled by
+	// softmax_scale * log2 e in fp32 and rounded once to bf16 (the reference rounds the scaled q too,
+	// src/csrc/dot_product_attention.cpp:95-98).  A batch row without live keys gets q = 0.
+	bf16x8 qf[ROWS][2];
+#pragma unroll
+	for(int r = 0; r < ROWS; r++) {
+		const float qmul = dropped[r] ? 0.f : p.softmax_scale * LOG2E;
+#pragma unroll
+		for(int c = 0; c < 2; c++) {
+			u32x4 sc4;
+#pragma unroll
+			for(int j = 0; j < 4; j++) {
+				const uint32_t w = qraw[r][c][j];
+				sc4[j] = pack_bf16x2(bf16_bits_to_f32(w & 0xffffu) * qmul, bf16_bits_to_f32(w >> 16) * qmul);
+			}
+			qf[r][c] = __builtin_bit_cast(bf16x8, sc4);
+		}
+	}
+	// Operands of the mask MFMA (v_mfma_f32_32x32x8_bf16: four contraction slots per half-wave, two registers per operand).
+	// A (per key): slot 0 = the key's mask value (from the table, zero-extended), slots 2 and 3 = 1.0.
+	// B (per query): slot 0 = 1.0, slots 2 and 3 = -m_hi and -m_lo, the softmax reference of this lane's query row as two
+	// bf16 terms (16 significant bits).  Lanes of the upper half-wave supply slots 4..7: their B is zero, so whatever
+	// finite value their A holds contributes nothing.
+	u32x2 maskA = {0u, 0x3F803F80u};
+	u32x2 maskB[ROWS];
+#pragma unroll
+	for(int r = 0; r < ROWS; r++) maskB[r] = u32x2{half == 0 ? 0x3F80u : 0u, 0u};
 
 	// ---- per-lane LDS read offsets inside a (buffer, batch row) block ----
 	int k_rd[2];
@@ -365,10 +429,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	// so that no instruction waits for the one issued just before it, and leaves S^T(next) in `sc`, P^T in `pprev`, this
 	// step's V^T fragments in `vprev`, the K fragments of the step after the next in `kf`.
 	// k_addr2: LDS byte address of the K tile of the step after the next; m_addr: (per lane) of the next step's mask
-	// entries; v_addr: of this step's V tile; mid: hook run once the first K.Q^T instruction of the next step is issued.
+	// entries; v_addr: of this step's V tile; hook(i): run behind the i-th matrix instruction of the step (i = 0..4; 1 is the
+	// first K.Q^T instruction of the next step).
 	// FIRST: the very first tile, which fixes every row's softmax reference.  ANYDROP: some batch row of this group has no
 	// live key (it then takes no bias: a wave-uniform branch the common instantiation does not carry).
-	auto step = [&](auto r_c, auto first_c, auto anydrop_c, int k_addr2, int m_addr, int v_addr, auto&& mid) {
+	auto step = [&](auto r_c, auto first_c, auto anydrop_c, int k_addr2, int m_addr, int v_addr, auto&& hook) {
 		constexpr int  R = decltype(r_c)::value, RN = (R + 1) % ROWS, RP = (R + ROWS - 1) % ROWS;
 		constexpr bool FIRST = decltype(first_c)::value != 0, ANYDROP = decltype(anydrop_c)::value != 0;
 		if constexpr(FIRST) rereference(r_c, sc, true);
@@ -400,6 +465,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	__builtin_amdgcn_sched_barrier(0)
 		__builtin_amdgcn_sched_barrier(0);
 		oacc[RP] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[0]), __builtin_bit_cast(bf16x8, pprev[0]), oacc[RP], 0, 0, 0);
+		hook(ic<0>{});
 		exp_part(sc, pcur, ic<0>{}, ic<2>{});
 		AF3_PIN3(oacc[RP][0], pcur[0][0], kf[0][0]);
 		{
@@ -411,7 +477,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 			if(with_bias) sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[0]), qf[RN][0], bias_frag, 0, 0, 0);
 			else sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[0]), qf[RN][0], z, 0, 0, 0);
 		}
-		mid();
+		hook(ic<1>{});
 		exp_part(sc, pcur, ic<2>{}, ic<2>{});
 		AF3_PIN3(sn[0], pcur[0][1], pprev[1][0]);
 		oacc[RP] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vprev[1]), __builtin_bit_cast(bf16x8, pprev[1]), oacc[RP], 0, 0, 0);
@@ -424,15 +490,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 				const u32x2 r2 = __builtin_bit_cast(u32x2, rr);
 				vprev[cp][2 * t] = r2[0], vprev[cp][2 * t + 1] = r2[1];
 			}
+		hook(ic<2>{});
 		exp_part(sc, pcur, ic<4>{}, ic<2>{});
 		AF3_PIN3(oacc[RP][0], pcur[0][2], kf[1][0]);
 		sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[1]), qf[RN][1], sn, 0, 0, 0);
 		// K fragments of the step after the next, now that the next step's are consumed
 		kf[0] = read_kfrag(k_addr2 + k_rd[0]);
 		kf[1] = read_kfrag(k_addr2 + k_rd[1]);
+		hook(ic<3>{});
 		exp_part(sc, pcur, ic<6>{}, ic<2>{});
 		AF3_PIN2(sn[0], pcur[0][3]);
 		rs = rowsum(rs, pcur[0]);
+		hook(ic<4>{});
 		exp_part(sc, pcur, ic<8>{}, ic<4>{});
 		AF3_PIN3(rs[0], pcur[1][0], pcur[1][1]);
 		{
@@ -477,15 +546,21 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 				const int     vc = buf + R * (2 * TILE_R);
 				if constexpr(R == ROWS - 2) {
 					asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-					step(r_c, first_c, anydrop_c, k2, m1, vc, [&] {
-						load_tile(t + 2, bufnn);  // (past the end of the rows: nothing is fetched)
-						next_bias_fragment();
-						load_bias_direct(t + 2);
+					step(r_c, first_c, anydrop_c, k2, m1, vc, [&](auto s_c) {
+						constexpr int S = decltype(s_c)::value;
+						if constexpr(S == 1) {
+							load_tile(t + 2, bufnn);
+							next_bias_fragment();
+							load_bias_direct(t + 2);
+						}
 					});
 				} else if constexpr(R == ROWS - 1) {
-					step(r_c, first_c, anydrop_c, k2, m1, vc, [&] { load_bias(t + 2); });
+					step(r_c, first_c, anydrop_c, k2, m1, vc, [&](auto s_c) {
+						constexpr int S = decltype(s_c)::value;
+						if constexpr(S == 1) load_bias(t + 2);   // (behind this step's first K.Q^T instruction, which has waited for the slot's reads)
+					});
 				} else {
-					step(r_c, first_c, anydrop_c, k2, m1, vc, [] {});
+					step(r_c, first_c, anydrop_c, k2, m1, vc, [](auto) {});
 				}
 			}
 		};
@@ -493,17 +568,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	};
 	auto run = [&](auto anydrop_c) {
 		constexpr bool ANYDROP = decltype(anydrop_c)::value != 0;
-		// ---- prologue: the first two tiles, the first two bias fragments, S^T of the first step, K fragments of the second ----
-		load_tile(0, 0);
-		load_bias(0);
-		load_bias_direct(0);
-		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+		// ---- prologue: the second tile and bias fragment, S^T of the first step, K fragments of the second ----
+		// (tile 0 and bias fragment 0 were requested at the top of the kernel and are complete)
 		next_bias_fragment();  // fragment 0 -> registers
 		asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 		load_tile(1, BUF_R);
 		load_bias(1);
 		load_bias_direct(1);
-		__syncthreads();   // tile 0 is complete (every wavefront has waited for its own pieces)
 		{
 			f32x16 s0;
 #pragma unroll

@@ -176,7 +176,7 @@ def set_rows_kernel(mode: str) -> str:
 def set_exact_bias(flag: bool) -> bool:
     """With True, batched bf16 calls read the bias in place and add it exactly instead of going
     through the kernel's fp16 log2-domain bias workspace (whose rounding error in a logit is at most
-    2^-12 * |bias| * log2 e: irrelevant for pair biases of ordinary size, 2 % of a softmax weight
+    2^-11 * |bias| * log2 e: irrelevant for pair biases of ordinary size, 2 % of a softmax weight
     at |bias| = 40).  Slower for B >= 2.  Returns the previous setting."""
     global _exact_bias
     prev, _exact_bias = _exact_bias, bool(flag)

@@ -108,7 +108,7 @@ typedef struct af3_dpa_params {
 	 * out in matrix-operand order, shared by all B batch rows) and then runs its fastest variant;
 	 * without it (NULL) the bias is read in place.  Contents are overwritten by every call.
 	 * Precision: the rewritten bias is fp16(bias * log2 e), i.e. each logit carries a rounding
-	 * error of at most 2^-12 * |bias| * 1.4427 (0.4 % of a softmax weight at |bias| = 8, 2 % at
+	 * error of at most 2^-11 * |bias| * 1.4427 (0.4 % of a softmax weight at |bias| = 8, 2 % at
 	 * |bias| = 40; values beyond +-45400 saturate).  Callers whose biases are that large and who
 	 * need them exact pass workspace = NULL: the in-place variant adds the bf16 bias exactly. */
 	void*          workspace;

@@ -187,10 +187,28 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	const int64_t L = p.L;
 	const int     D = (int)p.D;
 
-	// ---- zero the K/V buffers: lanes of padded head columns never write them, and whatever a
-	// bounds-checked load leaves behind for rows past L must be finite (0 * stale NaN = NaN) ----
-	if(!FUSED && (D != DP || L % KT != 0))
-		for(int i = tid; i < (LDS_SETS * 6 * TILE_BYTES + RING_BYTES) / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
+	// ---- key-mask bytes: requested first, so that their latency covers the zeroing below.  With 4-byte aligned mask rows
+	// a lane takes four keys per load (a chunk of 256 keys = four tiles per wavefront and load) and all of a wavefront's
+	// loads -- up to eight per pass -- are in flight together: one memory latency, not one per tile (a single row's walk
+	// is short enough for that to show). ----
+	const uint8_t* keep     = p.key_mask ? p.key_mask + b * p.key_mask_stride_b : nullptr;
+	const bool     mask_vec = !keep || (((reinterpret_cast<uintptr_t>(p.key_mask) | (uintptr_t)p.key_mask_stride_b | (uintptr_t)L) & 3) == 0);
+	const int      n_chunks = (n_ktiles * KT + 255) / 256;
+	uint32_t       mraw[8];
+	auto request_mask = [&](int c0) {
+#pragma unroll
+		for(int i = 0; i < 8; i++) {
+			const int64_t key0 = (int64_t)(c0 + i * NW) * 256 + 4 * lane;
+			mraw[i]            = 0u;
+			if(c0 + i * NW < n_chunks) mraw[i] = !keep ? 0x01010101u : (key0 < L ? *reinterpret_cast<const uint32_t*>(keep + key0) : 0u);
+		}
+	};
+	if(mask_vec) request_mask(wave);
+
+	// (The K/V buffers and the bias ring are not cleared: every load of a tile writes every byte of its buffer with finite
+	// data -- lanes of padded head columns fetch the row's first chunk again (q is zero there), rows and keys past L fetch the
+	// last row / the row's last chunk again (their logits get the out-of-range mask value) -- so no stale LDS content is
+	// ever read.  Clearing 72 KB with 128 threads cost a single-row call 3600 of its 24000 clocks.)
 	// ---- key-mask table and list of tiles with at least one live key ----
 	// entry = bf16 additive mask value in the low half (contraction slot 0) and, in the log2
 	// variant, 1.0 in the high half (slot 1, multiplies -m_ref); the last 64 entries are zero
@@ -198,17 +216,44 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	if(tid == 0) s_nvalid = 0;
 	if(tid < 64) mask_tab[n_ktiles * KT + tid] = 0u;
 	__syncthreads();
-	const uint8_t* keep = p.key_mask ? p.key_mask + b * p.key_mask_stride_b : nullptr;
-	for(int kt = wave; kt < n_ktiles; kt += NW) {
-		const int64_t  key  = (int64_t)kt * KT + lane;
-		const bool     in   = key < L;
-		const bool     live = in && (keep ? keep[key] != 0 : true);
-		const uint32_t mv   = live ? 0u : (in ? (uint32_t)MASK_DROPPED_BF16 : (uint32_t)MASK_OUT_OF_RANGE_BF16);
-		mask_tab[kt * KT + lane] = mv | (L2DOM ? 0x3F800000u : 0u);
-		const unsigned long long bal = __ballot(live);
-		if(lane == 0) {
-			live_list[kt] = bal ? 1 : 0;
-			if(bal) atomicAdd(&s_nvalid, 1);
+	if(mask_vec) {
+		for(int c0 = wave; c0 < n_chunks; c0 += 8 * NW) {
+			if(c0 != wave) request_mask(c0);
+#pragma unroll
+			for(int i = 0; i < 8; i++) {
+				const int c = c0 + i * NW;
+				if(c >= n_chunks) break;
+				const int64_t key0 = (int64_t)c * 256 + 4 * lane;
+				u32x4         e;
+				bool          any = false;
+#pragma unroll
+				for(int j = 0; j < 4; j++) {
+					const bool in   = key0 + j < L;
+					const bool live = in && ((mraw[i] >> (8 * j)) & 0xffu) != 0;
+					any             = any || live;
+					e[j]            = (live ? 0u : (in ? (uint32_t)MASK_DROPPED_BF16 : (uint32_t)MASK_OUT_OF_RANGE_BF16)) | (L2DOM ? 0x3F800000u : 0u);
+				}
+				if(key0 < (int64_t)n_ktiles * KT) *reinterpret_cast<u32x4*>(mask_tab + key0) = e;
+				const unsigned long long bal = __ballot(any);   // 16 lanes per tile
+				if(lane < 4 && 4 * c + lane < n_ktiles) {
+					const bool tile_live = ((bal >> (16 * lane)) & 0xffffull) != 0;
+					live_list[4 * c + lane] = tile_live ? 1 : 0;
+					if(tile_live) atomicAdd(&s_nvalid, 1);
+				}
+			}
+		}
+	} else {
+		for(int kt = wave; kt < n_ktiles; kt += NW) {
+			const int64_t  key  = (int64_t)kt * KT + lane;
+			const bool     in   = key < L;
+			const bool     live = in && keep[in ? key : 0] != 0;
+			const uint32_t mv   = live ? 0u : (in ? (uint32_t)MASK_DROPPED_BF16 : (uint32_t)MASK_OUT_OF_RANGE_BF16);
+			mask_tab[kt * KT + lane] = mv | (L2DOM ? 0x3F800000u : 0u);
+			const unsigned long long bal = __ballot(live);
+			if(lane == 0) {
+				live_list[kt] = bal ? 1 : 0;
+				if(bal) atomicAdd(&s_nvalid, 1);
+			}
 		}
 	}
 	__syncthreads();
@@ -435,17 +480,27 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		// ---- K/V tile loader: buffer loads that write LDS directly ----
 		// One wave load moves 1 KB: lane i -> LDS chunk i of the load's 1 KB window, i.e. tile row
 		// j*RPI + i/CPR, physical chunk i%CPR.  The lane picks the global chunk that belongs there
-		// under the swizzle; lanes of padded head columns (chunk*8 >= D) stay idle.
+		// under the swizzle; lanes of padded head columns (chunk*8 >= D) fetch the row's first chunk.
 		const u32x4 k_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1], (uint32_t)(((L - 1) * p.k_stride[2] + D) * 2));
 		const u32x4 v_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.v) + b * p.v_stride[0] + h * p.v_stride[1], (uint32_t)(((L - 1) * p.v_stride[2] + D) * 2));
 		const int  ld_row  = lane / CPR, ld_pc = lane % CPR;
 		const int  k_chunk = ld_pc ^ k_swizzle<DP>(ld_row);
 		const int  v_chunk = ld_pc ^ v_swizzle<DP>(ld_row);
-		const int  k_voff  = (int)(ld_row * p.k_stride[2] * 2) + k_chunk * 16;
-		const int  v_voff  = (int)(ld_row * p.v_stride[2] * 2) + v_chunk * 16;
-		const bool k_act   = k_chunk * 8 < D, v_act = v_chunk * 8 < D;
+		const int  k_voff  = (int)(ld_row * p.k_stride[2] * 2) + (k_chunk * 8 < D ? k_chunk * 16 : 0);   // (padded head columns: the first chunk again)
+		const int  v_voff  = (int)(ld_row * p.v_stride[2] * 2) + (v_chunk * 8 < D ? v_chunk * 16 : 0);
+		const int  k_row_bytes = (int)(p.k_stride[2] * 2), v_row_bytes = (int)(p.v_stride[2] * 2);
 		const int  k_tile_stride = (int)(KT * p.k_stride[2] * 2), v_tile_stride = (int)(KT * p.v_stride[2] * 2);
 		const int  k_ld_stride   = (int)(RPI * p.k_stride[2] * 2), v_ld_stride = (int)(RPI * p.v_stride[2] * 2);
+		// byte offsets of piece j of tile kt for this lane; a piece that reaches past the last key (rare, wave-uniform test)
+		// sends the lanes of rows >= L to row L - 1
+		auto kv_offsets = [&](int kt, int j, int& ko, int& vo) {
+			ko = k_voff + (kt * k_tile_stride + j * k_ld_stride), vo = v_voff + (kt * v_tile_stride + j * v_ld_stride);
+			const int row0 = kt * KT + j * RPI;
+			if(row0 + RPI > (int)L) {
+				const int over = row0 + lane / CPR - ((int)L - 1);
+				if(over > 0) ko -= over * k_row_bytes, vo -= over * v_row_bytes;
+			}
+		};
 		const uint32_t k_lds_addr = lds_addr_of(k_lds), v_lds_addr = lds_addr_of(v_lds);
 		auto load_tile = [&](int kt, int buf) {
 			if(FUSED) return;  // K and V of every tile are already in LDS
@@ -453,19 +508,20 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 #pragma unroll
 				for(int t = 0; t < 2 * NI / NW; t++) {
 					const int pc = wave + NW * t;  // (wave-uniform)
-					if(pc < NI) {
-						if(k_act) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + pc * 1024, k_voff + (kt * k_tile_stride + pc * k_ld_stride));
-					} else {
-						if(v_act) lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + (pc - NI) * 1024, v_voff + (kt * v_tile_stride + (pc - NI) * v_ld_stride));
-					}
+					int       ko, vo;
+					kv_offsets(kt, pc < NI ? pc : pc - NI, ko, vo);
+					if(pc < NI) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + pc * 1024, ko);
+					else lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + (pc - NI) * 1024, vo);
 				}
 				return;
 			}
 #pragma unroll
 			for(int t = 0; t < (SPLIT ? NI : NI / NW); t++) {
 				const int j = SPLIT ? t : wave + NW * t;  // split: this wavefront fetches whole tiles into its private buffers
-				if(k_act) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + j * 1024, k_voff + (kt * k_tile_stride + j * k_ld_stride));
-				if(v_act) lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + j * 1024, v_voff + (kt * v_tile_stride + j * v_ld_stride));
+				int ko, vo;
+				kv_offsets(kt, j, ko, vo);
+				lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + j * 1024, ko);
+				lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + j * 1024, vo);
 			}
 		};
 
@@ -473,9 +529,9 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		// HBM -> LDS by four LDS-direct loads of whole 128-byte row segments (eight lanes per row), two
 		// tiles ahead of its use and without occupying registers.  Slot layout: [row 32][128 B], the
 		// 16-byte chunk c of row r stored at chunk position c ^ (r & 7) so that the fragment reads (one
-		// chunk per lane, 32 rows at once) spread over the banks.  Rows past L lie beyond the buffer's
-		// range; chunks of keys past L (last tile) are sent there too, so padding behind a row's L valid
-		// entries is never read.  Whatever such lanes leave in LDS is finite: the ring starts zeroed.
+		// chunk per lane, 32 rows at once) spread over the banks.  Rows past L fetch row L - 1 and chunks of
+		// keys past L (last tile) the row's last valid chunk, so padding behind a row's L valid entries is
+		// never read and every byte of a slot is written with finite data by every load.
 		const u32x4    b_rsrc    = raw_rsrc(BRING ? static_cast<const uint16_t*>(p.bias) + h * p.bias_stride[0] : nullptr,
 											BRING ? (uint32_t)(((L - 1) * p.bias_stride[1] + L) * 2) : 0u);
 		unsigned char* const bring = smem + LDS_SETS * 6 * TILE_BYTES + (BRING ? (KS2 ? wblk : wave) * 3 * 4096 : 0);
@@ -486,9 +542,17 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		const int      b_key      = ((lane & 7) ^ (lane >> 3)) * 8;  // first key of this lane's chunk within a tile
 		auto load_bias_tile = [&](int kt, int slot_i) {
 			if(!BRING || (KS2 && sub != 0)) return;  // (KS2: the pair's first wavefront fetches the whole 32 x 64 tile for both)
-			const int in_row = kt * KT + b_key < (int)L ? b_voff + kt * (KT * 2) : 0x7FFF0000;
+			const int in_row   = kt * KT + b_key < (int)L ? b_voff + kt * (KT * 2) : b_voff - b_key * 2 + ((int)L - 8) * 2;
+			const int blk_row0 = (int)(qtile * QT + wblk * 32);
 #pragma unroll
-			for(int j = 0; j < 4; j++) lds_dma_b128(b_rsrc, bring_addr + slot_i * 4096 + j * 1024, in_row + (b_row0 + j * b_row8));
+			for(int j = 0; j < 4; j++) {
+				int off = in_row + (b_row0 + j * b_row8);
+				if(blk_row0 + 32 > (int)L) {   // (rare, wave-uniform: the matrix' last query block)
+					const int over = blk_row0 + 8 * j + (lane >> 3) - ((int)L - 1);
+					if(over > 0) off -= over * (int)(p.bias_stride[1] * 2);
+				}
+				lds_dma_b128(b_rsrc, bring_addr + slot_i * 4096 + j * 1024, off);
+			}
 		};
 		// fragment read: lane (n, half) takes chunk 4*sub + 2*c2 + half of row n
 		const int b_rd = (n * 128 + (((n & 7) ^ half) << 4)) ^ (sub << 6);  // (KS2: chunks 4..7 of a row hold keys 32..63)

@@ -446,6 +446,28 @@ def test_named_configs_full_size(af3, oracle, name, sample_rows):
 # ---- the kernel for batches that share a bias (four batch rows per wavefront) -----------------------------------------
 # Large launches take it by themselves (the named configs above do); here it is forced on small and awkward shapes.
 
+@pytest.mark.parametrize("B,H,L,D,rows", [(1, 2, 192, 24, "never"), (3, 2, 64, 32, "never"), (5, 2, 192, 32, "always"), (17, 1, 64, 32, "always")])
+def test_key_mask_rows_that_are_not_4_byte_aligned(af3, oracle, B, H, L, D, rows):
+    """The kernels read 4-byte aligned mask rows four keys per load and anything else byte by byte: a mask that is a view
+    into a wider tensor (odd storage offset, odd row stride) must give what its contiguous copy gives."""
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=L + B, mask="random")
+    wide = torch.zeros(B, L + 7, dtype=torch.bool)
+    wide[:, 3:3 + L] = m
+    dq, dk, dv, db, dwide = dev(q, k, v, bias, wide)
+    view = dwide[:, 3:3 + L]
+    assert view.data_ptr() % 4 != 0 and view.stride(0) % 4 != 0
+    prev = af3.set_rows_kernel(rows)
+    try:
+        got_view = af3.dot_product_attention_cpp(dq, dk, dv, view, db)
+        got_copy = af3.dot_product_attention_cpp(dq, dk, dv, view.contiguous(), db)
+    finally:
+        af3.set_rows_kernel(prev)
+    torch.cuda.synchronize()
+    assert torch.equal(got_view, got_copy)
+    want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), f32np(bias))
+    assert float(np.abs(f32np(got_view) - want).max()) <= TOL[torch.bfloat16]
+
+
 @pytest.fixture
 def rows_kernel(af3):
     prev = af3.set_rows_kernel("always")

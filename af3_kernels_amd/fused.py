@@ -269,10 +269,22 @@ def self_attention_cpp(
     """Diffusion-transformer self-attention on one token sequence:
         q = x . Wq + q_bias;  k, v, g = x . Wk, Wv, Wg;  out = softmax(q k^T K^-1/2 + bias, mask) v * sigmoid(g)
     pair (x) [N, C]; mask [N]; bias [head, N, N]; q_bias [C] (or [head, C/head]); weights as in
-    _attention_cpp.  Returns [N, C]."""
+    _attention_cpp.  Returns [N, C].
+
+    Beyond the reference (which takes one sequence per call, src/csrc/dot_product_attention.cpp:380-543): pair may be
+    [S, N, C] -- S diffusion samples of the same tokens, mask [N] or [S, N] -- and the S samples then go through ONE
+    projection GEMM and ONE attention launch in which they share every bias tile (the pair bias, the largest operand,
+    is streamed once instead of S times).  Returns [S, N, C]."""
     ops._require_device(pair, mask, bias, q_proj, q_bias, k_proj, v_proj, gating_query)
+    if pair.dim() == 3:
+        S, N, C = pair.shape
+        _check_weights(C, head, (q_proj, k_proj, v_proj, gating_query))
+        if ops._DTYPE_CODE.get(pair.dtype) not in (ops.AF3_F32, ops.AF3_BF16):
+            raise ValueError(f"unsupported dtype {pair.dtype}: float32 or bfloat16")
+        y = _project(pair.reshape(S * N, C), (q_proj, k_proj, v_proj, gating_query), q_bias, head)
+        return _attend(y, S, N, head, mask, bias)
     if pair.dim() != 2:
-        raise ValueError(f"pair must be [N, C], got {tuple(pair.shape)}")
+        raise ValueError(f"pair must be [N, C] or [S, N, C], got {tuple(pair.shape)}")
     N, C = pair.shape
     _check_weights(C, head, (q_proj, k_proj, v_proj, gating_query))
     dtype = pair.dtype

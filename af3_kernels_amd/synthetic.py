@@ -138,6 +138,8 @@ FUSED_CASES = {
     # so this one runs as projection GEMM + attention kernel + output GEMM
     "grid_n1536": FusedCase("grid_n1536", "grid", 1536, 1536, 128, 4),
     "self_n1536": FusedCase("self_n1536", "self", 1, 1536, 768, 16),
+    # five diffusion samples of the same tokens in one call (16 heads of 24 channels: the shape of cfg5, in bf16): the samples share every bias tile
+    "self5_n1536": FusedCase("self5_n1536", "self", 5, 1536, 384, 16),
 }
 
 
@@ -166,6 +168,6 @@ def make_fused_inputs(case, device="cpu", batch=None):
     else:
         mask = torch.rand(case.N, generator=mgen) < case.keep
         mask[0] = True
-        x = draw(case.N, case.C).to(dt).to(device)
+        x = (draw(case.N, case.C) if case.B == 1 else torch.stack([draw(case.N, case.C) for _ in range(B)])).to(dt).to(device)
     return dict(x=x, mask=mask.to(device), bias=bias, wq=ws[0], wk=ws[1], wv=ws[2], wg=ws[3], wo=ws[4] if case.kind == "grid" else None,
                 q_bias=q_bias if case.kind == "self" else None)

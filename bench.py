@@ -128,7 +128,7 @@ def cpu_baseline(case, budget_s=12.0):
 
 
 def bench_fused(args, case):
-    """--case grid_n384 | grid_n768 | self_n1536: a step is one call of _attention_cpp / self_attention_cpp (the drop-ins
+    """--case grid_n384 | grid_n768 | grid_n1536 | self_n1536 | self5_n1536: a step is one call of _attention_cpp / self_attention_cpp (the drop-ins
     for the reference's fused callers of the attention core) on synthetic rows already resident in HBM."""
     import torch
     import af3_kernels_amd as af3
@@ -188,8 +188,10 @@ def bench_fused(args, case):
         else:
             ach = case.flops_attention / (kernel_ms * 1e-3) / 1e12
             roofline = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS["bf16"], 4),
-                        "traffic": None, "kernel": "attention kernel with the gate in its epilogue (+ bias prepass; of projection GEMM + attention + output GEMM)",
+                        "traffic": None, "kernel": "attention kernel with the gate in its epilogue (+ bias prepass; of projection GEMM + attention" + (" + output GEMM)" if case.kind == "grid" else ")"),
                         "algorithmic_flops_per_launch": case.flops_attention, **timing}
+            if case.kind == "self":   # several samples of one sequence: the [head, N, N] bias is streamed once for all of them
+                roofline["bias_stream_GBps"] = round(case.head * case.N * case.N * 2 / (kernel_ms * 1e-3) / 1e9, 1)
     tflops = case.flops / (ms_per_step * 1e-3) / 1e12
     line = {"metric": f"fused {case.kind} self-attention TFLOP/s ({case.name})", "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",

@@ -192,6 +192,35 @@ def test_self_attention_cpp_matches_formula(af3, oracle, N, C, head, dtype):
     check(out, want, ref, dtype)
 
 
+@pytest.mark.parametrize("S,N,C,head", [(5, 200, 384, 16), (5, 192, 768, 16), (3, 77, 128, 4), (2, 64, 256, 8)])
+def test_self_attention_cpp_takes_several_samples_that_share_the_bias(af3, oracle, S, N, C, head):
+    """[S, N, C] input: one projection and one attention launch for all samples (heads of up to 32 channels: the shared-bias
+    kernel; wider heads: the one-row kernel over a shared bias workspace); every sample must come out as from its own call."""
+    x, mask, bias, wq, wk, wv, wg, _, qb = make(None, N, C, head, torch.bfloat16, seed=S * N + C, with_out=False, with_qbias=True)
+    g = torch.Generator().manual_seed(S + N)
+    xs = torch.stack([x] + [torch.randn(N, C, generator=g).to(torch.bfloat16) for _ in range(S - 1)])
+    masks = torch.stack([mask] + [(torch.rand(N, generator=g) < 0.8) for _ in range(S - 1)])
+    masks[:, 0] = True
+    d = lambda t: t.cuda()
+    packed = [pack(af3, d(w), head) for w in (wq, wk, wv, wg)]
+    print(f"self_attention_cpp S,N,C,head={S, N, C, head}", flush=True)
+    out = af3.self_attention_cpp(d(xs), d(masks), d(bias), packed[0], d(qb), packed[1], packed[2], packed[3], head)
+    torch.cuda.synchronize()
+    assert out.shape == xs.shape and out.dtype == torch.bfloat16
+    for s_i in range(S):
+        one = af3.self_attention_cpp(d(xs[s_i]), d(masks[s_i]), d(bias), packed[0], d(qb), packed[1], packed[2], packed[3], head)
+        assert float((out[s_i].float() - one.float()).abs().max()) <= 2e-2
+    for s_i in (0, S - 1):
+        args = [f32np(xs[s_i]), masks[s_i].numpy(), f32np(bias), f32np(wq), f32np(wk), f32np(wv), f32np(wg), None, f32np(qb)]
+        want = oracle.fused_attention_formula(*args, head=head)
+        ref = oracle.fused_attention_reference(*args, head=head, dtype=oracle.BF16, BLK_SZ=64)
+        check(out[s_i], want, ref, torch.bfloat16)
+    # one mask for all samples
+    out1 = af3.self_attention_cpp(d(xs), d(masks[0]), d(bias), packed[0], d(qb), packed[1], packed[2], packed[3], head)
+    one = af3.self_attention_cpp(d(xs[1]), d(masks[0]), d(bias), packed[0], d(qb), packed[1], packed[2], packed[3], head)
+    assert float((out1[1].float() - one.float()).abs().max()) <= 2e-2
+
+
 def _self_sweep(n, seed):
     """Seeded (N, C, head) for the diffusion op: head widths 16..64 (padded to 32 or 64 in the kernel), sequence lengths on
     both sides of the 32- and 64-key boundaries and long enough for every key-split variant."""
@@ -252,7 +281,7 @@ def test_attention_cpp_rejects_malformed_calls(af3):
     with pytest.raises(RuntimeError):
         af3._attention_cpp(x.cpu(), mask, bias, w, w, w, w, w, head)           # no CPU path
     with pytest.raises(ValueError):
-        af3.self_attention_cpp(x, mask[0], bias, w, None, w, w, w, head)       # the diffusion op takes [N, C]
+        af3.self_attention_cpp(x[None], mask[0], bias, w, None, w, w, w, head)  # the diffusion op takes [N, C] or [S, N, C]
 
 
 @pytest.mark.parametrize("transpose", [False, True])

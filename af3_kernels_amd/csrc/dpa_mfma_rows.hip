@@ -728,7 +728,10 @@ int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
 	// remainder of one borrows from the last full group); every group of one launch has the same number of rows.  Four
 	// rows share a bias tile best, but what counts is how evenly the workgroups fill the GPU's 512 slots (two per
 	// compute unit): the launch time is about (rounds of 512 workgroups) x (rows per group) x (cost per row, which grows
-	// as fewer rows share a tile: measured 1 : 1.075 : 1.09 for 4 : 3 : 2 rows), and the cheapest plan is taken.
+	// as fewer rows share a tile: measured 1 : 1.075 : 1.09 for 4 : 3 : 2 rows), and the cheapest plan is taken.  For a
+	// small batch the cheapest plan is often ONE launch whose last group is short (its missing rows repeat the last batch
+	// row and are not stored): launches run one after the other, so 3 + 2 rows in two launches of half-empty rounds take
+	// the time of five rows, the same five rows as 3 + (2 and a repeated one) in one launch the time of three.
 	const int64_t B = p.B, per_row_wgs = p.H * ((p.L + 127) / 128);
 	auto plan = [&](int rows, int64_t (&count)[3], int (&rows_of)[3]) -> double {
 		static const double cost_per_row[5] = {0, 0, 1.09, 1.075, 1.0};
@@ -762,6 +765,16 @@ int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
 		if(t < best * 0.999) {
 			best = t;
 			for(int i = 0; i < 3; i++) count[i] = c[i], rows_of[i] = r[i];
+		}
+		if(B % rows != 0) {   // one launch, last group short
+			static const double cost_per_row[5] = {0, 0, 1.09, 1.075, 1.0};
+			const int64_t wgs = ((B + rows - 1) / rows) * per_row_wgs;
+			const double  t1  = (double)((wgs + 511) / 512) * rows * cost_per_row[rows];
+			if(t1 < best * 0.999) {
+				best = t1;
+				count[0] = B, rows_of[0] = rows;
+				count[1] = count[2] = 0, rows_of[1] = rows_of[2] = 0;
+			}
 		}
 	}
 	if(best >= 1e30) return AF3_ERR_BAD_SHAPE;  // (B == 1 is not eligible)

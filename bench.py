@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0
 #     kernel_sources_sha256: <digest of the kernel sources the run was made with>
 # and the figure is only reported while the sources still have that digest: after any kernel change it is null until
 # the counters are collected again.
-TRAFFIC_PROFILES = {"cfg4": "dpa_rows_bf16_cfg4_hbm_traffic.txt", "cfg2": "dpa_mfma_bf16_cfg2_hbm_traffic.txt", "cfg3": "dpa_mfma_bf16_cfg3_hbm_traffic.txt",
+TRAFFIC_PROFILES = {"cfg4": "dpa_rows_bf16_cfg4_hbm_traffic.txt", "cfg2": "dpa_rows_bf16_cfg2_hbm_traffic.txt", "cfg3": "dpa_mfma_bf16_cfg3_hbm_traffic.txt",
                     "cfg5": "dpa_mfma_fp8_cfg5_hbm_traffic.txt", "grid_n768": "grid_attention_one_kernel_grid_n768_hbm_traffic.txt"}
 KERNEL_SOURCES = ("common.hpp", "mfma_helpers.hpp", "dpa_mfma.hip", "dpa_mfma_rows.hip", "dpa_mfma_fp8.hip", "elementwise.hip")
 

@@ -187,7 +187,88 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	const int64_t L = p.L;
 	const int     D = (int)p.D;
 
-	// ---- key-mask bytes: requested first, so that their latency covers the zeroing below.  With 4-byte aligned mask rows
+	const int sub  = KS2 ? (wave & 1) : 0;                  // KS2: which 32 keys of every 64-key tile this wavefront takes
+	const int wblk = SPLIT ? 0 : KS2 ? (wave >> 1) : wave;  // this wavefront's block of 32 query rows within the workgroup's QT rows
+
+	// ---- K/V tile loader: buffer loads that write LDS directly ----
+	// One wave load moves 1 KB: lane i -> LDS chunk i of the load's 1 KB window, i.e. tile row
+	// j*RPI + i/CPR, physical chunk i%CPR.  The lane picks the global chunk that belongs there
+	// under the swizzle; lanes of padded head columns (chunk*8 >= D) fetch the row's first chunk.
+	const u32x4 k_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1], (uint32_t)(((L - 1) * p.k_stride[2] + D) * 2));
+	const u32x4 v_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.v) + b * p.v_stride[0] + h * p.v_stride[1], (uint32_t)(((L - 1) * p.v_stride[2] + D) * 2));
+	const int  ld_row  = lane / CPR, ld_pc = lane % CPR;
+	const int  k_chunk = ld_pc ^ k_swizzle<DP>(ld_row);
+	const int  v_chunk = ld_pc ^ v_swizzle<DP>(ld_row);
+	const int  k_voff  = (int)(ld_row * p.k_stride[2] * 2) + (k_chunk * 8 < D ? k_chunk * 16 : 0);   // (padded head columns: the first chunk again)
+	const int  v_voff  = (int)(ld_row * p.v_stride[2] * 2) + (v_chunk * 8 < D ? v_chunk * 16 : 0);
+	const int  k_row_bytes = (int)(p.k_stride[2] * 2), v_row_bytes = (int)(p.v_stride[2] * 2);
+	const int  k_tile_stride = (int)(KT * p.k_stride[2] * 2), v_tile_stride = (int)(KT * p.v_stride[2] * 2);
+	const int  k_ld_stride   = (int)(RPI * p.k_stride[2] * 2), v_ld_stride = (int)(RPI * p.v_stride[2] * 2);
+	// byte offsets of piece j of tile kt for this lane; a piece that reaches past the last key (rare, wave-uniform test)
+	// sends the lanes of rows >= L to row L - 1
+	auto kv_offsets = [&](int kt, int j, int& ko, int& vo) {
+		ko = k_voff + (kt * k_tile_stride + j * k_ld_stride), vo = v_voff + (kt * v_tile_stride + j * v_ld_stride);
+		const int row0 = kt * KT + j * RPI;
+		if(row0 + RPI > (int)L) {
+			const int over = row0 + lane / CPR - ((int)L - 1);
+			if(over > 0) ko -= over * k_row_bytes, vo -= over * v_row_bytes;
+		}
+	};
+	const uint32_t k_lds_addr = lds_addr_of(k_lds), v_lds_addr = lds_addr_of(v_lds);
+	auto load_tile = [&](int kt, int buf) {
+		if(FUSED) return;  // K and V of every tile are already in LDS
+		if constexpr(KS2) {  // the 2 * NI pieces of K and V are dealt out over all NW wavefronts
+#pragma unroll
+			for(int t = 0; t < 2 * NI / NW; t++) {
+				const int pc = wave + NW * t;  // (wave-uniform)
+				int       ko, vo;
+				kv_offsets(kt, pc < NI ? pc : pc - NI, ko, vo);
+				if(pc < NI) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + pc * 1024, ko);
+				else lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + (pc - NI) * 1024, vo);
+			}
+			return;
+		}
+#pragma unroll
+		for(int t = 0; t < (SPLIT ? NI : NI / NW); t++) {
+			const int j = SPLIT ? t : wave + NW * t;  // split: this wavefront fetches whole tiles into its private buffers
+			int ko, vo;
+			kv_offsets(kt, j, ko, vo);
+			lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + j * 1024, ko);
+			lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + j * 1024, vo);
+		}
+	};
+
+	// ---- bias ring (BRING): the 32 x 64 bias tile of this wavefront's query block, 4 KB, travels
+	// HBM -> LDS by four LDS-direct loads of whole 128-byte row segments (eight lanes per row), two
+	// tiles ahead of its use and without occupying registers.  Slot layout: [row 32][128 B], the
+	// 16-byte chunk c of row r stored at chunk position c ^ (r & 7) so that the fragment reads (one
+	// chunk per lane, 32 rows at once) spread over the banks.  Rows past L fetch row L - 1 and chunks of
+	// keys past L (last tile) the row's last valid chunk, so padding behind a row's L valid entries is
+	// never read and every byte of a slot is written with finite data by every load.
+	const u32x4    b_rsrc    = raw_rsrc(BRING ? static_cast<const uint16_t*>(p.bias) + h * p.bias_stride[0] : nullptr,
+										BRING ? (uint32_t)(((L - 1) * p.bias_stride[1] + L) * 2) : 0u);
+	unsigned char* const bring = smem + LDS_SETS * 6 * TILE_BYTES + (BRING ? (KS2 ? wblk : wave) * 3 * 4096 : 0);
+	const uint32_t bring_addr = lds_addr_of(bring);
+	const int      b_voff     = (int)((lane >> 3) * p.bias_stride[1] * 2) + (((lane & 7) ^ (lane >> 3)) << 4);
+	const int      b_row0     = (int)((qtile * QT + wblk * 32) * p.bias_stride[1] * 2);
+	const int      b_row8     = (int)(8 * p.bias_stride[1] * 2);
+	const int      b_key      = ((lane & 7) ^ (lane >> 3)) * 8;  // first key of this lane's chunk within a tile
+	auto load_bias_tile = [&](int kt, int slot_i) {
+		if(!BRING) return;
+		const int in_row   = kt * KT + b_key < (int)L ? b_voff + kt * (KT * 2) : b_voff - b_key * 2 + ((int)L - 8) * 2;
+		const int blk_row0 = (int)(qtile * QT + wblk * 32);
+#pragma unroll
+		for(int j = 0; j < 4; j++) {
+			if(KS2 && sub != (j >> 1)) continue;  // (KS2: each wavefront of the pair fetches half of the 32 x 64 tile for both)
+			int off = in_row + (b_row0 + j * b_row8);
+			if(blk_row0 + 32 > (int)L) {   // (rare, wave-uniform: the matrix' last query block)
+				const int over = blk_row0 + 8 * j + (lane >> 3) - ((int)L - 1);
+				if(over > 0) off -= over * (int)(p.bias_stride[1] * 2);
+			}
+			lds_dma_b128(b_rsrc, bring_addr + slot_i * 4096 + j * 1024, off);
+		}
+	};
+	// ---- key-mask bytes: requested first.  With 4-byte aligned mask rows
 	// a lane takes four keys per load (a chunk of 256 keys = four tiles per wavefront and load) and all of a wavefront's
 	// loads -- up to eight per pass -- are in flight together: one memory latency, not one per tile (a single row's walk
 	// is short enough for that to show). ----
@@ -204,6 +285,34 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		}
 	};
 	if(mask_vec) request_mask(wave);
+	[[maybe_unused]] u32x4 qraw[NC];
+	if constexpr(!FUSED) {
+		const int64_t   qrow0 = (int64_t)qtile * QT + wblk * 32 + n;
+		const uint16_t* qp    = static_cast<const uint16_t*>(p.q) + b * p.q_stride[0] + h * p.q_stride[1] + qrow0 * p.q_stride[2];
+#pragma unroll
+		for(int c = 0; c < NC; c++) {
+			const int d0 = 16 * c + 8 * half;
+			qraw[c]      = u32x4{0u, 0u, 0u, 0u};
+			if(qrow0 < L && d0 < D) qraw[c] = *reinterpret_cast<const u32x4*>(qp + d0);
+		}
+	}
+
+	// ---- The other first requests go out now as well: the two tiles of K and V (and of the bias ring) that this wavefront
+	// walks first if the leading tiles all hold a live key -- the tile list below tells; a wrong guess costs a second load
+	// into the same buffer, and loads land in issue order.  One memory latency then covers the mask bytes, q and the first
+	// tiles: a call too small to keep other workgroups on the compute unit has nothing else to hide them behind.  (These
+	// loads are younger than the mask bytes, and the compiler does not count them: its wait for the mask bytes also waits
+	// for most of them, which costs little since all were issued within a fraction of one latency.) ----
+	const int  guess_kt0 = SPLIT ? wave : 0, guess_kt1 = SPLIT ? wave + NW : 1;
+	const bool guessed0 = !FUSED && guess_kt0 < n_ktiles, guessed1 = !FUSED && guess_kt1 < n_ktiles;  // (wave-uniform)
+	if(guessed0) {
+		load_tile(guess_kt0, 0);
+		load_bias_tile(guess_kt0, 0);
+	}
+	if(guessed1) {
+		load_tile(guess_kt1, 1);
+		load_bias_tile(guess_kt1, 1);
+	}
 
 	// (The K/V buffers and the bias ring are not cleared: every load of a tile writes every byte of its buffer with finite
 	// data -- lanes of padded head columns fetch the row's first chunk again (q is zero there), rows and keys past L fetch the
@@ -398,8 +507,6 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	// ---- one pass per block of 32 query rows: exactly one pass unless FUSED ----
 	for(; qb_f >= 0; qb_f -= FUSED ? NW : 1) {
 		// ---- per-lane constants ----
-		const int     sub    = KS2 ? (wave & 1) : 0;             // KS2: which 32 keys of every 64-key tile this wavefront takes
-		const int     wblk   = SPLIT ? 0 : KS2 ? (wave >> 1) : wave;  // this wavefront's block of 32 query rows within the workgroup's QT rows
 		const int64_t qrow   = FUSED ? (int64_t)qb_f * 32 + n : (int64_t)qtile * QT + wblk * 32 + n;
 		const bool    row_ok = qrow < L;
 
@@ -407,13 +514,10 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		// scaled and rounded to bf16 (the reference also rounds the scaled q,
 		// src/csrc/dot_product_attention.cpp:95-98).
 		if constexpr(!FUSED) {
-			const uint16_t* qp = static_cast<const uint16_t*>(p.q) + b * p.q_stride[0] + h * p.q_stride[1] + qrow * p.q_stride[2];
 #pragma unroll
 			for(int c = 0; c < NC; c++) {
-				const int d0  = 16 * c + 8 * half;
-				u32x4     raw = {0u, 0u, 0u, 0u};
-				if(row_ok && d0 < D) raw = *reinterpret_cast<const u32x4*>(qp + d0);
-				u32x4 sc;
+				const u32x4 raw = qraw[c];
+				u32x4       sc;
 #pragma unroll
 				for(int j = 0; j < 4; j++) sc[j] = pack_bf16x2(bf16_bits_to_f32(raw[j] & 0xffffu) * qmul, bf16_bits_to_f32(raw[j] >> 16) * qmul);
 				qf[c] = __builtin_bit_cast(bf16x8, sc);
@@ -477,83 +581,6 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 			}
 		}
 
-		// ---- K/V tile loader: buffer loads that write LDS directly ----
-		// One wave load moves 1 KB: lane i -> LDS chunk i of the load's 1 KB window, i.e. tile row
-		// j*RPI + i/CPR, physical chunk i%CPR.  The lane picks the global chunk that belongs there
-		// under the swizzle; lanes of padded head columns (chunk*8 >= D) fetch the row's first chunk.
-		const u32x4 k_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.k) + b * p.k_stride[0] + h * p.k_stride[1], (uint32_t)(((L - 1) * p.k_stride[2] + D) * 2));
-		const u32x4 v_rsrc = raw_rsrc(static_cast<const uint16_t*>(p.v) + b * p.v_stride[0] + h * p.v_stride[1], (uint32_t)(((L - 1) * p.v_stride[2] + D) * 2));
-		const int  ld_row  = lane / CPR, ld_pc = lane % CPR;
-		const int  k_chunk = ld_pc ^ k_swizzle<DP>(ld_row);
-		const int  v_chunk = ld_pc ^ v_swizzle<DP>(ld_row);
-		const int  k_voff  = (int)(ld_row * p.k_stride[2] * 2) + (k_chunk * 8 < D ? k_chunk * 16 : 0);   // (padded head columns: the first chunk again)
-		const int  v_voff  = (int)(ld_row * p.v_stride[2] * 2) + (v_chunk * 8 < D ? v_chunk * 16 : 0);
-		const int  k_row_bytes = (int)(p.k_stride[2] * 2), v_row_bytes = (int)(p.v_stride[2] * 2);
-		const int  k_tile_stride = (int)(KT * p.k_stride[2] * 2), v_tile_stride = (int)(KT * p.v_stride[2] * 2);
-		const int  k_ld_stride   = (int)(RPI * p.k_stride[2] * 2), v_ld_stride = (int)(RPI * p.v_stride[2] * 2);
-		// byte offsets of piece j of tile kt for this lane; a piece that reaches past the last key (rare, wave-uniform test)
-		// sends the lanes of rows >= L to row L - 1
-		auto kv_offsets = [&](int kt, int j, int& ko, int& vo) {
-			ko = k_voff + (kt * k_tile_stride + j * k_ld_stride), vo = v_voff + (kt * v_tile_stride + j * v_ld_stride);
-			const int row0 = kt * KT + j * RPI;
-			if(row0 + RPI > (int)L) {
-				const int over = row0 + lane / CPR - ((int)L - 1);
-				if(over > 0) ko -= over * k_row_bytes, vo -= over * v_row_bytes;
-			}
-		};
-		const uint32_t k_lds_addr = lds_addr_of(k_lds), v_lds_addr = lds_addr_of(v_lds);
-		auto load_tile = [&](int kt, int buf) {
-			if(FUSED) return;  // K and V of every tile are already in LDS
-			if constexpr(KS2) {  // the 2 * NI pieces of K and V are dealt out over all NW wavefronts
-#pragma unroll
-				for(int t = 0; t < 2 * NI / NW; t++) {
-					const int pc = wave + NW * t;  // (wave-uniform)
-					int       ko, vo;
-					kv_offsets(kt, pc < NI ? pc : pc - NI, ko, vo);
-					if(pc < NI) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + pc * 1024, ko);
-					else lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + (pc - NI) * 1024, vo);
-				}
-				return;
-			}
-#pragma unroll
-			for(int t = 0; t < (SPLIT ? NI : NI / NW); t++) {
-				const int j = SPLIT ? t : wave + NW * t;  // split: this wavefront fetches whole tiles into its private buffers
-				int ko, vo;
-				kv_offsets(kt, j, ko, vo);
-				lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + j * 1024, ko);
-				lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + j * 1024, vo);
-			}
-		};
-
-		// ---- bias ring (BRING): the 32 x 64 bias tile of this wavefront's query block, 4 KB, travels
-		// HBM -> LDS by four LDS-direct loads of whole 128-byte row segments (eight lanes per row), two
-		// tiles ahead of its use and without occupying registers.  Slot layout: [row 32][128 B], the
-		// 16-byte chunk c of row r stored at chunk position c ^ (r & 7) so that the fragment reads (one
-		// chunk per lane, 32 rows at once) spread over the banks.  Rows past L fetch row L - 1 and chunks of
-		// keys past L (last tile) the row's last valid chunk, so padding behind a row's L valid entries is
-		// never read and every byte of a slot is written with finite data by every load.
-		const u32x4    b_rsrc    = raw_rsrc(BRING ? static_cast<const uint16_t*>(p.bias) + h * p.bias_stride[0] : nullptr,
-											BRING ? (uint32_t)(((L - 1) * p.bias_stride[1] + L) * 2) : 0u);
-		unsigned char* const bring = smem + LDS_SETS * 6 * TILE_BYTES + (BRING ? (KS2 ? wblk : wave) * 3 * 4096 : 0);
-		const uint32_t bring_addr = lds_addr_of(bring);
-		const int      b_voff     = (int)((lane >> 3) * p.bias_stride[1] * 2) + (((lane & 7) ^ (lane >> 3)) << 4);
-		const int      b_row0     = (int)((qtile * QT + wblk * 32) * p.bias_stride[1] * 2);
-		const int      b_row8     = (int)(8 * p.bias_stride[1] * 2);
-		const int      b_key      = ((lane & 7) ^ (lane >> 3)) * 8;  // first key of this lane's chunk within a tile
-		auto load_bias_tile = [&](int kt, int slot_i) {
-			if(!BRING || (KS2 && sub != 0)) return;  // (KS2: the pair's first wavefront fetches the whole 32 x 64 tile for both)
-			const int in_row   = kt * KT + b_key < (int)L ? b_voff + kt * (KT * 2) : b_voff - b_key * 2 + ((int)L - 8) * 2;
-			const int blk_row0 = (int)(qtile * QT + wblk * 32);
-#pragma unroll
-			for(int j = 0; j < 4; j++) {
-				int off = in_row + (b_row0 + j * b_row8);
-				if(blk_row0 + 32 > (int)L) {   // (rare, wave-uniform: the matrix' last query block)
-					const int over = blk_row0 + 8 * j + (lane >> 3) - ((int)L - 1);
-					if(over > 0) off -= over * (int)(p.bias_stride[1] * 2);
-				}
-				lds_dma_b128(b_rsrc, bring_addr + slot_i * 4096 + j * 1024, off);
-			}
-		};
 		// fragment read: lane (n, half) takes chunk 4*sub + 2*c2 + half of row n
 		const int b_rd = (n * 128 + (((n & 7) ^ half) << 4)) ^ (sub << 6);  // (KS2: chunks 4..7 of a row hold keys 32..63)
 
@@ -839,11 +866,16 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		if(my_n > 0) {
 			// ---- prologue: first two tiles, first sub-tile's S^T and its row maximum ----
 			const int kt0 = __builtin_amdgcn_readfirstlane(live_at(0));
-			load_tile(kt0, 0);
-			load_bias_tile(kt0, 0);
+			if(!guessed0 || kt0 != guess_kt0) {
+				load_tile(kt0, 0);
+				load_bias_tile(kt0, 0);
+			}
 			if(my_n > 1) {
-				load_tile(__builtin_amdgcn_readfirstlane(live_at(1)), 1);
-				load_bias_tile(__builtin_amdgcn_readfirstlane(live_at(1)), 1);
+				const int kt1_first = __builtin_amdgcn_readfirstlane(live_at(1));
+				if(!guessed1 || kt1_first != guess_kt1) {
+					load_tile(kt1_first, 1);
+					load_bias_tile(kt1_first, 1);
+				}
 			}
 #pragma unroll
 			for(int f = 0; f < 4; f++) bfrag[f] = u32x4{0u, 0u, 0u, 0u};
@@ -1207,9 +1239,14 @@ static int launch_nw(const af3_dpa_params& p, hipStream_t s) {
 		// Long rows with too few 128-row workgroups to fill the 256 compute units: pairs of wavefronts share a query block and
 		// the workgroup's K/V tiles.  The work per SIMD is unchanged -- two wavefronts of half the length instead of one -- but
 		// the two overlap their matrix and vector phases (measured, B=1 H=16 L=1536: 26.0 against 31.1 us at head_dim 24; at
-		// head_dim 48, padded to 64, nothing is gained, so that size keeps one wavefront per query block).
+		// head_dim 48, padded to 64, nothing is gained, so that size keeps one wavefront per query block).  With 256..511
+		// query blocks the same pairing in 4-wave workgroups gives every compute unit at most one workgroup of uniform
+		// length, where 2-wave workgroups with private tiles put two on half of the compute units and fetch every tile
+		// twice as often (measured, B=1 H=16 L=768 D=24: 12.5 against 12.8 us; with 192 blocks, L=384, the four-way split
+		// of private tiles stays ahead: 7.5 against 9.0 us).
 		if constexpr(DP == 32) {
 			if(blocks1 >= 512 && blocks1 <= 1024 && ktiles >= 8) return launch_one<DP, 8, L2DOM, BMODE, false, true>(p, s);
+			if(blocks1 >= 256 && blocks1 < 512 && ktiles >= 8) return launch_one<DP, 4, L2DOM, BMODE, false, true>(p, s);
 		}
 		if(blocks1 >= 512) return launch_one<DP, 4, L2DOM, BMODE>(p, s);
 		// (the split variants' private buffers plus a long row's mask table can exceed the LDS of a compute unit: then the next one)

@@ -398,6 +398,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	// clamped from below like the workspace's values (packed unsigned minimum: -2^16 and everything beyond it, -inf and
 	// -NaN patterns included), widened to fp32 and scaled by log2 e
 	auto next_bias_fragment = [&] {
+		// (The old fragment is named once more behind its last reader: the registers it occupied then are the only free block of
+		// 16 when the new one is defined, so the fragment keeps its place from tile to tile.  Without this the compiler lets
+		// that reader's result overwrite the old fragment, puts the new one elsewhere and copies 16 registers per tile.)
+		asm volatile("" ::"v"(bias_frag));
 		if constexpr(SLOT) {
 #pragma unroll
 			for(int ld = 0; ld < 4; ld++) {

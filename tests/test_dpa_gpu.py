@@ -237,6 +237,25 @@ def test_values_at_dropped_keys_do_not_matter(af3):
     assert torch.equal(a, b_)
 
 
+@pytest.mark.parametrize("B,H,L,D,first_live", [
+    (48, 4, 256, 32, 64),     # four-wave workgroups, bias through the workspace: tile 0 is dead, tile 1 is the first
+    (48, 4, 256, 32, 130),    # tiles 0 and 1 are dead
+    (1, 16, 768, 24, 200),    # one row, key tiles split over two wavefronts: neither starts where it would without a mask
+    (1, 16, 1536, 24, 64),    # pairs of wavefronts on shared tiles, bias ring
+])
+def test_rows_whose_first_key_tiles_hold_no_live_key(af3, oracle, B, H, L, D, first_live):
+    """The kernel requests the tile it expects to walk first before it has read the key mask; when that tile turns out to
+    hold no live key the walk starts elsewhere and the tile's buffer is loaded again.  Some batch rows keep every key, so
+    both outcomes occur in one launch."""
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=L + first_live)
+    m[::2, :first_live] = False
+    prev = af3.set_rows_kernel("never")
+    try:
+        run_case(af3, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+    finally:
+        af3.set_rows_kernel(prev)
+
+
 def test_strided_inputs_and_prepadded_bias(af3, oracle):
     B, H, L, D, M = 2, 4, 100, 32, 128
     q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=10, mask="random")

@@ -122,7 +122,9 @@ __global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restric
 // KS2: the other cure for launches too small to fill the chip, for long rows: two wavefronts share each block of 32
 // query rows AND the workgroup's K/V tiles -- wavefront 2q + s takes keys [32s, 32s + 32) of every 64-key tile for
 // query block q, so a wavefront's dependent chain is half as long and no LDS is spent on private buffers; the two
-// partial (O, m, l) are merged through LDS at the end.  Requires NW even, no SPLIT, not FUSED.
+// partial (O, m, l) are merged through LDS at the end.  The workgroup has NW + 4 wavefronts: the last four only issue the
+// tile loads (a ring of four tiles, two tiles ahead), so that the NW computing ones never stand still behind a load that the
+// compute unit's load path has not taken in yet.  Requires NW even, head_dim <= 32, no SPLIT, not FUSED.
 // FUSED: the grid-attention variant.  One workgroup = one (batch, head); q, k, v and the gate are not
 // read from memory but projected in the kernel from the input rows x[b] (C channels) with the four
 // weight matrices of this head, K and V of ALL keys stay in LDS for the whole workgroup, and each
@@ -132,7 +134,7 @@ template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT, bool FUSED, bool KS
 // (at least 2 wavefronts per SIMD: keeps the register budget at 256 so that the compiler writes MFMA
 // results to ordinary VGPRs instead of AGPRs, which every softmax operand would have to be copied out of;
 // the key-split variants are limited to fewer than 2 wavefronts per SIMD by their LDS buffers anyway)
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FUSED ? (NW <= 4 ? 3 : (NW + 3) / 4) : DP == 32 && !SPLIT && !KS2 ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups, fused_grid_args fa) {
+__global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdgpu_waves_per_eu(FUSED ? (NW <= 4 ? 3 : (NW + 3) / 4) : KS2 ? 3 : DP == 32 && !SPLIT ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups, fused_grid_args fa) {
 	constexpr int NC         = DP / 16;            // contraction chunks of QK^T
 	constexpr int NDB        = DP / 32;            // 32-row blocks of O^T
 	constexpr int CPR        = DP / 8;             // 16-byte chunks per K/V row
@@ -143,21 +145,22 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	constexpr int  LDS_SETS   = SPLIT ? NW : 1;  // private K/V buffer sets
 	constexpr bool BIAS_F32   = BMODE == 1;      // natural variant, bias stored as fp32, read in place
 	constexpr bool BRING      = BMODE == 2;      // natural variant, bf16 bias streamed through a per-wavefront LDS ring
-	constexpr int  RING_BYTES = BRING ? (KS2 ? NW / 2 : NW) * 3 * 4096 : 0;  // (KS2: one ring per pair of wavefronts)
-	constexpr int  MASK_BASE  = LDS_SETS * 6 * TILE_BYTES + RING_BYTES;
+	constexpr int  NBUF       = KS2 ? 4 : 3;     // tile buffers of the K/V ring and slots of a bias ring (KS2: loads run two tiles ahead)
+	constexpr int  RING_BYTES = BRING ? (KS2 ? NW / 2 : NW) * NBUF * 4096 : 0;  // (KS2: one ring per pair of wavefronts)
+	constexpr int  MASK_BASE  = LDS_SETS * 2 * NBUF * TILE_BYTES + RING_BYTES;
 	static_assert(!(L2DOM && BMODE != 0), "the log2 variant reads its bias from the workspace");
 	static_assert(FUSED || (KS2 ? (2 * NI) % NW == 0 : NW <= NI), "every wavefront fetches a whole number of 1 KB pieces of each tile");
 	static_assert(!KS2 || (!SPLIT && !FUSED && NW % 2 == 0), "the shared-tile key split pairs up the wavefronts of an unfused workgroup");
 	static_assert(!FUSED || (DP == 32 && L2DOM && !SPLIT && NW % 2 == 0), "the fused variant exists for 32-channel heads in the log2 variant");
 
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-	// [K x3][V x3][bias ring: 3 x 4 KB per wavefront (BRING)][mask table: (n_ktiles*64 + 64) dwords][live list]
+	// [K x NBUF][V x NBUF][bias ring: NBUF x 4 KB per wavefront (BRING)][mask table: (n_ktiles*64 + 64) dwords][live list]
 	const int            tid_pre   = threadIdx.x;
 	// FUSED: [K of all tiles][V of all tiles][Wq fragments][Wgate fragments][mask table][live list]
 	const int            n_ktiles  = (int)((p.L + KT - 1) / KT);
 	constexpr int        NS        = 8;  // FUSED: contraction steps of a projection (C = 128 input channels, 16 per MFMA)
-	unsigned char* const k_lds     = smem + (SPLIT ? __builtin_amdgcn_readfirstlane(tid_pre >> 6) * 6 * TILE_BYTES : 0);
-	unsigned char* const v_lds     = k_lds + (FUSED ? n_ktiles : 3) * TILE_BYTES;
+	unsigned char* const k_lds     = smem + (SPLIT ? __builtin_amdgcn_readfirstlane(tid_pre >> 6) * 2 * NBUF * TILE_BYTES : 0);
+	unsigned char* const v_lds     = k_lds + (FUSED ? n_ktiles : NBUF) * TILE_BYTES;
 	unsigned char* const w_lds     = v_lds + n_ktiles * TILE_BYTES;  // FUSED only
 	const int            mask_base = FUSED ? 2 * n_ktiles * TILE_BYTES + 2 * NS * 1024 : MASK_BASE;
 	uint32_t* const      mask_tab  = reinterpret_cast<uint32_t*>(smem + mask_base);
@@ -185,6 +188,14 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	const int     wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int     n = lane & 31, half = lane >> 5;
 	const int64_t L = p.L;
+	// KS2: the workgroup has four wavefronts more than the NW that compute (one per SIMD).  They issue the tile loads of the
+	// workgroup, two tiles ahead, a quarter of every tile each, and otherwise only keep the barriers' count.  A wavefront that
+	// issues a tile's loads itself stands still while the compute unit's load path (64 bytes per clock) takes them in -- with
+	// one compute wavefront per SIMD nothing else runs in that time, and it was a quarter of the key loop.  (A single loader
+	// is too few: one wavefront gets a load accepted every 45-64 clocks at best.)
+	const bool    is_loader = KS2 && wave >= NW;
+	const int     ld        = wave - NW;  // which quarter (loader wavefronts)
+	static_assert(!KS2 || NI == 4, "four loader wavefronts take one 1 KB piece of K and one of V each");
 	const int     D = (int)p.D;
 
 	const int sub  = KS2 ? (wave & 1) : 0;                  // KS2: which 32 keys of every 64-key tile this wavefront takes
@@ -217,15 +228,12 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	const uint32_t k_lds_addr = lds_addr_of(k_lds), v_lds_addr = lds_addr_of(v_lds);
 	auto load_tile = [&](int kt, int buf) {
 		if(FUSED) return;  // K and V of every tile are already in LDS
-		if constexpr(KS2) {  // the 2 * NI pieces of K and V are dealt out over all NW wavefronts
-#pragma unroll
-			for(int t = 0; t < 2 * NI / NW; t++) {
-				const int pc = wave + NW * t;  // (wave-uniform)
-				int       ko, vo;
-				kv_offsets(kt, pc < NI ? pc : pc - NI, ko, vo);
-				if(pc < NI) lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + pc * 1024, ko);
-				else lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + (pc - NI) * 1024, vo);
-			}
+		if constexpr(KS2) {  // piece ld of K and of V, by loader wavefront ld
+			if(!is_loader) return;
+			int ko, vo;
+			kv_offsets(kt, ld, ko, vo);
+			lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + ld * 1024, ko);
+			lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + ld * 1024, vo);
 			return;
 		}
 #pragma unroll
@@ -247,7 +255,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	// never read and every byte of a slot is written with finite data by every load.
 	const u32x4    b_rsrc    = raw_rsrc(BRING ? static_cast<const uint16_t*>(p.bias) + h * p.bias_stride[0] : nullptr,
 										BRING ? (uint32_t)(((L - 1) * p.bias_stride[1] + L) * 2) : 0u);
-	unsigned char* const bring = smem + LDS_SETS * 6 * TILE_BYTES + (BRING ? (KS2 ? wblk : wave) * 3 * 4096 : 0);
+	unsigned char* const bring = smem + LDS_SETS * 2 * NBUF * TILE_BYTES + (BRING ? (KS2 ? wblk : wave) * NBUF * 4096 : 0);  // (compute wavefronts)
 	const uint32_t bring_addr = lds_addr_of(bring);
 	const int      b_voff     = (int)((lane >> 3) * p.bias_stride[1] * 2) + (((lane & 7) ^ (lane >> 3)) << 4);
 	const int      b_row0     = (int)((qtile * QT + wblk * 32) * p.bias_stride[1] * 2);
@@ -256,10 +264,24 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	auto load_bias_tile = [&](int kt, int slot_i) {
 		if(!BRING) return;
 		const int in_row   = kt * KT + b_key < (int)L ? b_voff + kt * (KT * 2) : b_voff - b_key * 2 + ((int)L - 8) * 2;
+		if constexpr(KS2) {  // eight rows (piece ld) of the tiles of all NW / 2 query blocks, by loader wavefront ld
+			if(!is_loader) return;
+			const uint32_t rings = lds_addr_of(smem + LDS_SETS * 2 * NBUF * TILE_BYTES);
+#pragma unroll
+			for(int wb = 0; wb < NW / 2; wb++) {
+				const int blk_row0 = (int)(qtile * QT + wb * 32);
+				int       off      = in_row + (int)(blk_row0 * p.bias_stride[1] * 2) + ld * b_row8;
+				if(blk_row0 + 32 > (int)L) {  // (rare, wave-uniform: the matrix' last query block and blocks past it)
+					const int over = blk_row0 + 8 * ld + (lane >> 3) - ((int)L - 1);
+					if(over > 0) off -= over * (int)(p.bias_stride[1] * 2);
+				}
+				lds_dma_b128(b_rsrc, rings + (wb * NBUF + slot_i) * 4096 + ld * 1024, off);
+			}
+			return;
+		}
 		const int blk_row0 = (int)(qtile * QT + wblk * 32);
 #pragma unroll
 		for(int j = 0; j < 4; j++) {
-			if(KS2 && sub != (j >> 1)) continue;  // (KS2: each wavefront of the pair fetches half of the 32 x 64 tile for both)
 			int off = in_row + (b_row0 + j * b_row8);
 			if(blk_row0 + 32 > (int)L) {   // (rare, wave-uniform: the matrix' last query block)
 				const int over = blk_row0 + 8 * j + (lane >> 3) - ((int)L - 1);
@@ -284,7 +306,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 			if(c0 + i * NW < n_chunks) mraw[i] = !keep ? 0x01010101u : (key0 < L ? *reinterpret_cast<const uint32_t*>(keep + key0) : 0u);
 		}
 	};
-	if(mask_vec) request_mask(wave);
+	if(mask_vec && !is_loader) request_mask(wave);
 	[[maybe_unused]] u32x4 qraw[NC];
 	if constexpr(!FUSED) {
 		const int64_t   qrow0 = (int64_t)qtile * QT + wblk * 32 + n;
@@ -293,7 +315,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 		for(int c = 0; c < NC; c++) {
 			const int d0 = 16 * c + 8 * half;
 			qraw[c]      = u32x4{0u, 0u, 0u, 0u};
-			if(qrow0 < L && d0 < D) qraw[c] = *reinterpret_cast<const u32x4*>(qp + d0);
+			if(qrow0 < L && d0 < D && !is_loader) qraw[c] = *reinterpret_cast<const u32x4*>(qp + d0);
 		}
 	}
 
@@ -325,7 +347,9 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	if(tid == 0) s_nvalid = 0;
 	if(tid < 64) mask_tab[n_ktiles * KT + tid] = 0u;
 	__syncthreads();
-	if(mask_vec) {
+	if(is_loader) {
+		// (the loader wavefront takes no part in the table)
+	} else if(mask_vec) {
 		for(int c0 = wave; c0 < n_chunks; c0 += 8 * NW) {
 			if(c0 != wave) request_mask(c0);
 #pragma unroll
@@ -388,6 +412,50 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 	// A batch row without any live key: q and the bias are dropped so that every logit is exactly
 	// the mask constant and the weights come out uniform whatever the accumulation order.
 	const bool all_dropped = __builtin_amdgcn_readfirstlane(s_nvalid) == 0;
+
+	if constexpr(KS2) {
+		if(is_loader) {
+			// ---- a loader wavefront: tile j of the walk goes to buffer j % NBUF and is requested two tiles before the compute
+			// wavefronts fetch K fragments from it.  Its barriers mirror theirs one for one: one in front of the first S^T, one
+			// per live tile, three in the merge. ----
+			constexpr int PER_TILE = 2 + (BRING ? NW / 2 : 0);  // this wavefront's loads per tile
+			static_assert(PER_TILE <= 63, "the wait counter has six bits");
+			auto walk = [&](int j) -> int { return __builtin_amdgcn_readfirstlane((int)live_list[j < nlive ? j : nlive - 1]); };
+			const int kt0 = walk(0);
+			if(!guessed0 || kt0 != guess_kt0) {
+				load_tile(kt0, 0);
+				load_bias_tile(kt0, 0);
+			}
+			if(nlive > 1) {
+				const int kt1 = walk(1);
+				if(!guessed1 || kt1 != guess_kt1) {
+					load_tile(kt1, 1);
+					load_bias_tile(kt1, 1);
+				}
+			}
+			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+			__syncthreads();  // (tiles 0 and 1 are in LDS)
+			if(nlive > 2) {
+				load_tile(walk(2), 2);
+				load_bias_tile(walk(2), 2);
+			}
+			for(int it = 0; it < nlive; it++) {
+				// tile it + 1 has landed (tile it + 2, if there is one, may still be on its way)
+				if(it + 2 < nlive) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_TILE) : "memory");
+				else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+				__syncthreads();  // (every wavefront is done with tile it - 1, whose buffer tile it + 3 takes)
+				if(it + 3 < nlive) {
+					load_tile(walk(it + 3), (it + 3) % NBUF);
+					load_bias_tile(walk(it + 3), (it + 3) % NBUF);
+				}
+			}
+			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+			__syncthreads();
+			__syncthreads();
+			__syncthreads();
+			return;
+		}
+	}
 
 	// ---- FUSED: projections.  out^T[d][token] = sum_c W[c][d] * x[token][c], 32 tokens per matrix instruction chain:
 	//   A operand (weights)    lane (d = lane%32, g = lane/32), step s: W[16s + 8g + 0..7][d]; in the panel layout
@@ -896,20 +964,14 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 			int kt = kt0, kt1 = __builtin_amdgcn_readfirstlane(live_at(1)), kt2 = __builtin_amdgcn_readfirstlane(live_at(2));
 			for(int it = 0; it < my_n; it++) {
 				const int kt3_v = live_at(it + 3);
-				const int bufn = buf == 2 ? 0 : buf + 1, bufnn = bufn == 2 ? 0 : bufn + 1;
+				const int bufn = buf == NBUF - 1 ? 0 : buf + 1, bufnn = bufn == NBUF - 1 ? 0 : bufn + 1;
 				// LDS offsets of tile it and of tile it+1: ring buffers, or the tiles' own places when all of K and V is resident
 				const int off_cur = (FUSED ? kt : buf) * TILE_BYTES, off_next = (FUSED ? kt1 : bufn) * TILE_BYTES;
 				if constexpr(KS2) {
-					// One stage per tile: this wavefront's 32 keys of tile `it` (exp, V fragments) and of tile it+1 (S^T).  Tile
-					// it+1 (issued one iteration ago, or in the prologue) must have landed and everyone must be done with tile
-					// it-1 before tile it+2 overwrites it; the only younger loads are the two bias fragments of the log2 variant.
-					if(L2DOM && has_bias) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-					else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+					// One stage per tile: this wavefront's 32 keys of tile `it` (exp, V fragments) and of tile it+1 (S^T).  Behind
+					// the barrier tile it+1 is in LDS (the loader wavefront has waited for it) and everyone is done with tile
+					// it-1, whose buffer the loader now hands to tile it+3.
 					__syncthreads();
-					if(it + 2 < my_n) {
-						load_tile(kt2, bufnn);
-						load_bias_tile(kt2, bufnn);
-					}
 					stage(ic<0>{}, off_next, mask_rd + kt1 * mask_stride, off_cur, ic<0>{}, kt2, ic<0>{}, bufn * 4096);
 					buf = bufn;
 					kt  = kt1;
@@ -955,7 +1017,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(FU
 			__syncthreads();  // all K/V buffers are dead: reuse the front of LDS
 			float* const mred = reinterpret_cast<float*>(smem);        // [NW][32] reference maxima
 			float* const obuf = mred + NW * 32;                        // [NW / 2][16*NDB + 1][64]
-			static_assert((NW * 32 + (NW / 2) * (16 * NDB + 1) * 64) * 4 <= 6 * TILE_BYTES, "the merge area fits in the K/V buffers");
+			static_assert((NW * 32 + (NW / 2) * (16 * NDB + 1) * 64) * 4 <= 2 * NBUF * TILE_BYTES, "the merge area fits in the K/V buffers");
 			if(half == 0) mred[wave * 32 + n] = m_ref;
 			__syncthreads();
 			const float mstar   = fmaxf(mred[(wave & ~1) * 32 + n], mred[(wave | 1) * 32 + n]);
@@ -1131,7 +1193,8 @@ template <int DP, int NW, int BMODE, bool SPLIT, bool KS2 = false>
 static size_t lds_bytes(const af3_dpa_params& p) {
 	const size_t n_ktiles = (size_t)((p.L + KT - 1) / KT);
 	const size_t writers  = SPLIT ? 1 : KS2 ? NW / 2 : NW;  // wavefronts that own a block of query rows
-	return (size_t)(SPLIT ? NW : 1) * 6 * KT * DP * 2 + (BMODE == 2 ? (KS2 ? NW / 2 : NW) * 3 * 4096 : 0) + (n_ktiles * KT + 64) * 4 + n_ktiles * 2 + 16 +
+	constexpr size_t NBUF = KS2 ? 4 : 3;  // (as in the kernel)
+	return (size_t)(SPLIT ? NW : 1) * 2 * NBUF * KT * DP * 2 + (BMODE == 2 ? (KS2 ? NW / 2 : NW) * NBUF * 4096 : 0) + (n_ktiles * KT + 64) * 4 + n_ktiles * 2 + 16 +
 		   (p.gate ? writers * 32 * DP * 2 : 0);
 }
 
@@ -1148,7 +1211,7 @@ static int launch_one(const af3_dpa_params& p, hipStream_t s) {
 	if(smem > 64 * 1024) {  // beyond the default dynamic-LDS limit: raise it for this kernel (idempotent, host side)
 		if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
 	}
-	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, n_qtiles, n_groups, fused_grid_args{});
+	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3((NW + (KS2 ? 4 : 0)) * 64), smem, s, p, n_qtiles, n_groups, fused_grid_args{});  // (KS2: plus the four loader wavefronts)
 	return launch_status();
 }
 
@@ -1238,12 +1301,13 @@ static int launch_nw(const af3_dpa_params& p, hipStream_t s) {
 		// single-wave workgroups; L=768 14.0 us split in two against 14.3 / 17.8; L=384 8.5 us split in four).
 		// Long rows with too few 128-row workgroups to fill the 256 compute units: pairs of wavefronts share a query block and
 		// the workgroup's K/V tiles.  The work per SIMD is unchanged -- two wavefronts of half the length instead of one -- but
-		// the two overlap their matrix and vector phases (measured, B=1 H=16 L=1536: 26.0 against 31.1 us at head_dim 24; at
-		// head_dim 48, padded to 64, nothing is gained, so that size keeps one wavefront per query block).  With 256..511
-		// query blocks the same pairing in 4-wave workgroups gives every compute unit at most one workgroup of uniform
-		// length, where 2-wave workgroups with private tiles put two on half of the compute units and fetch every tile
-		// twice as often (measured, B=1 H=16 L=768 D=24: 12.5 against 12.8 us; with 192 blocks, L=384, the four-way split
-		// of private tiles stays ahead: 7.5 against 9.0 us).
+		// the two overlap their matrix and vector phases, and four more wavefronts issue the workgroup's loads (measured,
+		// B=1 H=16 L=1536: 22.0 against 31.1 us at head_dim 24; at head_dim 48, padded to 64, the pairing gained nothing, so
+		// that size keeps one wavefront per query block).  With 256..511 query blocks the same pairing in workgroups of
+		// four compute wavefronts gives every compute unit at most one workgroup of uniform length, where 2-wave
+		// workgroups with private tiles put two on half of the compute units and fetch every tile twice as often
+		// (measured, B=1 H=16 L=768 D=24: 11.2 against 12.8 us; with 192 blocks, L=384, the four-way split of private
+		// tiles stays ahead: 7.5 against 8.4 us, and with 768 blocks eight compute wavefronts per workgroup: 22.0 against 29.9).
 		if constexpr(DP == 32) {
 			if(blocks1 >= 512 && blocks1 <= 1024 && ktiles >= 8) return launch_one<DP, 8, L2DOM, BMODE, false, true>(p, s);
 			if(blocks1 >= 256 && blocks1 < 512 && ktiles >= 8) return launch_one<DP, 4, L2DOM, BMODE, false, true>(p, s);

@@ -344,9 +344,9 @@ __global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdg
 	// entry = bf16 additive mask value in the low half (contraction slot 0) and, in the log2
 	// variant, 1.0 in the high half (slot 1, multiplies -m_ref); the last 64 entries are zero
 	// (read by the lanes of the upper half-wave, whose contraction slots are unused).
-	if(tid == 0) s_nvalid = 0;
+	// (No barrier in front of the table: each tile's flag has one writer, the count of live tiles is taken from the flags
+	// below, and the zero entries are first read in the key loop.)
 	if(tid < 64) mask_tab[n_ktiles * KT + tid] = 0u;
-	__syncthreads();
 	if(is_loader) {
 		// (the loader wavefront takes no part in the table)
 	} else if(mask_vec) {
@@ -371,7 +371,6 @@ __global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdg
 				if(lane < 4 && 4 * c + lane < n_ktiles) {
 					const bool tile_live = ((bal >> (16 * lane)) & 0xffffull) != 0;
 					live_list[4 * c + lane] = tile_live ? 1 : 0;
-					if(tile_live) atomicAdd(&s_nvalid, 1);
 				}
 			}
 		}
@@ -385,7 +384,6 @@ __global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdg
 			const unsigned long long bal = __ballot(live);
 			if(lane == 0) {
 				live_list[kt] = bal ? 1 : 0;
-				if(bal) atomicAdd(&s_nvalid, 1);
 			}
 		}
 	}
@@ -394,7 +392,9 @@ __global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdg
 	// number of live tiles below).  If no key of this batch row is live every tile is kept: the
 	// result is then the mean over all L keys.
 	if(wave == 0) {
-		const bool all = (s_nvalid == 0);
+		bool any_live = false;
+		for(int base = 0; base < n_ktiles; base += 64) any_live = any_live || __ballot(base + lane < n_ktiles && live_list[base + lane] != 0) != 0;
+		const bool all = !any_live;
 		int        cnt = 0;
 		for(int base = 0; base < n_ktiles; base += 64) {
 			const int  kt   = base + lane;
@@ -405,7 +405,7 @@ __global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdg
 			if(keepit) live_list[cnt + rank] = (int16_t)kt;
 			cnt += __builtin_popcountll(bal);
 		}
-		if(lane == 0) s_nlive = cnt;
+		if(lane == 0) s_nlive = cnt, s_nvalid = any_live ? 1 : 0;
 	}
 	__syncthreads();
 	const int nlive = __builtin_amdgcn_readfirstlane(s_nlive);

@@ -147,6 +147,10 @@ def test_small_grids_split_keys_over_wavefronts(af3, oracle, B, H, L, D, live):
     (8, 2048, 32, "f32", None),            # fp32 bias read in place
     (16, 1000, 32, "unaligned", 900),      # bias rows that cannot take 16-byte loads: element-wise path; ragged last tile
     (16, 1536, 16, "none_live_tail", 33),  # only the first 33 keys are live
+    (12, 1000, 32, "bf16", (100, 900)),    # 384 query blocks: workgroups of four computing wavefronts; ragged last tile, dead tiles at both ends
+    (10, 1000, 32, "f32", None),           # the same with an fp32 bias read in place
+    (10, 1000, 16, "unaligned", 900),      # ... and with bias rows that cannot take 16-byte loads
+    (9, 1056, 24, "bf16", 70),             # 297 blocks, 17 key tiles of which two are live: the loading wavefronts have nothing to fetch after the first two
 ])
 def test_long_rows_pair_up_wavefronts_on_shared_tiles(af3, oracle, H, L, D, bias_kind, live):
     """B = 1 with 512..1024 query blocks and at least 8 key tiles: two wavefronts share each query block and the workgroup's

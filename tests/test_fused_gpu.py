@@ -171,6 +171,8 @@ SELF_CASES = [
     (64, 768, 16, torch.bfloat16),       # the diffusion transformer's shape: 16 heads of 48 channels
     (1536, 768, 16, torch.bfloat16),     # its longest sequence (heads of 48 channels: one wavefront per query block, gate rows in LDS)
     (1536, 384, 16, torch.bfloat16),     # heads of 24 channels: pairs of wavefronts per query block share K/V tiles; the pair's first one applies the gate
+    (768, 384, 16, torch.bfloat16),      # 384 query blocks: the same pairing in workgroups of four computing wavefronts
+    (1000, 384, 16, torch.bfloat16),     # ragged last key tile and last query block
     (200, 768, 16, torch.bfloat16),
     (77, 256, 8, torch.bfloat16),
     (150, 128, 4, torch.float32),

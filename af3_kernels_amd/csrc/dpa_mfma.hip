@@ -124,32 +124,37 @@ __global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restric
 // query block q, so a wavefront's dependent chain is half as long and no LDS is spent on private buffers; the two
 // partial (O, m, l) are merged through LDS at the end.  The workgroup has NW + 4 wavefronts: the last four only issue the
 // tile loads (a ring of four tiles, two tiles ahead), so that the NW computing ones never stand still behind a load that the
-// compute unit's load path has not taken in yet.  Requires NW even, head_dim <= 32, no SPLIT, not FUSED.
+// compute unit's load path has not taken in yet.  Requires NW even, no SPLIT, not FUSED.  (KSL = 1.  KSL = 2: the four
+// loading wavefronts and the ring of four tiles for workgroups of NW wavefronts with a query block each -- the form that
+// single rows of head_dim 48 or 64 take.)
 // FUSED: the grid-attention variant.  One workgroup = one (batch, head); q, k, v and the gate are not
 // read from memory but projected in the kernel from the input rows x[b] (C channels) with the four
 // weight matrices of this head, K and V of ALL keys stay in LDS for the whole workgroup, and each
 // wavefront then walks query blocks qb = wave, wave + NW, ... on its own (no barrier after the
 // projection of K and V).  Requires DP = 32, the log2 variant, no key split.
-template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT, bool FUSED, bool KS2>
+template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT, bool FUSED, int KSL>
 // (at least 2 wavefronts per SIMD: keeps the register budget at 256 so that the compiler writes MFMA
 // results to ordinary VGPRs instead of AGPRs, which every softmax operand would have to be copied out of;
 // the key-split variants are limited to fewer than 2 wavefronts per SIMD by their LDS buffers anyway)
-__global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdgpu_waves_per_eu(FUSED ? (NW <= 4 ? 3 : (NW + 3) / 4) : KS2 ? 3 : DP == 32 && !SPLIT ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups, fused_grid_args fa) {
+__global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdgpu_waves_per_eu(FUSED ? (NW <= 4 ? 3 : (NW + 3) / 4) : KSL ? (NW + 7) / 4 : DP == 32 && !SPLIT ? (L2DOM ? 4 : 3) : 2))) dpa_mfma_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups, fused_grid_args fa) {
 	constexpr int NC         = DP / 16;            // contraction chunks of QK^T
 	constexpr int NDB        = DP / 32;            // 32-row blocks of O^T
 	constexpr int CPR        = DP / 8;             // 16-byte chunks per K/V row
 	constexpr int TILE_BYTES = KT * DP * 2;
 	constexpr int NI         = TILE_BYTES / 1024;  // 1 KB wave loads per tile and tensor
 	constexpr int RPI        = 512 / DP;           // tile rows covered by one wave load
+	constexpr bool KS2       = KSL == 1;           // pairs of wavefronts on shared tiles (with loading wavefronts)
+	constexpr bool LOADERS   = KSL != 0;           // four more wavefronts issue the tile loads (KSL == 2: one computing wavefront per query block)
 	constexpr int QT         = SPLIT ? 32 : KS2 ? NW * 16 : NW * 32;
 	constexpr int  LDS_SETS   = SPLIT ? NW : 1;  // private K/V buffer sets
 	constexpr bool BIAS_F32   = BMODE == 1;      // natural variant, bias stored as fp32, read in place
 	constexpr bool BRING      = BMODE == 2;      // natural variant, bf16 bias streamed through a per-wavefront LDS ring
-	constexpr int  NBUF       = KS2 ? 4 : 3;     // tile buffers of the K/V ring and slots of a bias ring (KS2: loads run two tiles ahead)
+	constexpr int  NBUF       = LOADERS ? 4 : 3;  // tile buffers of the K/V ring and slots of a bias ring (with loading wavefronts: loads run two tiles ahead)
 	constexpr int  RING_BYTES = BRING ? (KS2 ? NW / 2 : NW) * NBUF * 4096 : 0;  // (KS2: one ring per pair of wavefronts)
 	constexpr int  MASK_BASE  = LDS_SETS * 2 * NBUF * TILE_BYTES + RING_BYTES;
 	static_assert(!(L2DOM && BMODE != 0), "the log2 variant reads its bias from the workspace");
-	static_assert(FUSED || (KS2 ? (2 * NI) % NW == 0 : NW <= NI), "every wavefront fetches a whole number of 1 KB pieces of each tile");
+	static_assert(FUSED || (LOADERS ? NI % 4 == 0 : NW <= NI), "every wavefront that loads fetches a whole number of 1 KB pieces of each tile");
+	static_assert(!LOADERS || (!SPLIT && !FUSED), "loading wavefronts serve workgroups that share their tiles");
 	static_assert(!KS2 || (!SPLIT && !FUSED && NW % 2 == 0), "the shared-tile key split pairs up the wavefronts of an unfused workgroup");
 	static_assert(!FUSED || (DP == 32 && L2DOM && !SPLIT && NW % 2 == 0), "the fused variant exists for 32-channel heads in the log2 variant");
 
@@ -193,9 +198,8 @@ __global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdg
 	// issues a tile's loads itself stands still while the compute unit's load path (64 bytes per clock) takes them in -- with
 	// one compute wavefront per SIMD nothing else runs in that time, and it was a quarter of the key loop.  (A single loader
 	// is too few: one wavefront gets a load accepted every 45-64 clocks at best.)
-	const bool    is_loader = KS2 && wave >= NW;
+	const bool    is_loader = LOADERS && wave >= NW;
 	const int     ld        = wave - NW;  // which quarter (loader wavefronts)
-	static_assert(!KS2 || NI == 4, "four loader wavefronts take one 1 KB piece of K and one of V each");
 	const int     D = (int)p.D;
 
 	const int sub  = KS2 ? (wave & 1) : 0;                  // KS2: which 32 keys of every 64-key tile this wavefront takes
@@ -228,12 +232,16 @@ __global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdg
 	const uint32_t k_lds_addr = lds_addr_of(k_lds), v_lds_addr = lds_addr_of(v_lds);
 	auto load_tile = [&](int kt, int buf) {
 		if(FUSED) return;  // K and V of every tile are already in LDS
-		if constexpr(KS2) {  // piece ld of K and of V, by loader wavefront ld
+		if constexpr(LOADERS) {  // pieces ld, ld + 4, ... of K and of V, by loader wavefront ld
 			if(!is_loader) return;
-			int ko, vo;
-			kv_offsets(kt, ld, ko, vo);
-			lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + ld * 1024, ko);
-			lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + ld * 1024, vo);
+#pragma unroll
+			for(int t = 0; t < NI / 4; t++) {
+				const int j = ld + 4 * t;
+				int       ko, vo;
+				kv_offsets(kt, j, ko, vo);
+				lds_dma_b128(k_rsrc, k_lds_addr + buf * TILE_BYTES + j * 1024, ko);
+				lds_dma_b128(v_rsrc, v_lds_addr + buf * TILE_BYTES + j * 1024, vo);
+			}
 			return;
 		}
 #pragma unroll
@@ -264,11 +272,11 @@ __global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdg
 	auto load_bias_tile = [&](int kt, int slot_i) {
 		if(!BRING) return;
 		const int in_row   = kt * KT + b_key < (int)L ? b_voff + kt * (KT * 2) : b_voff - b_key * 2 + ((int)L - 8) * 2;
-		if constexpr(KS2) {  // eight rows (piece ld) of the tiles of all NW / 2 query blocks, by loader wavefront ld
+		if constexpr(LOADERS) {  // eight rows (piece ld) of the tiles of all the workgroup's query blocks, by loader wavefront ld
 			if(!is_loader) return;
 			const uint32_t rings = lds_addr_of(smem + LDS_SETS * 2 * NBUF * TILE_BYTES);
 #pragma unroll
-			for(int wb = 0; wb < NW / 2; wb++) {
+			for(int wb = 0; wb < (KS2 ? NW / 2 : NW); wb++) {
 				const int blk_row0 = (int)(qtile * QT + wb * 32);
 				int       off      = in_row + (int)(blk_row0 * p.bias_stride[1] * 2) + ld * b_row8;
 				if(blk_row0 + 32 > (int)L) {  // (rare, wave-uniform: the matrix' last query block and blocks past it)
@@ -413,12 +421,12 @@ __global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdg
 	// the mask constant and the weights come out uniform whatever the accumulation order.
 	const bool all_dropped = __builtin_amdgcn_readfirstlane(s_nvalid) == 0;
 
-	if constexpr(KS2) {
+	if constexpr(LOADERS) {
 		if(is_loader) {
 			// ---- a loader wavefront: tile j of the walk goes to buffer j % NBUF and is requested two tiles before the compute
 			// wavefronts fetch K fragments from it.  Its barriers mirror theirs one for one: one in front of the first S^T, one
-			// per live tile, three in the merge. ----
-			constexpr int PER_TILE = 2 + (BRING ? NW / 2 : 0);  // this wavefront's loads per tile
+			// per live tile, and (pairs) three in the merge. ----
+			constexpr int PER_TILE = 2 * (NI / 4) + (BRING ? (KS2 ? NW / 2 : NW) : 0);  // this wavefront's loads per tile
 			static_assert(PER_TILE <= 63, "the wait counter has six bits");
 			auto walk = [&](int j) -> int { return __builtin_amdgcn_readfirstlane((int)live_list[j < nlive ? j : nlive - 1]); };
 			const int kt0 = walk(0);
@@ -450,9 +458,11 @@ __global__ void __launch_bounds__((NW + (KS2 ? 4 : 0)) * 64) __attribute__((amdg
 				}
 			}
 			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-			__syncthreads();
-			__syncthreads();
-			__syncthreads();
+			if constexpr(KS2) {
+				__syncthreads();
+				__syncthreads();
+				__syncthreads();
+			}
 			return;
 		}
 	}
@@ -1189,29 +1199,30 @@ static int launch_bias_prepass(const af3_dpa_params& p, hipStream_t s) {
 constexpr size_t LDS_LIMIT = 160 * 1024;  // per workgroup on gfx950
 
 // dynamic LDS of one variant: K/V buffers, bias ring, mask table, tile list, gate rows of every wavefront that writes results
-template <int DP, int NW, int BMODE, bool SPLIT, bool KS2 = false>
+template <int DP, int NW, int BMODE, bool SPLIT, int KSL = 0>
 static size_t lds_bytes(const af3_dpa_params& p) {
 	const size_t n_ktiles = (size_t)((p.L + KT - 1) / KT);
+	constexpr bool   KS2  = KSL == 1;
 	const size_t writers  = SPLIT ? 1 : KS2 ? NW / 2 : NW;  // wavefronts that own a block of query rows
-	constexpr size_t NBUF = KS2 ? 4 : 3;  // (as in the kernel)
+	constexpr size_t NBUF = KSL ? 4 : 3;  // (as in the kernel)
 	return (size_t)(SPLIT ? NW : 1) * 2 * NBUF * KT * DP * 2 + (BMODE == 2 ? (KS2 ? NW / 2 : NW) * NBUF * 4096 : 0) + (n_ktiles * KT + 64) * 4 + n_ktiles * 2 + 16 +
 		   (p.gate ? writers * 32 * DP * 2 : 0);
 }
 
-template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT = false, bool KS2 = false>
+template <int DP, int NW, bool L2DOM, int BMODE, bool SPLIT = false, int KSL = 0>
 static int launch_one(const af3_dpa_params& p, hipStream_t s) {
-	constexpr int QT       = SPLIT ? 32 : KS2 ? NW * 16 : NW * 32;
+	constexpr int QT       = SPLIT ? 32 : KSL == 1 ? NW * 16 : NW * 32;
 	const int     n_qtiles = (int)((p.L + QT - 1) / QT);
 	const int64_t n_groups = p.B * p.H;
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
-	const size_t smem = lds_bytes<DP, NW, BMODE, SPLIT, KS2>(p);
+	const size_t smem = lds_bytes<DP, NW, BMODE, SPLIT, KSL>(p);
 	if(smem > LDS_LIMIT) return AF3_ERR_BAD_SHAPE;  // (launch_nw only picks variants that fit)
-	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BMODE, SPLIT, false, KS2>;
+	auto         kern = dpa_mfma_bf16_kernel<DP, NW, L2DOM, BMODE, SPLIT, false, KSL>;
 	if(smem > 64 * 1024) {  // beyond the default dynamic-LDS limit: raise it for this kernel (idempotent, host side)
 		if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
 	}
-	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3((NW + (KS2 ? 4 : 0)) * 64), smem, s, p, n_qtiles, n_groups, fused_grid_args{});  // (KS2: plus the four loader wavefronts)
+	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3((NW + (KSL ? 4 : 0)) * 64), smem, s, p, n_qtiles, n_groups, fused_grid_args{});  // (plus the four loader wavefronts)
 	return launch_status();
 }
 
@@ -1258,7 +1269,7 @@ static int launch_fused_nw(const af3_dpa_params& p, const fused_grid_args& fa, h
 	const int64_t blocks   = 16 * ((p.B + 3) / 4);  // see the kernel's workgroup -> (batch row, head) map
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
 	const size_t smem = fused_lds_bytes(p.L);
-	auto         kern = dpa_mfma_bf16_kernel<32, NW, true, 0, false, true, false>;
+	auto         kern = dpa_mfma_bf16_kernel<32, NW, true, 0, false, true, 0>;
 	if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
 	hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), smem, s, p, 1, n_groups, fa);
 	return launch_status();
@@ -1312,6 +1323,9 @@ static int launch_nw(const af3_dpa_params& p, hipStream_t s) {
 			if(blocks1 >= 512 && blocks1 <= 1024 && ktiles >= 8) return launch_one<DP, 8, L2DOM, BMODE, false, true>(p, s);
 			if(blocks1 >= 256 && blocks1 < 512 && ktiles >= 8) return launch_one<DP, 4, L2DOM, BMODE, false, true>(p, s);
 		}
+		// One wavefront per query block, too few 128-row workgroups to give a compute unit more than one: the four loading
+		// wavefronts again (measured, B=1 H=16 L=1536 D=48: 27.0 against 31.0 us).
+		if(blocks1 >= 512 && blocks1 <= 1024 && lds_bytes<DP, 4, BMODE, false, 2>(p) <= LDS_LIMIT) return launch_one<DP, 4, L2DOM, BMODE, false, 2>(p, s);
 		if(blocks1 >= 512) return launch_one<DP, 4, L2DOM, BMODE>(p, s);
 		// (the split variants' private buffers plus a long row's mask table can exceed the LDS of a compute unit: then the next one)
 		if(DP == 32 && ktiles >= 4 && blocks1 <= 256 && lds_bytes<DP, 4, BMODE, true>(p) <= LDS_LIMIT) return launch_one<DP, 4, L2DOM, BMODE, true>(p, s);

@@ -163,7 +163,40 @@ __device__ __forceinline__ void quantize_e4m3_body(const void* __restrict__ src,
 		w = __builtin_amdgcn_cvt_pk_fp8_f32(f2 - lo23[0], f3 - lo23[1], w, true);
 		return w;
 	};
-	if(!transpose) {
+	if(!transpose && src_row_stride == cols && dst_row_stride == cols && (reinterpret_cast<uintptr_t>(src) & 15) == 0 && (reinterpret_cast<uintptr_t>(dst) & 7) == 0 &&
+	   (!dst_lo || (reinterpret_cast<uintptr_t>(dst_lo) & 7) == 0) && rows * cols < ((int64_t)1 << 31)) {
+		// dense rows on both sides: the tensor is one run of elements; one thread = 8 consecutive elements (16- or 2 x 16-byte
+		// loads, 8-byte stores), no index arithmetic beyond the running offset
+		const int total8 = (int)((rows * cols) >> 3), step = (int)stride;
+		for(int i = (int)(blockIdx.x * EW_THREADS + threadIdx.x); i < total8; i += step) {
+			float f[8];
+			if(SRC_BF16) {
+				const u32x4 w = static_cast<const u32x4*>(src)[i];
+#pragma unroll
+				for(int j = 0; j < 4; j++) f[2 * j] = bf16_bits_to_f32(w[j] & 0xffffu), f[2 * j + 1] = bf16_bits_to_f32(w[j] >> 16);
+			} else {
+				const u32x4 w0 = static_cast<const u32x4*>(src)[2 * i], w1 = static_cast<const u32x4*>(src)[2 * i + 1];
+#pragma unroll
+				for(int j = 0; j < 4; j++) f[j] = __uint_as_float(w0[j]), f[4 + j] = __uint_as_float(w1[j]);
+			}
+#pragma unroll
+			for(int j = 0; j < 8; j++) f[j] = fminf(fmaxf(f[j] * mul, -448.f), 448.f);
+			uint32_t w0 = 0, w1 = 0;
+			w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], w0, false), w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w0, true);
+			w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], w1, false), w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], w1, true);
+			reinterpret_cast<u32x2*>(dst)[i] = u32x2{w0, w1};
+			if(dst_lo) reinterpret_cast<u32x2*>(dst_lo)[i] = u32x2{residual(f[0], f[1], f[2], f[3], w0), residual(f[4], f[5], f[6], f[7], w1)};
+		}
+		// (a tail of 4 elements when rows * cols is not a multiple of 8: cols % 4 == 0 is checked by the launcher)
+		if(((rows * cols) & 7) && blockIdx.x == 0 && threadIdx.x == 0) {
+			const int64_t e0 = (rows * cols) & ~(int64_t)7;
+			const float   f0 = ld(0, e0), f1 = ld(0, e0 + 1), f2 = ld(0, e0 + 2), f3 = ld(0, e0 + 3);
+			uint32_t      w  = 0;
+			w = __builtin_amdgcn_cvt_pk_fp8_f32(f0, f1, w, false), w = __builtin_amdgcn_cvt_pk_fp8_f32(f2, f3, w, true);
+			*reinterpret_cast<uint32_t*>(dst + e0) = w;
+			if(dst_lo) *reinterpret_cast<uint32_t*>(dst_lo + e0) = residual(f0, f1, f2, f3, w);
+		}
+	} else if(!transpose) {
 		// one thread = 4 consecutive columns of one row (cols % 4 == 0 is checked by the launcher)
 		const int64_t cq = cols >> 2, total = rows * cq;
 		for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += stride) {
@@ -180,18 +213,24 @@ __device__ __forceinline__ void quantize_e4m3_body(const void* __restrict__ src,
 		// rows past the end of a matrix quantise to zero, and the whole padded length of every output row
 		// (dst_row_stride, a multiple of 4) is written, so the destination needs no clearing beforehand
 		const int64_t rq = dst_row_stride >> 2, n_mat = rows / rows_per_matrix, total = n_mat * rq * cols;
-		for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += stride) {
-			const int64_t c   = i % cols;
-			const int64_t r4  = (i / cols) % rq;
-			const int64_t mat = i / (cols * rq);
-			const int64_t r   = mat * rows_per_matrix + (r4 << 2);
-			const int64_t left = rows_per_matrix - (r4 << 2);
+		// (index arithmetic in 32 bits when the count allows: 64-bit divisions cost several times the rest of the body)
+		auto element = [&](auto i, auto cols_i, auto rq_i) {
+			const auto    c    = i % cols_i;
+			const auto    r4   = (i / cols_i) % rq_i;
+			const int64_t mat  = i / (cols_i * rq_i);
+			const int64_t r    = mat * rows_per_matrix + ((int64_t)r4 << 2);
+			const int64_t left = rows_per_matrix - ((int64_t)r4 << 2);
 			const float   f0 = left > 0 ? ld(r, c) : 0.f, f1 = left > 1 ? ld(r + 1, c) : 0.f, f2 = left > 2 ? ld(r + 2, c) : 0.f, f3 = left > 3 ? ld(r + 3, c) : 0.f;
 			uint32_t      w   = 0;
 			w = __builtin_amdgcn_cvt_pk_fp8_f32(f0, f1, w, false);
 			w = __builtin_amdgcn_cvt_pk_fp8_f32(f2, f3, w, true);
-			*reinterpret_cast<uint32_t*>(dst + (mat * cols + c) * dst_row_stride + (r4 << 2)) = w;
-			if(dst_lo) *reinterpret_cast<uint32_t*>(dst_lo + (mat * cols + c) * dst_row_stride + (r4 << 2)) = residual(f0, f1, f2, f3, w);
+			*reinterpret_cast<uint32_t*>(dst + (mat * cols + c) * dst_row_stride + ((int64_t)r4 << 2)) = w;
+			if(dst_lo) *reinterpret_cast<uint32_t*>(dst_lo + (mat * cols + c) * dst_row_stride + ((int64_t)r4 << 2)) = residual(f0, f1, f2, f3, w);
+		};
+		if(total < ((int64_t)1 << 31) && stride < ((int64_t)1 << 30)) {
+			for(uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x; i < (uint32_t)total; i += (uint32_t)stride) element(i, (uint32_t)cols, (uint32_t)rq);
+		} else {
+			for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += stride) element(i, cols, rq);
 		}
 	}
 }

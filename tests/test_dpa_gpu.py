@@ -504,6 +504,7 @@ def rows_kernel(af3):
     (13, 1, 1, 32, "none", 2), (4, 5, 33, 32, "random", 2), (12, 4, 1491, 32, "random", 2),
     (2, 4, 128, 32, "none", 2), (3, 2, 200, 32, "random", 2), (5, 16, 256, 24, "tail", 1), (6, 3, 36, 24, "random", 2),   # groups of two and three rows
     (17, 2, 100, 32, "random", 2), (18, 2, 37, 32, "random", 2), (19, 1, 64, 16, "tail", 2),                          # 4 ... 4 + 3 + 2, + 2, + 3
+    (16, 1, 1024, 32, "random", 2), (18, 2, 992, 24, "tail", 2), (5, 16, 1536, 24, "random", 2),   # few workgroups, long rows
 ])
 def test_shared_bias_kernel_matches_formula(rows_kernel, oracle, B, H, L, D, mask, rank):
     """Every way the batch is cut into groups of four, three and two rows, with the bias through the rewritten workspace
@@ -520,6 +521,35 @@ def test_shared_bias_kernel_matches_formula(rows_kernel, oracle, B, H, L, D, mas
         run_case(rows_kernel, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
     finally:
         rows_kernel.set_exact_bias(prev)
+
+
+@pytest.mark.parametrize("pattern", ["even_tiles", "odd_tiles", "first_40", "last_tile", "row_without_keys"])
+def test_shared_bias_kernel_with_lopsided_masks(rows_kernel, oracle, pattern):
+    """Masks that leave whole key tiles without a live key (every other tile, everything but the first 40 keys, everything
+    but the last tile) or a batch row without any: the walk stops behind the last live key of the group, dead tiles in
+    between contribute exactly nothing, and both bf16 kernels agree."""
+    B, H, L, D = 3, 2, 800, 32
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=len(pattern))
+    tile = torch.arange(L) // 32
+    if pattern == "even_tiles":
+        m[:] = (tile % 2 == 0)[None, :]
+    elif pattern == "odd_tiles":
+        m[:] = (tile % 2 == 1)[None, :]
+        m[1] = (tile % 2 == 0)
+    elif pattern == "first_40":
+        m[:, 40:] = False
+    elif pattern == "last_tile":
+        m[:] = False
+        m[:, 790:] = True
+    else:
+        m[1, :] = False
+    run_case(rows_kernel, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
+    dq, dk, dv, dm, db = dev(q, k, v, m, bias)
+    a = rows_kernel.dot_product_attention_cpp(dq, dk, dv, dm, db)
+    rows_kernel.set_rows_kernel("never")
+    b = rows_kernel.dot_product_attention_cpp(dq, dk, dv, dm, db)
+    rows_kernel.set_rows_kernel("always")
+    assert (a.float() - b.float()).abs().max().item() <= 2e-2
 
 
 def test_shared_bias_kernel_applies_the_output_gate(rows_kernel, oracle):

@@ -709,6 +709,16 @@ int64_t mfma_rows_workspace_bytes(const af3_dpa_params& p) {
 
 bool mfma_rows_can_serve(const af3_dpa_params& p) { return mfma_rows_eligible(p) && rows_bias_mode(p) >= 0; }
 
+// A few batch rows that share a large bias of long rows: the one-row kernel's workspace rewrite is a pass over the whole
+// bias (read 2 bytes, write 2 bytes per entry: 23 us for 16 x 1536 x 1536) that no row of the batch amortises, while this
+// kernel reads the bias in place once per group of rows.  Measured on B x 16 x 1536 x 24 (one-row kernel with its rewrite
+// against this one): B = 2 61 / 53 us, 3 78 / 62 us, 5 79 / 75 us; with a 19 MB bias (5 x 16 x 768 x 24) 33 / 34 us, with a
+// 34 MB one (8 x 4 x 2048 x 32) 63 / 68 us; five samples through the fused caller (strided q, k, v, gate) 81 / 83 us of GPU
+// time: taken for up to four batch rows from 64 MB on.
+bool mfma_rows_saves_a_large_rewrite(const af3_dpa_params& p) {
+	return p.bias && p.B <= 4 && p.L >= 1024 && p.H * p.L * p.L * 2 >= (int64_t)64 << 20 && direct_bias_ok(p);
+}
+
 int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
 	const int mode = rows_bias_mode(p);
 	if(mode < 0) return AF3_ERR_BAD_ARGUMENT;

@@ -161,6 +161,7 @@ def _attend(y: torch.Tensor, B: int, N: int, head: int, mask, bias) -> torch.Ten
     p = _lib.DpaParams.from_buffer_copy(template)
     p.k, p.v, p.q, p.gate = base, base + K * esz, base + 2 * K * esz, base + 3 * K * esz   # per token and head: (k | v | q | gate)
     p.out = out.data_ptr()
+    p.reserved = ops._rows_kernel_hint
     if bias is not None:
         p.bias = bias.data_ptr()
         p.bias_stride[0], p.bias_stride[1] = bias.stride(0), bias.stride(1)

@@ -350,6 +350,13 @@ def main():
     import torch
     import af3_kernels_amd as af3
     from af3_kernels_amd.synthetic import CASES, FUSED_CASES, make_inputs
+    # Python's cyclic garbage collector runs a full collection every few hundred calls of the small cases (about 40 ms with
+    # torch loaded): a host pause that a GPU-bound step hides behind the launch queue and a 100-us step does not (measured:
+    # 104 -> 250 us per call of self5_n1536 in every third batch of 230 calls).  As timeit does, the collector is switched
+    # off while steps are timed; a long-running caller gets the same effect from gc.freeze() after start-up.
+    import gc
+    gc.collect()
+    gc.disable()
     af3._lib.load()
     if args.case in FUSED_CASES:
         return bench_fused(args, FUSED_CASES[args.case])

@@ -1165,15 +1165,14 @@ static int64_t ws_bytes_needed(const af3_dpa_params& p) {
 }
 
 // Whether the call goes to the kernel of dpa_mfma_rows.hip (four batch rows per wavefront sharing each bias tile): its
-// shape limits, enough workgroups of four-row groups to give every compute unit one (smaller launches mostly do better with
-// this file's variants: 16 x 4 x 768 x 32 26 us here against 32 us there) unless a few rows share a bias so large that the
-// workspace rewrite this file's variants need outweighs that, and the caller's hint (af3_dpa_params.reserved: 1 = take it
-// whenever the shape allows, 2 = never).
+// shape limits, enough workgroups of four-row groups to give every compute unit one (smaller launches through its workspace
+// do better with this file's variants: 16 x 4 x 768 x 32 26 us here against 32 us there) or fewer than 16 batch rows whose
+// bias it can stage in place, and the caller's hint (af3_dpa_params.reserved: 1 = take it whenever the shape allows, 2 = never).
 static bool rows_kernel_wanted(const af3_dpa_params& p) {
 	if(p.reserved == 2 || !mfma_rows_eligible(p)) return false;
 	if(p.reserved == 1) return true;
 	if((p.B / 4) * p.H * ((p.L + 127) / 128) >= 256) return true;  // (workgroups of the launch that takes the groups of four rows)
-	return mfma_rows_saves_a_large_rewrite(p);
+	return mfma_rows_suits_a_small_batch(p);
 }
 
 // The rewrite costs one extra pass over the bias; it pays off as soon as two batch rows share it.

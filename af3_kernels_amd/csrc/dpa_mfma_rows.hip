@@ -86,16 +86,19 @@ __global__ void __launch_bounds__(256) bias_rows_prepass_kernel(const void* __re
 // fetches the K and V tiles of batch row w.
 // BMODE: 0 = no bias (C operand zero); 1 = bias from the rewritten fp32 workspace, one 4 KB fragment per tile through this
 // wavefront's LDS slot; 2 = bf16 bias read in place (no workspace: for batches too small to pay for the rewrite), four
-// 8-byte loads per lane and tile, converted to the accumulator layout in registers.
+// 8-byte loads per lane and tile, converted to the accumulator layout in registers; 3 = bf16 bias read in place through LDS: the
+// 32 x 32 tile of this wavefront's query block travels as two 1 KB loads of whole 64-byte row segments straight into one of
+// two 2 KB halves of the wavefront's slot, a tile ahead of its conversion (needs 16-byte aligned rows; a quarter of mode
+// 2's cache-line requests, whose lanes each fetch from a row of their own).
 // The launch covers batch rows [b_first, b_first + b_count) in groups of ROWS.
 template <int ROWS, int BMODE>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) dpa_rows_bf16_kernel(af3_dpa_params p, int n_qtiles, int64_t n_groups, int64_t b_first, int64_t b_count) {
 	static_assert(ROWS >= 2 && ROWS <= 4, "two to four row chains per wavefront");
 	constexpr int  NW       = 4;
-	constexpr bool HAS_BIAS = BMODE != 0, SLOT = BMODE == 1, DIRECT = BMODE == 2;
+	constexpr bool HAS_BIAS = BMODE != 0, SLOT = BMODE == 1, DIRECT = BMODE == 2, STAGED = BMODE == 3;
 	constexpr int  BUF_R    = ROWS * 2 * TILE_R;                    // one buffer: [row][K tile | V tile]
 	constexpr int  SLOT_BASE = NBUF_R * BUF_R;                      // per-wavefront bias slots (4 KB each)
-	constexpr int  MASK_BASE = SLOT_BASE + (SLOT ? NW * 4096 : 0);
+	constexpr int  MASK_BASE = SLOT_BASE + (SLOT || STAGED ? NW * 4096 : 0);
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 	// [buffer 3][batch row 4][K tile 2 KB | V tile 2 KB] [bias slot 4 KB per wavefront] [mask table: (tiles + 1) x 4 rows x 32 keys, bf16 bits]
 	const int64_t L        = p.L;
@@ -124,6 +127,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	// stale LDS contents there must be finite ----
 	if(D != 32 || L % KT_R != 0) {
 		for(int i = tid; i < NBUF_R * BUF_R / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
+		__syncthreads();
+	}
+
+	if constexpr(STAGED) {  // (chunks past L are never fetched: what the slots hold there must be finite)
+		for(int i = tid; i < NW * 4096 / 16; i += NW * 64) reinterpret_cast<u32x4*>(smem + SLOT_BASE)[i] = u32x4{0u, 0u, 0u, 0u};
 		__syncthreads();
 	}
 
@@ -179,6 +187,27 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	const __amdgpu_buffer_rsrc_t bd_rsrc = __builtin_amdgcn_make_buffer_rsrc(
 		DIRECT ? const_cast<uint16_t*>(static_cast<const uint16_t*>(p.bias)) + h * p.bias_stride[0] : nullptr, 0, DIRECT ? (int)(((L - 1) * p.bias_stride[1] + L) * 2) : 0, 0x00020000);
 	const int bd_voff = (int)((qrow_b * p.bias_stride[1] + 4 * half) * 2);
+	// staged mode: lane i of load j fetches 16 bytes of row 16 j + i / 4 of the tile; the chunk it fetches is the one that
+	// belongs at its place under the swizzle (chunk c of row r sits at position c ^ ((r >> 2) & 3): the fragment reads of 32
+	// rows then spread over the banks).  Rows past L fetch row L - 1; chunks whose keys lie at or beyond L are sent out of
+	// range (nothing is fetched: the slot keeps finite data, and those keys carry the out-of-range mask value).
+	const u32x4 st_rsrc = raw_rsrc(STAGED ? static_cast<const uint16_t*>(p.bias) + h * p.bias_stride[0] : nullptr, STAGED ? (uint32_t)(((L - 1) * p.bias_stride[1] + L) * 2) : 0u);
+	int st_voff[2] = {0, 0};
+	int st_key[2]  = {0, 0};  // first key (within a tile) of the chunk this lane fetches
+	if constexpr(STAGED) {
+#pragma unroll
+		for(int j = 0; j < 2; j++) {
+			const int     r   = 16 * j + (lane >> 2), c = (lane & 3) ^ ((r >> 2) & 3);
+			const int64_t row = (int64_t)qtile * (NW * 32) + wave * 32 + r;
+			st_voff[j] = (int)((row < L ? row : L - 1) * p.bias_stride[1] * 2) + c * 16;
+			st_key[j]  = c * 8;
+		}
+	}
+	auto load_bias_staged = [&](int t) {
+		if(!STAGED || t >= n_t) return;
+#pragma unroll
+		for(int j = 0; j < 2; j++) lds_dma_b128(st_rsrc, lds_slot + (t & 1) * 2048 + j * 1024, t * KT_R + st_key[j] < L ? st_voff[j] + t * (KT_R * 2) : 0x40000000);
+	};
 	auto load_bias_direct = [&](int t) {
 		if(!DIRECT || t >= n_t) return;
 #pragma unroll
@@ -194,6 +223,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	load_tile(0, 0);
 	load_bias(0);
 	load_bias_direct(0);
+	load_bias_staged(0);
 	u32x4 qraw[ROWS][2];
 #pragma unroll
 	for(int r = 0; r < ROWS; r++) {
@@ -397,7 +427,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	// the next tile's bias fragment -> registers: from the slot, or (direct mode) from the raw bf16 pieces loaded a tile ago:
 	// clamped from below like the workspace's values (packed unsigned minimum: -2^16 and everything beyond it, -inf and
 	// -NaN patterns included), widened to fp32 and scaled by log2 e
-	auto next_bias_fragment = [&] {
+	auto next_bias_fragment = [&](int t_next) {  // t_next: the tile the fragment belongs to (staged mode: which half of the slot holds it)
 		// (The old fragment is named once more behind its last reader: the registers it occupied then are the only free block of
 		// 16 when the new one is defined, so the fragment keeps its place from tile to tile.  Without this the compiler lets
 		// that reader's result overwrite the old fragment, puts the new one elsewhere and copies 16 registers per tile.)
@@ -408,9 +438,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 				const f32x4 v = *reinterpret_cast<const f32x4*>(smem + slot_rd + ld * 1024);
 				bias_frag[4 * ld] = v[0], bias_frag[4 * ld + 1] = v[1], bias_frag[4 * ld + 2] = v[2], bias_frag[4 * ld + 3] = v[3];
 			}
-		} else if constexpr(DIRECT) {
+		} else if constexpr(DIRECT || STAGED) {
 			typedef __attribute__((ext_vector_type(2))) unsigned short u16x2;
 			const u16x2 lim = {(unsigned short)0xC780, (unsigned short)0xC780};
+			if constexpr(STAGED) {  // this lane's four 8-byte pieces, keys 8 ld + 4 half .. + 3 of row n: chunk ld at its swizzled place
+#pragma unroll
+				for(int ld = 0; ld < 4; ld++)
+					braw[ld] = *reinterpret_cast<const u32x2*>(smem + SLOT_BASE + wave * 4096 + (t_next & 1) * 2048 + n * 64 + ((ld ^ ((n >> 2) & 3)) << 4) + half * 8);
+			}
 #pragma unroll
 			for(int ld = 0; ld < 4; ld++)
 #pragma unroll
@@ -554,8 +589,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 						constexpr int S = decltype(s_c)::value;
 						if constexpr(S == 1) {
 							load_tile(t + 2, bufnn);
-							next_bias_fragment();
+							next_bias_fragment(t + 1);
 							load_bias_direct(t + 2);
+							load_bias_staged(t + 2);   // (into the half that held fragment t, read a tile ago)
 						}
 					});
 				} else if constexpr(R == ROWS - 1) {
@@ -574,11 +610,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 		constexpr bool ANYDROP = decltype(anydrop_c)::value != 0;
 		// ---- prologue: the second tile and bias fragment, S^T of the first step, K fragments of the second ----
 		// (tile 0 and bias fragment 0 were requested at the top of the kernel and are complete)
-		next_bias_fragment();  // fragment 0 -> registers
+		next_bias_fragment(0);  // fragment 0 -> registers
 		asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 		load_tile(1, BUF_R);
 		load_bias(1);
 		load_bias_direct(1);
+		load_bias_staged(1);
 		{
 			f32x16 s0;
 #pragma unroll
@@ -659,13 +696,18 @@ bool direct_bias_ok(const af3_dpa_params& p) {
 		   ((p.L - 1) * p.bias_stride[1] + p.L) * 2 < 0x40000000LL;
 }
 
-// 0 = no bias, 1 = through the rewritten workspace, 2 = read in place, -1 = this kernel cannot serve the call.  The
+// ... and through LDS, in whole 16-byte chunks of whole rows, when rows start on 16-byte boundaries and keys come in groups of eight.
+bool staged_bias_ok(const af3_dpa_params& p) {
+	return direct_bias_ok(p) && p.L % 8 == 0 && (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0 && p.bias_stride[0] % 8 == 0 && p.bias_stride[1] % 8 == 0;
+}
+
+// 0 = no bias, 1 = through the rewritten workspace, 2 = read in place (3: through LDS), -1 = this kernel cannot serve the call.  The
 // rewrite costs three passes over the bias and pays off from four groups of batch rows on.
 int rows_bias_mode(const af3_dpa_params& p) {
 	if(!p.bias) return 0;
 	const bool ws_ok = p.workspace && p.workspace_bytes >= rows_ws_bytes(p) && (reinterpret_cast<uintptr_t>(p.workspace) & 15) == 0;
 	if(p.B >= 16 && ws_ok) return 1;
-	if(direct_bias_ok(p)) return 2;
+	if(direct_bias_ok(p)) return staged_bias_ok(p) ? 3 : 2;
 	return ws_ok ? 1 : -1;
 }
 
@@ -676,7 +718,7 @@ int launch_rows(const af3_dpa_params& p, int64_t b_first, int64_t b_count, hipSt
 	const int64_t blocks   = ((n_groups + 7) / 8) * 8 * n_qtiles;
 	if(blocks <= 0 || blocks > 0x7fffffffLL) return AF3_ERR_BAD_SHAPE;
 	const size_t n_t_all = (size_t)((p.L + KT_R - 1) / KT_R);
-	const size_t smem    = (size_t)NBUF_R * ROWS * 2 * TILE_R + (BMODE == 1 ? 4 * 4096 : 0) + (n_t_all + 1) * ROWS * 32 * 2;
+	const size_t smem    = (size_t)NBUF_R * ROWS * 2 * TILE_R + (BMODE == 1 || BMODE == 3 ? 4 * 4096 : 0) + (n_t_all + 1) * ROWS * 32 * 2;
 	auto         kern    = dpa_rows_bf16_kernel<ROWS, BMODE>;
 	if(smem > 64 * 1024) {
 		if(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return AF3_ERR_LAUNCH;
@@ -709,15 +751,13 @@ int64_t mfma_rows_workspace_bytes(const af3_dpa_params& p) {
 
 bool mfma_rows_can_serve(const af3_dpa_params& p) { return mfma_rows_eligible(p) && rows_bias_mode(p) >= 0; }
 
-// A few batch rows that share a large bias of long rows: the one-row kernel's workspace rewrite is a pass over the whole
-// bias (read 2 bytes, write 2 bytes per entry: 23 us for 16 x 1536 x 1536) that no row of the batch amortises, while this
-// kernel reads the bias in place once per group of rows.  Measured on B x 16 x 1536 x 24 (one-row kernel with its rewrite
-// against this one): B = 2 61 / 53 us, 3 78 / 62 us, 5 79 / 75 us; with a 19 MB bias (5 x 16 x 768 x 24) 33 / 34 us, with a
-// 34 MB one (8 x 4 x 2048 x 32) 63 / 68 us; five samples through the fused caller (strided q, k, v, gate) 81 / 83 us of GPU
-// time: taken for up to four batch rows from 64 MB on.
-bool mfma_rows_saves_a_large_rewrite(const af3_dpa_params& p) {
-	return p.bias && p.B <= 4 && p.L >= 1024 && p.H * p.L * p.L * 2 >= (int64_t)64 << 20 && direct_bias_ok(p);
-}
+// Fewer than 16 batch rows whose bias this kernel can stage in place: the one-row kernel would first rewrite the whole bias
+// into its workspace (a pass that so few rows do not amortise) and then stream the rewritten copy once per row; here each
+// group of rows streams the original once.  Measured (one-row kernel with its rewrite / this kernel, us): 2 x 16 x 1536 x 24
+// 61 / 38, 5 x 16 x 1536 x 24 79 / 67, 12 x 16 x 1536 x 24 139 / 109, 5 x 16 x 768 x 24 32 / 28, 8 x 4 x 2048 x 32 62 / 50,
+// 12 x 4 x 384 x 32 21 / 17, 8 x 4 x 768 x 32 21 / 21.  (From 16 rows on this kernel goes through its own workspace and needs
+// the larger launches: 16 x 4 x 768 x 32 26 / 32.)
+bool mfma_rows_suits_a_small_batch(const af3_dpa_params& p) { return p.bias && p.B < 16 && staged_bias_ok(p); }
 
 int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
 	const int mode = rows_bias_mode(p);
@@ -795,7 +835,7 @@ int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
 	int64_t done = 0;
 	for(int i = 0; i < 3; i++) {
 		if(count[i] == 0) continue;
-		const int rc = mode == 0 ? launch_rows_n<0>(rows_of[i], p, done, count[i], s) : mode == 1 ? launch_rows_n<1>(rows_of[i], p, done, count[i], s) : launch_rows_n<2>(rows_of[i], p, done, count[i], s);
+		const int rc = mode == 0 ? launch_rows_n<0>(rows_of[i], p, done, count[i], s) : mode == 1 ? launch_rows_n<1>(rows_of[i], p, done, count[i], s) : mode == 2 ? launch_rows_n<2>(rows_of[i], p, done, count[i], s) : launch_rows_n<3>(rows_of[i], p, done, count[i], s);
 		if(rc != AF3_OK) return rc;
 		done += count[i];
 	}

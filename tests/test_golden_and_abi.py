@@ -380,7 +380,8 @@ def test_static_scratch_entry_point_rejects_calls_beyond_its_limit_on_the_host()
     assert fwd(ctypes.byref(_params(L=0)), None) == -3
     L = 2048
     st = (ctypes.c_int64 * 3)(4 * L * 32, L * 32, 32)
-    big = _params(B=2, H=4, L=L, bias=0x1000, bias_stride=(ctypes.c_int64 * 2)(L * L, L), q_stride=st, k_stride=st, v_stride=st, out_stride=st)
+    # (a bias whose rows are only 8-byte aligned: a call with so few batch rows would otherwise read it in place, without scratch)
+    big = _params(B=2, H=4, L=L, bias=0x1008, bias_stride=(ctypes.c_int64 * 2)(L * L, L), q_stride=st, k_stride=st, v_stride=st, out_stride=st)
     assert need(ctypes.byref(big)) > _lib.STATIC_SCRATCH_BYTES
     assert fwd(ctypes.byref(big), None) == -9
     assert b"scratch" in lib.af3_status_string(-9)

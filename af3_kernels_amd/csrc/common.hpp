@@ -70,7 +70,7 @@ int launch_dpa_mfma_fp8(const af3_dpa_params& p, hipStream_t s);
 bool mfma_rows_eligible(const af3_dpa_params& p);
 bool mfma_rows_can_serve(const af3_dpa_params& p);   // eligible, and its bias can be served (workspace given, or readable in place)
 int64_t mfma_rows_workspace_bytes(const af3_dpa_params& p);
-bool mfma_rows_suits_a_small_batch(const af3_dpa_params& p);  // fewer than 16 batch rows and a bias that this kernel stages in place
+bool mfma_rows_suits_a_small_batch(const af3_dpa_params& p);  // fewer than 128 batch rows and a bias that this kernel stages in place
 int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s);
 bool mfma_bf16_eligible(const af3_dpa_params& p);
 int64_t mfma_bf16_workspace_bytes(const af3_dpa_params& p);

@@ -1166,7 +1166,7 @@ static int64_t ws_bytes_needed(const af3_dpa_params& p) {
 
 // Whether the call goes to the kernel of dpa_mfma_rows.hip (four batch rows per wavefront sharing each bias tile): its
 // shape limits, enough workgroups of four-row groups to give every compute unit one (smaller launches through its workspace
-// do better with this file's variants: 16 x 4 x 768 x 32 26 us here against 32 us there) or fewer than 16 batch rows whose
+// do better with this file's variants: 16 x 4 x 768 x 32 26 us here against 32 us there) or fewer than 128 batch rows whose
 // bias it can stage in place, and the caller's hint (af3_dpa_params.reserved: 1 = take it whenever the shape allows, 2 = never).
 static bool rows_kernel_wanted(const af3_dpa_params& p) {
 	if(p.reserved == 2 || !mfma_rows_eligible(p)) return false;

@@ -701,11 +701,16 @@ bool staged_bias_ok(const af3_dpa_params& p) {
 	return direct_bias_ok(p) && p.L % 8 == 0 && (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0 && p.bias_stride[0] % 8 == 0 && p.bias_stride[1] % 8 == 0;
 }
 
-// 0 = no bias, 1 = through the rewritten workspace, 2 = read in place (3: through LDS), -1 = this kernel cannot serve the call.  The
-// rewrite costs three passes over the bias and pays off from four groups of batch rows on.
+// Staging the bf16 bias costs each step 8 vector instructions (widening it) that the fp32 workspace does not, the workspace
+// a prepass over the whole bias and twice the bytes per tile: the workspace pays off from about 128 batch rows on (staged /
+// workspace, us: 32 x 16 x 1536 x 24 245 / 299, 64 x 4 x 768 x 32 50 / 55, 128 x 4 x 768 x 32 90 / 91, 192 x 4 x 768 x 32 117 / 118).
+constexpr int64_t STAGED_MAX_B = 128;
+
+// 0 = no bias, 1 = through the rewritten workspace, 2 = read in place (3: through LDS), -1 = this kernel cannot serve the call.
 int rows_bias_mode(const af3_dpa_params& p) {
 	if(!p.bias) return 0;
 	const bool ws_ok = p.workspace && p.workspace_bytes >= rows_ws_bytes(p) && (reinterpret_cast<uintptr_t>(p.workspace) & 15) == 0;
+	if(p.B < STAGED_MAX_B && staged_bias_ok(p)) return 3;
 	if(p.B >= 16 && ws_ok) return 1;
 	if(direct_bias_ok(p)) return staged_bias_ok(p) ? 3 : 2;
 	return ws_ok ? 1 : -1;
@@ -745,19 +750,19 @@ bool mfma_rows_eligible(const af3_dpa_params& p) {
 // Workspace the call would use: none when the bias is better read in place (few batch rows).
 int64_t mfma_rows_workspace_bytes(const af3_dpa_params& p) {
 	if(!p.bias) return 0;
-	if(p.B < 16 && direct_bias_ok(p)) return 0;
+	if((p.B < STAGED_MAX_B && staged_bias_ok(p)) || (p.B < 16 && direct_bias_ok(p))) return 0;
 	return rows_ws_bytes(p);
 }
 
 bool mfma_rows_can_serve(const af3_dpa_params& p) { return mfma_rows_eligible(p) && rows_bias_mode(p) >= 0; }
 
-// Fewer than 16 batch rows whose bias this kernel can stage in place: the one-row kernel would first rewrite the whole bias
+// Fewer than 128 batch rows whose bias this kernel can stage in place: the one-row kernel would first rewrite the whole bias
 // into its workspace (a pass that so few rows do not amortise) and then stream the rewritten copy once per row; here each
 // group of rows streams the original once.  Measured (one-row kernel with its rewrite / this kernel, us): 2 x 16 x 1536 x 24
 // 61 / 38, 5 x 16 x 1536 x 24 79 / 67, 12 x 16 x 1536 x 24 139 / 109, 5 x 16 x 768 x 24 32 / 28, 8 x 4 x 2048 x 32 62 / 50,
-// 12 x 4 x 384 x 32 21 / 17, 8 x 4 x 768 x 32 21 / 21.  (From 16 rows on this kernel goes through its own workspace and needs
-// the larger launches: 16 x 4 x 768 x 32 26 / 32.)
-bool mfma_rows_suits_a_small_batch(const af3_dpa_params& p) { return p.bias && p.B < 16 && staged_bias_ok(p); }
+// 12 x 4 x 384 x 32 21 / 17, 8 x 4 x 768 x 32 21 / 21, 16 x 4 x 768 x 32 26 / 22, 48 x 4 x 768 x 32 45 / 40,
+// 16 x 16 x 1536 x 24 172 / 149, 40 x 4 x 384 x 32 22 / 18.
+bool mfma_rows_suits_a_small_batch(const af3_dpa_params& p) { return p.bias && p.B < STAGED_MAX_B && staged_bias_ok(p); }
 
 int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
 	const int mode = rows_bias_mode(p);

@@ -761,8 +761,13 @@ bool mfma_rows_can_serve(const af3_dpa_params& p) { return mfma_rows_eligible(p)
 // group of rows streams the original once.  Measured (one-row kernel with its rewrite / this kernel, us): 2 x 16 x 1536 x 24
 // 61 / 38, 5 x 16 x 1536 x 24 79 / 67, 12 x 16 x 1536 x 24 139 / 109, 5 x 16 x 768 x 24 32 / 28, 8 x 4 x 2048 x 32 62 / 50,
 // 12 x 4 x 384 x 32 21 / 17, 8 x 4 x 768 x 32 21 / 21, 16 x 4 x 768 x 32 26 / 22, 48 x 4 x 768 x 32 45 / 40,
-// 16 x 16 x 1536 x 24 172 / 149, 40 x 4 x 384 x 32 22 / 18.
-bool mfma_rows_suits_a_small_batch(const af3_dpa_params& p) { return p.bias && p.B < STAGED_MAX_B && staged_bias_ok(p); }
+// 16 x 16 x 1536 x 24 172 / 149, 40 x 4 x 384 x 32 22 / 18.  Not for long rows in so few workgroups that most compute units
+// would stay empty (2 x 4 x 1536 x 32: 48 workgroups, 30 / 37 us: the one-row kernel splits the key axis of such rows).
+bool mfma_rows_suits_a_small_batch(const af3_dpa_params& p) {
+	if(!p.bias || p.B >= STAGED_MAX_B || !staged_bias_ok(p)) return false;
+	const int64_t wgs = ((p.B + 3) / 4) * p.H * ((p.L + 127) / 128);
+	return wgs >= 64 || p.L < 1024;
+}
 
 int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
 	const int mode = rows_bias_mode(p);

@@ -113,34 +113,53 @@ def print_debug_thread_imbalance():
 # ------------------------------------------------------------------------------------------
 # attention
 # ------------------------------------------------------------------------------------------
+_PARAM_TEMPLATES = {}   # layout of a call (shapes, strides, dtypes, flags) -> bytes of an af3_dpa_params block with everything but the addresses
+
+
 def _fill_params(q, k, v, keep, bias, out, mma_dtype, force_generic, descales=None, softmax_scale=None, v_transposed=False, gate=None) -> DpaParams:
-    B, H, L, D = q.shape
-    p = DpaParams()
+    """The argument block of one call.  Everything that depends on the layout alone is filled once per layout and copied
+    from a byte template afterwards (building the ctypes arrays anew costs more host time than a small call's kernel runs);
+    only the addresses are set per call."""
+    key = (q.shape, q.stride(), k.stride(), v.stride(), out.stride(), q.dtype, out.dtype, mma_dtype, bool(force_generic), _rows_kernel_hint, softmax_scale,
+           None if bias is None else (bias.stride(0), bias.stride(1), bias.dtype),
+           None if keep is None else (keep.shape[0], keep.stride(0)),
+           None if gate is None else gate.stride())
+    template = _PARAM_TEMPLATES.get(key)
+    if template is None:
+        B, H, L, D = q.shape
+        t = DpaParams()
+        t.B, t.H, t.L, t.D = B, H, L, D
+        t.q_stride = (ctypes.c_int64 * 3)(*q.stride()[:3])
+        t.k_stride = (ctypes.c_int64 * 3)(*k.stride()[:3])
+        t.v_stride = (ctypes.c_int64 * 3)(*v.stride()[:3])
+        t.out_stride = (ctypes.c_int64 * 3)(*out.stride()[:3])
+        if bias is not None:
+            t.bias_stride = (ctypes.c_int64 * 2)(bias.stride(0), bias.stride(1))
+            t.bias_dtype = _DTYPE_CODE[bias.dtype]
+        if keep is not None:
+            t.key_mask_stride_b = 0 if keep.shape[0] == 1 else keep.stride(0)
+        t.io_dtype = _DTYPE_CODE[q.dtype]
+        t.out_dtype = _DTYPE_CODE[out.dtype]
+        t.mma_dtype = mma_dtype
+        t.softmax_scale = float(D) ** -0.5 if softmax_scale is None else softmax_scale
+        t.q_descale = t.k_descale = t.v_descale = 1.0
+        t.force_generic = int(bool(force_generic))
+        t.reserved = _rows_kernel_hint
+        if gate is not None:
+            t.gate_stride = (ctypes.c_int64 * 3)(*gate.stride()[:3])
+        if len(_PARAM_TEMPLATES) >= 256:
+            _PARAM_TEMPLATES.clear()
+        template = _PARAM_TEMPLATES[key] = bytes(t)
+    p = DpaParams.from_buffer_copy(template)
     p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
-    p.B, p.H, p.L, p.D = B, H, L, D
-    p.q_stride = (ctypes.c_int64 * 3)(*q.stride()[:3])
-    p.k_stride = (ctypes.c_int64 * 3)(*k.stride()[:3])
-    p.v_stride = (ctypes.c_int64 * 3)(*v.stride()[:3])
-    p.out_stride = (ctypes.c_int64 * 3)(*out.stride()[:3])
     if bias is not None:
         p.bias = bias.data_ptr()
-        p.bias_stride = (ctypes.c_int64 * 2)(bias.stride(0), bias.stride(1))
-        p.bias_dtype = _DTYPE_CODE[bias.dtype]
     if keep is not None:
         p.key_mask = keep.data_ptr()
-        p.key_mask_stride_b = 0 if keep.shape[0] == 1 else keep.stride(0)
-    p.io_dtype = _DTYPE_CODE[q.dtype]
-    p.out_dtype = _DTYPE_CODE[out.dtype]
-    p.mma_dtype = mma_dtype
-    p.softmax_scale = float(D) ** -0.5 if softmax_scale is None else softmax_scale
-    p.q_descale = p.k_descale = p.v_descale = 1.0
-    p.force_generic = int(bool(force_generic))
-    p.reserved = _rows_kernel_hint
     if descales is not None:
         p.device_descales = descales.data_ptr()
     if gate is not None:
         p.gate = gate.data_ptr()
-        p.gate_stride = (ctypes.c_int64 * 3)(*gate.stride()[:3])
     return p
 
 
@@ -293,10 +312,16 @@ def dot_product_attention_cpp(
         raise ValueError(f"unsupported dtype {q.dtype}: float32 or bfloat16 (use dot_product_attention_fp8 for the fp8 path)")
     dtype = q.dtype
     keep = _lift_mask(mask, q.shape[2]) if mask is not None else None
-    bias = bias.to(dtype) if bias is not None else None
+    # (a cast to the dtype a tensor already has returns the tensor, but the call alone costs a microsecond of a 20-us call)
+    if bias is not None and bias.dtype != dtype:
+        bias = bias.to(dtype)
+    if k.dtype != dtype:
+        k = k.to(dtype)
+    if v.dtype != dtype:
+        v = v.to(dtype)
     # (straight into the implementation: the registered op torch.ops.af3_kernels.dpa_forward is the same function
     # behind torch's dispatcher, whose per-call cost is comparable to a small attention kernel)
-    return _dpa_forward_impl(q, k.to(dtype), v.to(dtype), keep, bias, code, False)
+    return _dpa_forward_impl(q, k, v, keep, bias, code, False)
 
 
 def selected_kernel(q, k, v, mask, bias, force_generic=False) -> str:

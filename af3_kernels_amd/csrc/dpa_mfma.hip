@@ -149,7 +149,11 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 	constexpr int  LDS_SETS   = SPLIT ? NW : 1;  // private K/V buffer sets
 	constexpr bool BIAS_F32   = BMODE == 1;      // natural variant, bias stored as fp32, read in place
 	constexpr bool BRING      = BMODE == 2;      // natural variant, bf16 bias streamed through a per-wavefront LDS ring
-	constexpr int  NBUF       = LOADERS ? 4 : 3;  // tile buffers of the K/V ring and slots of a bias ring (with loading wavefronts: loads run two tiles ahead)
+	// tile buffers of the K/V ring and slots of a bias ring.  With loading wavefronts the loads run two tiles ahead; KS2 in
+	// addition has every tile in LDS one barrier before its first use, so that a stage's LDS operands are fetched at the end of
+	// the stage before it (AHEAD: the tile that has landed when iteration j passes its barrier is j + AHEAD).
+	constexpr int  AHEAD      = KS2 ? 2 : 1;
+	constexpr int  NBUF       = LOADERS ? AHEAD + 3 : 3;
 	constexpr int  RING_BYTES = BRING ? (KS2 ? NW / 2 : NW) * NBUF * 4096 : 0;  // (KS2: one ring per pair of wavefronts)
 	constexpr int  MASK_BASE  = LDS_SETS * 2 * NBUF * TILE_BYTES + RING_BYTES;
 	static_assert(!(L2DOM && BMODE != 0), "the log2 variant reads its bias from the workspace");
@@ -443,18 +447,20 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 			}
 			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 			__syncthreads();  // (tiles 0 and 1 are in LDS)
-			if(nlive > 2) {
-				load_tile(walk(2), 2);
-				load_bias_tile(walk(2), 2);
-			}
+#pragma unroll
+			for(int j = 2; j <= AHEAD + 1; j++)
+				if(j < nlive) {
+					load_tile(walk(j), j);
+					load_bias_tile(walk(j), j);
+				}
 			for(int it = 0; it < nlive; it++) {
-				// tile it + 1 has landed (tile it + 2, if there is one, may still be on its way)
-				if(it + 2 < nlive) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_TILE) : "memory");
+				// tile it + AHEAD has landed (the tile behind it, if there is one, may still be on its way)
+				if(it + AHEAD + 1 < nlive) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_TILE) : "memory");
 				else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-				__syncthreads();  // (every wavefront is done with tile it - 1, whose buffer tile it + 3 takes)
-				if(it + 3 < nlive) {
-					load_tile(walk(it + 3), (it + 3) % NBUF);
-					load_bias_tile(walk(it + 3), (it + 3) % NBUF);
+				__syncthreads();  // (every wavefront is done with tile it - 1, whose buffer tile it + AHEAD + 2 takes)
+				if(it + AHEAD + 2 < nlive) {
+					load_tile(walk(it + AHEAD + 2), (it + AHEAD + 2) % NBUF);
+					load_bias_tile(walk(it + AHEAD + 2), (it + AHEAD + 2) % NBUF);
 				}
 			}
 			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -866,14 +872,24 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 			for(int c2 = 0; c2 < 2; c2++) bfrag[2 * SUB + c2] = bias_frag_finite(*reinterpret_cast<const u32x4*>(bring + slot_off + (b_rd ^ ((4 * SUB + 2 * c2) << 4))));
 		};
 		// ring_off (BRING): byte offset of the ring slot that holds the bias tile of sub-tile j+1
-		auto stage = [&](auto subn_c, int k_off, int mask_addr_next, int v_off, auto subc_c, int bias_kt, auto bias_sub_c, int ring_off) {
-			constexpr int SUBN = decltype(subn_c)::value, SUBC = decltype(subc_c)::value, FB = 2 * SUBN;
+		// The LDS operands of S^T(j+1): K fragments, bias fragments (ring variants), mask entries.  KS2 fetches them at the end of
+		// the stage before (every tile is in LDS one barrier early there), so that their latency hides behind that stage's
+		// row-sum check instead of standing in front of this stage's first matrix instruction: a lone wavefront has nothing
+		// else to run in that time.
+		u32x4    kf[NC];
+		uint32_t mask_next = 0;
+		auto fetch_operands = [&](auto subn_c, int k_off, int mask_addr_next, int ring_off) {
+			constexpr int SUBN = decltype(subn_c)::value;
 			if(BRING) read_bias_ring(ring_off, subn_c);
-			// operands of S^T(j+1) from LDS
-			u32x4 kf[NC];
 #pragma unroll
 			for(int c = 0; c < NC; c++) kf[c] = read_kfrag(k_off, SUBN, c);
-			maskA[0] = *reinterpret_cast<const uint32_t*>(smem + mask_addr_next + SUBN * 32 * 4);
+			mask_next = *reinterpret_cast<const uint32_t*>(smem + mask_addr_next + SUBN * 32 * 4);
+		};
+		// k_next / mask_next_addr / ring_next (KS2): where the operands of the stage after this one are
+		auto stage = [&](auto subn_c, int k_off, int mask_addr_next, int v_off, auto subc_c, int bias_kt, auto bias_sub_c, int ring_off, int k_next, int mask_next_addr, int ring_next) {
+			constexpr int SUBN = decltype(subn_c)::value, SUBC = decltype(subc_c)::value, FB = 2 * SUBN;
+			if constexpr(!KS2) fetch_operands(subn_c, k_off, mask_addr_next, ring_off);
+			maskA[0] = mask_next;
 			u32x4  pcur[2];
 			f32x16 sn;
 #pragma unroll
@@ -922,6 +938,7 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 			AF3_CHUNK_END();
 #undef AF3_CHUNK_END
 			rowsum_mfma(pcur[1]);
+			if constexpr(KS2) fetch_operands(subn_c, k_next, mask_next_addr, ring_next);  // (this stage's have been consumed)
 			// The running sum stays below L * 2^REF_SLACK <= 2^25 while every probability respects the
 			// reference, so this also catches a single probability near or beyond the limit (inf, NaN).
 			if(__ballot(!(lacc[0] < PSUM_LIMIT))) {  // rare
@@ -964,33 +981,47 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 			if(BRING) read_bias_ring(0, ic<0>{});
 			sc = compute_s_plain(FUSED ? kt0 * TILE_BYTES : 0, 0, mask_rd + kt0 * mask_stride, 0);
 			rereference(sc, nullptr, true);
-			if(KS2) load_bias_frags(__builtin_amdgcn_readfirstlane(live_at(1)), ic<0>{});  // this wavefront's next sub-tile is in the next tile
-			else if(BIAS_LATE) load_bias_frags(kt0, ic<1>{});
+			if constexpr(KS2) {
+				const int kt1_first = __builtin_amdgcn_readfirstlane(live_at(1));
+				load_bias_frags(kt1_first, ic<0>{});                                                // this wavefront's next sub-tile is in the next tile
+				fetch_operands(ic<0>{}, TILE_BYTES, mask_rd + kt1_first * mask_stride, 4096);  // operands of the first stage: second tile of the walk, buffer 1
+			} else if(BIAS_LATE) load_bias_frags(kt0, ic<1>{});
 			else if(my_n > 1) load_bias_frags(__builtin_amdgcn_readfirstlane(live_at(1)), ic<0>{});
 
 			int buf = 0;  // LDS buffer of tile `it` (it % 3)
 			// tile indices of iterations it, it+1, it+2 are carried in scalar registers; the list entry for
 			// it+3 is fetched at the top of an iteration and only consumed at its end
 			int kt = kt0, kt1 = __builtin_amdgcn_readfirstlane(live_at(1)), kt2 = __builtin_amdgcn_readfirstlane(live_at(2));
+			if constexpr(KS2) {
+				// One stage per tile: this wavefront's 32 keys of tile `it` (exp, V fragments) and of tile it+1 (S^T).  Behind the
+				// barrier tile it+2 is in LDS (the loading wavefronts have waited for it) and everyone is done with tile it-1,
+				// whose buffer they now hand to tile it+4.
+				auto tile_step = [&](int it) {
+					const int bufn = buf == NBUF - 1 ? 0 : buf + 1, bufnn = bufn == NBUF - 1 ? 0 : bufn + 1;
+					__syncthreads();
+					const int kt3_v = live_at(it + 3);  // (behind the barrier, which would wait for this read)
+					stage(ic<0>{}, bufn * TILE_BYTES, mask_rd + kt1 * mask_stride, buf * TILE_BYTES, ic<0>{}, kt2, ic<0>{}, bufn * 4096, bufnn * TILE_BYTES, mask_rd + kt2 * mask_stride,
+						  bufnn * 4096);
+					buf = bufn;
+					kt  = kt1;
+					kt1 = kt2;
+					kt2 = __builtin_amdgcn_readfirstlane(kt3_v);
+				};
+				// two stages per trip, so that the score registers of consecutive stages swap roles instead of being copied
+				int it = 0;
+				for(; it + 1 < my_n; it += 2) {
+					tile_step(it);
+					tile_step(it + 1);
+				}
+				if(it < my_n) tile_step(it);
+			} else
 			for(int it = 0; it < my_n; it++) {
 				const int kt3_v = live_at(it + 3);
 				const int bufn = buf == NBUF - 1 ? 0 : buf + 1, bufnn = bufn == NBUF - 1 ? 0 : bufn + 1;
 				// LDS offsets of tile it and of tile it+1: ring buffers, or the tiles' own places when all of K and V is resident
 				const int off_cur = (FUSED ? kt : buf) * TILE_BYTES, off_next = (FUSED ? kt1 : bufn) * TILE_BYTES;
-				if constexpr(KS2) {
-					// One stage per tile: this wavefront's 32 keys of tile `it` (exp, V fragments) and of tile it+1 (S^T).  Behind
-					// the barrier tile it+1 is in LDS (the loader wavefront has waited for it) and everyone is done with tile
-					// it-1, whose buffer the loader now hands to tile it+3.
-					__syncthreads();
-					stage(ic<0>{}, off_next, mask_rd + kt1 * mask_stride, off_cur, ic<0>{}, kt2, ic<0>{}, bufn * 4096);
-					buf = bufn;
-					kt  = kt1;
-					kt1 = kt2;
-					kt2 = __builtin_amdgcn_readfirstlane(kt3_v);
-					continue;
-				}
 				// sub-tile (it, 0): next is (it, 1) in the same buffer
-				stage(ic<1>{}, off_cur, mask_rd + kt * mask_stride, off_cur, ic<0>{}, kt1, ic<0>{}, buf * 4096);
+				stage(ic<1>{}, off_cur, mask_rd + kt * mask_stride, off_cur, ic<0>{}, kt1, ic<0>{}, buf * 4096, 0, 0, 0);
 				if(!BIAS_LATE) load_bias_frags(kt1, ic<1>{});
 				// Tile it+1 (issued one iteration ago) must have landed, and every wavefront must be done
 				// with tile it-1, whose buffer tile it+2 is about to overwrite.  Loads complete in issue
@@ -1006,7 +1037,7 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 					load_bias_tile(kt2, bufnn);  // (its slot held tile it-1, last read in the stage above)
 				}
 				// sub-tile (it, 1): next is (it+1, 0) in the next buffer (harmless stale data after the last tile)
-				stage(ic<0>{}, off_next, mask_rd + kt1 * mask_stride, off_cur, ic<1>{}, kt1, ic<1>{}, bufn * 4096);
+				stage(ic<0>{}, off_next, mask_rd + kt1 * mask_stride, off_cur, ic<1>{}, kt1, ic<1>{}, bufn * 4096, 0, 0, 0);
 				if(!BIAS_LATE) load_bias_frags(kt2, ic<0>{});
 				buf = bufn;
 				kt  = kt1;
@@ -1206,7 +1237,7 @@ static size_t lds_bytes(const af3_dpa_params& p) {
 	const size_t n_ktiles = (size_t)((p.L + KT - 1) / KT);
 	constexpr bool   KS2  = KSL == 1;
 	const size_t writers  = SPLIT ? 1 : KS2 ? NW / 2 : NW;  // wavefronts that own a block of query rows
-	constexpr size_t NBUF = KSL ? 4 : 3;  // (as in the kernel)
+	constexpr size_t NBUF = KSL == 1 ? 5 : KSL ? 4 : 3;  // (as in the kernel)
 	return (size_t)(SPLIT ? NW : 1) * 2 * NBUF * KT * DP * 2 + (BMODE == 2 ? (KS2 ? NW / 2 : NW) * NBUF * 4096 : 0) + (n_ktiles * KT + 64) * 4 + n_ktiles * 2 + 16 +
 		   (p.gate ? writers * 32 * DP * 2 : 0);
 }

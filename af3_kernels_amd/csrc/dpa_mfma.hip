@@ -998,7 +998,11 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 				// whose buffer they now hand to tile it+4.
 				auto tile_step = [&](int it) {
 					const int bufn = buf == NBUF - 1 ? 0 : buf + 1, bufnn = bufn == NBUF - 1 ? 0 : bufn + 1;
-					__syncthreads();
+					// The barrier hands the buffer of tile it-1 back to the loading wavefronts, so this wavefront's reads of that
+					// tile must have returned; the operands fetched at the end of the stage before (the last OPERAND_READS LDS
+					// reads issued, from the buffer of tile it+1) may stay in flight.  LDS reads return in issue order.
+					constexpr int OPERAND_READS = NC + 1 + (BRING ? 2 : 0);
+					asm volatile("s_waitcnt lgkmcnt(%0)\n\ts_barrier" ::"n"(OPERAND_READS) : "memory");
 					const int kt3_v = live_at(it + 3);  // (behind the barrier, which would wait for this read)
 					stage(ic<0>{}, bufn * TILE_BYTES, mask_rd + kt1 * mask_stride, buf * TILE_BYTES, ic<0>{}, kt2, ic<0>{}, bufn * 4096, bufnn * TILE_BYTES, mask_rd + kt2 * mask_stride,
 						  bufnn * 4096);

@@ -182,6 +182,13 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 	// robin, so all query tiles of one (batch, head) are given ids that are congruent mod 8:
 	// they share that XCD's L2 copy of K and V, and an XCD only ever sees heads h = xcd % H
 	// (for H | 8), so its share of the bias stays L2-resident across the whole batch.
+	// The kernel arguments that the start of a workgroup needs, requested in one batch: left to itself the compiler fetches the
+	// two launch counts, waits, tests the early exit below, and only then requests the fields of p -- two memory latencies
+	// in a row, which every wavefront of a launch too small to hide them stands through.
+	asm volatile("" ::"s"(n_qtiles), "s"(n_groups), "s"(p.q), "s"(p.k), "s"(p.v), "s"(p.bias), "s"(p.key_mask), "s"(p.H), "s"(p.L), "s"(p.D), "s"(p.key_mask_stride_b),
+				 "s"(p.bias_stride[0]), "s"(p.bias_stride[1]));
+	asm volatile("" ::"s"(p.q_stride[0]), "s"(p.q_stride[1]), "s"(p.q_stride[2]), "s"(p.k_stride[0]), "s"(p.k_stride[1]), "s"(p.k_stride[2]), "s"(p.v_stride[0]), "s"(p.v_stride[1]),
+				 "s"(p.v_stride[2]));
 	const int64_t wg    = blockIdx.x;
 	const int     xcd   = (int)(wg & 7);
 	const int64_t slot  = wg >> 3;

@@ -46,6 +46,12 @@ __global__ void __launch_bounds__(F32_NW * 64) dpa_mfma_f32_kernel(af3_dpa_param
 
 	// workgroup -> (batch row, head, query tile); consecutive workgroups go round the 8 XCDs, so the
 	// query tiles of one (b, h) are kept on one XCD and share its L2 copy of K and V
+	// the kernel arguments that the start of a workgroup needs, requested in one batch (otherwise: the launch counts, a wait,
+	// the early exit, and only then the fields of p -- memory latencies in a row that a small launch cannot hide)
+	asm volatile("" ::"s"(n_qtiles), "s"(n_groups), "s"(p.q), "s"(p.k), "s"(p.v), "s"(p.bias), "s"(p.key_mask), "s"(p.H), "s"(p.L), "s"(p.D), "s"(p.key_mask_stride_b),
+				 "s"(p.bias_stride[0]), "s"(p.bias_stride[1]));
+	asm volatile("" ::"s"(p.q_stride[0]), "s"(p.q_stride[1]), "s"(p.q_stride[2]), "s"(p.k_stride[0]), "s"(p.k_stride[1]), "s"(p.k_stride[2]), "s"(p.v_stride[0]), "s"(p.v_stride[1]),
+				 "s"(p.v_stride[2]));
 	const int64_t wg    = blockIdx.x;
 	const int     xcd   = (int)(wg & 7);
 	const int64_t slot  = wg >> 3;

@@ -59,6 +59,12 @@ __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2
 	__shared__ int       s_nvalid, s_nlive;
 
 	// workgroup -> (batch, head, query tile), all query tiles of one (batch, head) on one XCD
+	// the kernel arguments that the start of a workgroup needs, requested in one batch (otherwise: the launch counts, a wait,
+	// the early exit, and only then the fields of p -- memory latencies in a row that a small launch cannot hide)
+	asm volatile("" ::"s"(n_qtiles), "s"(n_groups), "s"(p.q), "s"(p.k), "s"(p.v), "s"(p.bias), "s"(p.key_mask), "s"(p.H), "s"(p.L), "s"(p.D), "s"(p.key_mask_stride_b),
+				 "s"(p.bias_stride[0]), "s"(p.bias_stride[1]), "s"(p.device_descales), "s"(p.k_lo));
+	asm volatile("" ::"s"(p.q_stride[0]), "s"(p.q_stride[1]), "s"(p.q_stride[2]), "s"(p.k_stride[0]), "s"(p.k_stride[1]), "s"(p.k_stride[2]), "s"(p.v_stride[0]), "s"(p.v_stride[1]),
+				 "s"(p.v_stride[2]));
 	const int64_t wg    = blockIdx.x;
 	const int     xcd   = (int)(wg & 7);
 	const int64_t slot  = wg >> 3;

@@ -110,6 +110,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	// ---- workgroup -> (group of batch rows, head, query tile): all query tiles of one (group, head) get ids congruent
 	// mod 8, i.e. the same XCD (they share that XCD's L2 copy of K and V), and an XCD only sees heads xcd % H (for H | 8),
 	// so its share of the bias workspace stays L2-resident across the whole batch.
+	// The kernel arguments that the start of a workgroup needs, requested in one batch (the compiler would fetch the launch
+	// counts, wait, test the early exit, and only then request the fields of p, in two more batches: three memory latencies
+	// in a row that the wavefronts of a small launch stand through).
+	asm volatile("" ::"s"(n_qtiles), "s"(n_groups), "s"(b_first), "s"(b_count), "s"(p.q), "s"(p.k), "s"(p.v), "s"(p.bias), "s"(p.key_mask), "s"(p.workspace), "s"(p.H), "s"(p.L),
+				 "s"(p.D), "s"(p.key_mask_stride_b), "s"(p.bias_stride[0]), "s"(p.bias_stride[1]));
+	asm volatile("" ::"s"(p.q_stride[0]), "s"(p.q_stride[1]), "s"(p.q_stride[2]), "s"(p.k_stride[0]), "s"(p.k_stride[1]), "s"(p.k_stride[2]), "s"(p.v_stride[0]), "s"(p.v_stride[1]),
+				 "s"(p.v_stride[2]));
 	const int64_t wg    = blockIdx.x;
 	const int     xcd   = (int)(wg & 7);
 	const int64_t slot  = wg >> 3;

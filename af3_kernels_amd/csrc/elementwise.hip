@@ -227,7 +227,37 @@ __device__ __forceinline__ void quantize_e4m3_body(const void* __restrict__ src,
 			*reinterpret_cast<uint32_t*>(dst + (mat * cols + c) * dst_row_stride + ((int64_t)r4 << 2)) = w;
 			if(dst_lo) *reinterpret_cast<uint32_t*>(dst_lo + (mat * cols + c) * dst_row_stride + ((int64_t)r4 << 2)) = residual(f0, f1, f2, f3, w);
 		};
-		if(total < ((int64_t)1 << 31) && stride < ((int64_t)1 << 30)) {
+		if(SRC_BF16 && cols % 8 == 0 && src_row_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 && total < ((int64_t)1 << 31) && stride < ((int64_t)1 << 30)) {
+			// bf16 rows of whole 16-byte chunks: one thread = 4 consecutive rows x 8 consecutive columns (four 16-byte loads, eight
+			// 4-byte stores).  Consecutive lanes take consecutive row quads, so each store instruction of a wavefront writes 256
+			// consecutive bytes of one output row.
+			const uint32_t cb_n = (uint32_t)(cols >> 3), rq_u = (uint32_t)rq, items = (uint32_t)(n_mat * rq * (cols >> 3));
+			for(uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x; i < items; i += (uint32_t)stride) {
+				const uint32_t r4 = i % rq_u, cb = (i / rq_u) % cb_n;
+				const int64_t  mat = i / (rq_u * cb_n), r = mat * rows_per_matrix + ((int64_t)r4 << 2), left = rows_per_matrix - ((int64_t)r4 << 2);
+				u32x4          w[4];
+#pragma unroll
+				for(int k = 0; k < 4; k++) {
+					w[k] = u32x4{0u, 0u, 0u, 0u};
+					if(left > k) w[k] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(src) + (r + k) * src_row_stride + (cb << 3));
+				}
+				uint8_t* const d0 = dst + (mat * cols + (cb << 3)) * dst_row_stride + ((int64_t)r4 << 2);
+#pragma unroll
+				for(int j = 0; j < 8; j++) {
+					float f[4];
+#pragma unroll
+					for(int k = 0; k < 4; k++) {
+						const float x = bf16_bits_to_f32((j & 1) ? (w[k][j >> 1] >> 16) : (w[k][j >> 1] & 0xffffu));
+						f[k]          = left > k ? fminf(fmaxf(x * mul, -448.f), 448.f) : 0.f;
+					}
+					uint32_t o = 0;
+					o = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], o, false);
+					o = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], o, true);
+					*reinterpret_cast<uint32_t*>(d0 + j * dst_row_stride) = o;
+					if(dst_lo) *reinterpret_cast<uint32_t*>(dst_lo + (d0 - dst) + j * dst_row_stride) = residual(f[0], f[1], f[2], f[3], o);
+				}
+			}
+		} else if(total < ((int64_t)1 << 31) && stride < ((int64_t)1 << 30)) {
 			for(uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x; i < (uint32_t)total; i += (uint32_t)stride) element(i, (uint32_t)cols, (uint32_t)rq);
 		} else {
 			for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += stride) element(i, cols, rq);
@@ -388,7 +418,9 @@ extern "C" int af3_quantize_qkv_fp8_e4m3(const void* q, const void* k, const voi
 	qa.dst_lo[0] = static_cast<uint8_t*>(q_lo), qa.dst_lo[1] = static_cast<uint8_t*>(k_lo), qa.dst_lo[2] = nullptr;
 	qa.rows = B * H * L, qa.cols = D, qa.rows_per_matrix = L, qa.v_row_stride = v8t_row_stride;
 	qa.pre_scale[0] = q_pre_scale, qa.pre_scale[1] = qa.pre_scale[2] = 1.f;
-	const dim3 ga(AMAX3_BLOCKS, 3), gq(ew_blocks(n / 4, 2048), 3);
+	// (quantise: a thread of the dense paths takes 8 elements per trip; two trips per thread, so that the three tensors'
+	// workgroups -- each of which first folds its tensor's partial maxima -- are all resident at once for the usual sizes)
+	const dim3 ga(AMAX3_BLOCKS, 3), gq(ew_blocks(n / 32, 1024), 3);
 	if(sd == AF3_F32) {
 		hipLaunchKernelGGL(amax3_kernel<false>, ga, dim3(EW_THREADS), 0, s, aa, scratch);
 		hipLaunchKernelGGL(quantize3_kernel<false>, gq, dim3(EW_THREADS), 0, s, qa, scratch, descales);

@@ -671,6 +671,19 @@ def test_quantize_fp8_per_tensor_scale(af3, dtype):
     assert d2.item() == 1.0 / scale1
 
 
+@pytest.mark.parametrize("shape", [(2, 2, 37, 24), (1, 3, 5, 8), (2, 1, 130, 48), (1, 2, 64, 20)], ids=str)
+def test_quantize_fp8_transposed_ragged_rows(af3, shape):
+    """Transposed e4m3 of bf16 rows whose count is no multiple of four (the last row quad of a matrix is partly padding),
+    with head sizes of whole 16-byte chunks (the 4-rows-by-8-columns path) and one that is not."""
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (torch.randn(*shape, generator=g) * 2).to(torch.bfloat16)
+    t8, d = af3.quantize_fp8_e4m3(x.cuda(), transpose_last2=True)
+    scale = 2.0 ** np.floor(np.log2(448.0 / x.float().abs().max().item()))
+    want = (x.float() * scale).clamp(-448, 448).to(torch.float8_e4m3fn).transpose(-1, -2).contiguous()
+    assert t8.shape == want.shape and d.item() == 1.0 / scale
+    assert torch.equal(t8.cpu().contiguous().view(torch.uint8), want.view(torch.uint8))
+
+
 def test_pad_and_vnni_repack(af3, oracle):
     x = torch.arange(2 * 3 * 5, dtype=torch.float32).reshape(2, 3, 5).cuda()
     y = af3.pad_and_align_tensor(x, (2, 4, 8), True, 1.0)

@@ -708,16 +708,24 @@ bool staged_bias_ok(const af3_dpa_params& p) {
 	return direct_bias_ok(p) && p.L % 8 == 0 && (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0 && p.bias_stride[0] % 8 == 0 && p.bias_stride[1] % 8 == 0;
 }
 
-// Staging the bf16 bias costs each step 8 vector instructions (widening it) that the fp32 workspace does not, the workspace
-// a prepass over the whole bias and twice the bytes per tile: the workspace pays off from about 128 batch rows on (staged /
-// workspace, us: 32 x 16 x 1536 x 24 245 / 299, 64 x 4 x 768 x 32 50 / 55, 128 x 4 x 768 x 32 90 / 91, 192 x 4 x 768 x 32 117 / 118).
-constexpr int64_t STAGED_MAX_B = 128;
+// Staging the bf16 bias costs each step 8 vector instructions (widening it) that the fp32 workspace does not -- about 5 % of
+// the kernel's time -- the workspace a prepass over the whole bias (about 3 us + 0.46 us per MB read and written) and twice
+// the bytes per tile.  Staged / workspace, us, prepass included: 32 x 16 x 1536 x 24 245 / 299, 64 x 4 x 768 x 32 50 / 55,
+// 128 x 4 x 768 x 32 90 / 91, 192 x 4 x 768 x 32 117 / 118, 384 x 4 x 384 x 32 60 / 62, 768 x 4 x 768 x 32 425 / 416.
+// The prepass is worth its time from about 224 + 2.4e8 / (H L^2) batch rows on (the second term: its fixed cost against the
+// time of one batch row).
+constexpr int64_t STAGED_MAX_B_SMALL = 128;  // below this the kernel is taken for launches the one-row kernel would otherwise serve
+static bool staged_preferred(const af3_dpa_params& p) {
+	if(!staged_bias_ok(p)) return false;
+	const double x = (double)p.H * (double)p.L * (double)p.L;
+	return (double)p.B < 224.0 + 2.44e8 / x;
+}
 
 // 0 = no bias, 1 = through the rewritten workspace, 2 = read in place (3: through LDS), -1 = this kernel cannot serve the call.
 int rows_bias_mode(const af3_dpa_params& p) {
 	if(!p.bias) return 0;
 	const bool ws_ok = p.workspace && p.workspace_bytes >= rows_ws_bytes(p) && (reinterpret_cast<uintptr_t>(p.workspace) & 15) == 0;
-	if(p.B < STAGED_MAX_B && staged_bias_ok(p)) return 3;
+	if(staged_preferred(p)) return 3;
 	if(p.B >= 16 && ws_ok) return 1;
 	if(direct_bias_ok(p)) return staged_bias_ok(p) ? 3 : 2;
 	return ws_ok ? 1 : -1;
@@ -757,7 +765,7 @@ bool mfma_rows_eligible(const af3_dpa_params& p) {
 // Workspace the call would use: none when the bias is better read in place (few batch rows).
 int64_t mfma_rows_workspace_bytes(const af3_dpa_params& p) {
 	if(!p.bias) return 0;
-	if((p.B < STAGED_MAX_B && staged_bias_ok(p)) || (p.B < 16 && direct_bias_ok(p))) return 0;
+	if(staged_preferred(p) || (p.B < 16 && direct_bias_ok(p))) return 0;
 	return rows_ws_bytes(p);
 }
 
@@ -771,7 +779,7 @@ bool mfma_rows_can_serve(const af3_dpa_params& p) { return mfma_rows_eligible(p)
 // 16 x 16 x 1536 x 24 172 / 149, 40 x 4 x 384 x 32 22 / 18.  Not for long rows in so few workgroups that most compute units
 // would stay empty (2 x 4 x 1536 x 32: 48 workgroups, 30 / 37 us: the one-row kernel splits the key axis of such rows).
 bool mfma_rows_suits_a_small_batch(const af3_dpa_params& p) {
-	if(!p.bias || p.B >= STAGED_MAX_B || !staged_bias_ok(p)) return false;
+	if(!p.bias || p.B >= STAGED_MAX_B_SMALL || !staged_bias_ok(p)) return false;
 	const int64_t wgs = ((p.B + 3) / 4) * p.H * ((p.L + 127) / 128);
 	return wgs >= 64 || p.L < 1024;
 }

@@ -142,8 +142,9 @@ typedef struct af3_dpa_params {
 int af3_dpa_forward(const af3_dpa_params* params, void* hip_stream);
 
 /* Bytes of workspace the call would use (0 when a workspace would not help, e.g. B == 1,
- * no bias, fewer than 128 batch rows with a bf16 bias whose rows are 16-byte aligned (read in
- * place, exactly), or a kernel that does not take one); negative = af3_status error.  Host only. */
+ * no bias, a bf16 bias with 16-byte aligned rows under too few batch rows for a rewrite to pay
+ * off -- fewer than about 224 + 2.4e8 / (H L^2); it is then read in place, exactly -- or a kernel
+ * that does not take one); negative = af3_status error.  Host only. */
 int64_t af3_dpa_workspace_bytes(const af3_dpa_params* params);
 
 /*

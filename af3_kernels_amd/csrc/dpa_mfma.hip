@@ -82,14 +82,16 @@ __device__ __forceinline__ u32x4 bias_frag_finite(u32x4 w) {
 template <bool BIAS_F32>
 __global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restrict__ bias, u32x4* __restrict__ ws, int64_t H, int64_t L, int64_t stride_h,
 															 int64_t stride_q, int n_qblocks, int n_ktiles, bool vec_ok) {
-	const int64_t total = H * n_qblocks * (int64_t)n_ktiles * 256;
-	for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-		const int     lane = (int)(i & 63), frag = (int)((i >> 6) & 3);
-		const int64_t t    = i >> 8;
-		const int     kt   = (int)(t % n_ktiles);
-		const int64_t t2   = t / n_ktiles;
-		const int     qb   = (int)(t2 % n_qblocks);
-		const int64_t h    = t2 / n_qblocks;
+	// one workgroup per (head, query block, key tile) and trip: the index arithmetic (divisions) is per workgroup, on the
+	// scalar unit, not per thread; the launcher keeps the number of units below 2^31
+	const uint32_t units = (uint32_t)(H * n_qblocks * (int64_t)n_ktiles);
+	const int      lane = threadIdx.x & 63, frag = threadIdx.x >> 6;
+	for(uint32_t u = blockIdx.x; u < units; u += gridDim.x) {
+		const int64_t i    = (int64_t)u * 256 + threadIdx.x;
+		const int     kt   = (int)(u % (uint32_t)n_ktiles);
+		const uint32_t t2  = u / (uint32_t)n_ktiles;
+		const int     qb   = (int)(t2 % (uint32_t)n_qblocks);
+		const int64_t h    = t2 / (uint32_t)n_qblocks;
 		const int64_t row  = (int64_t)qb * 32 + (lane & 31);
 		const int64_t key  = (int64_t)kt * KT + 16 * frag + 8 * (lane >> 5);
 		const int64_t esz  = BIAS_F32 ? 4 : 2;
@@ -1229,6 +1231,7 @@ static int launch_bias_prepass(const af3_dpa_params& p, hipStream_t s) {
 	const bool     bf32      = p.bias_dtype == AF3_F32;
 	const int      n_qblocks = (int)((p.L + 31) / 32), n_ktiles = (int)((p.L + KT - 1) / KT);
 	const int64_t  total     = p.H * n_qblocks * (int64_t)n_ktiles * 256;
+	if(total / 256 >= ((int64_t)1 << 31)) return AF3_ERR_BAD_SHAPE;  // (the prepass counts its units in 32 bits)
 	const unsigned g         = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
 	const bool     vec_ok    = ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) && (p.bias_stride[0] % 8 == 0) && (p.bias_stride[1] % 8 == 0);
 	if(bf32)

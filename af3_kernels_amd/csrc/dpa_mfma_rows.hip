@@ -39,14 +39,16 @@ constexpr float BIAS_FLOOR = -0x1p17f;     // lowest value the rewritten bias ho
 template <bool BIAS_F32>
 __global__ void __launch_bounds__(256) bias_rows_prepass_kernel(const void* __restrict__ bias, f32x4* __restrict__ ws, int64_t H, int64_t L, int64_t stride_h, int64_t stride_q,
 																  int n_qblocks, int n_tiles, bool vec_ok) {
-	const int64_t total = H * n_qblocks * (int64_t)n_tiles * 256;
-	for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-		const int     lane = (int)(i & 63), ld = (int)((i >> 6) & 3);
-		const int64_t t1   = i >> 8;
-		const int     t    = (int)(t1 % n_tiles);
-		const int64_t t2   = t1 / n_tiles;
-		const int     qb   = (int)(t2 % n_qblocks);
-		const int64_t h    = t2 / n_qblocks;
+	// one workgroup per (head, query block, key tile) and trip: the index arithmetic (divisions) is per workgroup, on the
+	// scalar unit, not per thread; the launcher keeps the number of units below 2^31
+	const uint32_t units = (uint32_t)(H * n_qblocks * (int64_t)n_tiles);
+	const int      lane = threadIdx.x & 63, ld = threadIdx.x >> 6;
+	for(uint32_t u = blockIdx.x; u < units; u += gridDim.x) {
+		const int64_t  i  = (int64_t)u * 256 + threadIdx.x;
+		const int      t  = (int)(u % (uint32_t)n_tiles);
+		const uint32_t t2 = u / (uint32_t)n_tiles;
+		const int      qb = (int)(t2 % (uint32_t)n_qblocks);
+		const int64_t  h  = t2 / (uint32_t)n_qblocks;
 		const int64_t row  = (int64_t)qb * 32 + (lane & 31);
 		const int64_t key  = (int64_t)t * KT_R + 8 * ld + 4 * (lane >> 5);
 		float         f[4] = {0.f, 0.f, 0.f, 0.f};
@@ -791,6 +793,7 @@ int launch_dpa_mfma_rows(const af3_dpa_params& p, hipStream_t s) {
 		const bool     bf32      = p.bias_dtype == AF3_F32;
 		const int      n_qblocks = (int)((p.L + 31) / 32), n_t_all = (int)((p.L + KT_R - 1) / KT_R);
 		const int64_t  total     = p.H * n_qblocks * (int64_t)n_t_all * 256;
+		if(total / 256 >= ((int64_t)1 << 31)) return AF3_ERR_BAD_SHAPE;  // (the prepass counts its units in 32 bits)
 		const unsigned g         = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
 		const int64_t  esz       = bf32 ? 4 : 2;
 		const bool     vec_ok    = ((reinterpret_cast<uintptr_t>(p.bias) & (4 * esz - 1)) == 0) && (p.bias_stride[0] % 4 == 0) && (p.bias_stride[1] % 4 == 0);

@@ -227,14 +227,16 @@ __device__ __forceinline__ void quantize_e4m3_body(const void* __restrict__ src,
 			*reinterpret_cast<uint32_t*>(dst + (mat * cols + c) * dst_row_stride + ((int64_t)r4 << 2)) = w;
 			if(dst_lo) *reinterpret_cast<uint32_t*>(dst_lo + (mat * cols + c) * dst_row_stride + ((int64_t)r4 << 2)) = residual(f0, f1, f2, f3, w);
 		};
-		if(SRC_BF16 && cols % 8 == 0 && src_row_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 && total < ((int64_t)1 << 31) && stride < ((int64_t)1 << 30)) {
+		if(SRC_BF16 && cols % 8 == 0 && src_row_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 && total < ((int64_t)1 << 29) && stride < ((int64_t)1 << 30)) {
 			// bf16 rows of whole 16-byte chunks: one thread = 4 consecutive rows x 8 consecutive columns (four 16-byte loads, eight
 			// 4-byte stores).  Consecutive lanes take consecutive row quads, so each store instruction of a wavefront writes 256
-			// consecutive bytes of one output row.
-			const uint32_t cb_n = (uint32_t)(cols >> 3), rq_u = (uint32_t)rq, items = (uint32_t)(n_mat * rq * (cols >> 3));
+			// consecutive bytes of one output row; consecutive wavefronts take the column blocks of the same 64 row quads, so
+			// the rows they share are fetched by one compute unit (in different workgroups they would be fetched once per XCD).
+			const uint32_t cb_n = (uint32_t)(cols >> 3), rq_u = (uint32_t)rq, rq_b = (rq_u + 63) >> 6, items = (uint32_t)n_mat * rq_b * cb_n * 64;
 			for(uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x; i < items; i += (uint32_t)stride) {
-				const uint32_t r4 = i % rq_u, cb = (i / rq_u) % cb_n;
-				const int64_t  mat = i / (rq_u * cb_n), r = mat * rows_per_matrix + ((int64_t)r4 << 2), left = rows_per_matrix - ((int64_t)r4 << 2);
+				const uint32_t wi = i >> 6, cb = wi % cb_n, r4 = ((wi / cb_n) % rq_b) * 64 + (i & 63);
+				if(r4 >= rq_u) continue;
+				const int64_t mat = wi / (cb_n * rq_b), r = mat * rows_per_matrix + ((int64_t)r4 << 2), left = rows_per_matrix - ((int64_t)r4 << 2);
 				u32x4          w[4];
 #pragma unroll
 				for(int k = 0; k < 4; k++) {

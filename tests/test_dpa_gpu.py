@@ -151,6 +151,9 @@ def test_small_grids_split_keys_over_wavefronts(af3, oracle, B, H, L, D, live):
     (10, 1000, 32, "f32", None),           # the same with an fp32 bias read in place
     (10, 1000, 16, "unaligned", 900),      # ... and with bias rows that cannot take 16-byte loads
     (9, 1056, 24, "bf16", 70),             # 297 blocks, 17 key tiles of which two are live: the loading wavefronts have nothing to fetch after the first two
+    (9, 1056, 24, "bf16", 150),            # three live tiles: the walk ends inside the loading wavefronts' first requests
+    (9, 1056, 24, "bf16", 250),            # four live tiles: exactly what is in flight behind the first barrier
+    (16, 1536, 32, "bf16", 300),           # five live tiles = the ring's length (eight computing wavefronts)
 ])
 def test_long_rows_pair_up_wavefronts_on_shared_tiles(af3, oracle, H, L, D, bias_kind, live):
     """B = 1 with 512..1024 query blocks and at least 8 key tiles: two wavefronts share each query block and the workgroup's

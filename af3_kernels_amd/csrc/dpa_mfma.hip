@@ -125,7 +125,8 @@ __global__ void __launch_bounds__(256) bias_prepass_kernel(const void* __restric
 // query rows AND the workgroup's K/V tiles -- wavefront 2q + s takes keys [32s, 32s + 32) of every 64-key tile for
 // query block q, so a wavefront's dependent chain is half as long and no LDS is spent on private buffers; the two
 // partial (O, m, l) are merged through LDS at the end.  The workgroup has NW + 4 wavefronts: the last four only issue the
-// tile loads (a ring of four tiles, two tiles ahead), so that the NW computing ones never stand still behind a load that the
+// tile loads (a ring of five tiles, three tiles ahead: every tile is in LDS one barrier before its first use, so that a
+// stage's LDS operands can be fetched at the end of the stage before), so that the NW computing ones never stand still behind a load that the
 // compute unit's load path has not taken in yet.  Requires NW even, no SPLIT, not FUSED.  (KSL = 1.  KSL = 2: the four
 // loading wavefronts and the ring of four tiles for workgroups of NW wavefronts with a query block each -- the form that
 // single rows of head_dim 48 or 64 take.)
@@ -207,7 +208,7 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 	const int     n = lane & 31, half = lane >> 5;
 	const int64_t L = p.L;
 	// KS2: the workgroup has four wavefronts more than the NW that compute (one per SIMD).  They issue the tile loads of the
-	// workgroup, two tiles ahead, a quarter of every tile each, and otherwise only keep the barriers' count.  A wavefront that
+	// workgroup, two or three tiles ahead, a quarter of every tile each, and otherwise only keep the barriers' count.  A wavefront that
 	// issues a tile's loads itself stands still while the compute unit's load path (64 bytes per clock) takes them in -- with
 	// one compute wavefront per SIMD nothing else runs in that time, and it was a quarter of the key loop.  (A single loader
 	// is too few: one wavefront gets a load accepted every 45-64 clocks at best.)
@@ -436,7 +437,7 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 
 	if constexpr(LOADERS) {
 		if(is_loader) {
-			// ---- a loader wavefront: tile j of the walk goes to buffer j % NBUF and is requested two tiles before the compute
+			// ---- a loader wavefront: tile j of the walk goes to buffer j % NBUF and is requested AHEAD + 1 tiles before the compute
 			// wavefronts fetch K fragments from it.  Its barriers mirror theirs one for one: one in front of the first S^T, one
 			// per live tile, and (pairs) three in the merge. ----
 			constexpr int PER_TILE = 2 * (NI / 4) + (BRING ? (KS2 ? NW / 2 : NW) : 0);  // this wavefront's loads per tile
@@ -997,7 +998,7 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 			} else if(BIAS_LATE) load_bias_frags(kt0, ic<1>{});
 			else if(my_n > 1) load_bias_frags(__builtin_amdgcn_readfirstlane(live_at(1)), ic<0>{});
 
-			int buf = 0;  // LDS buffer of tile `it` (it % 3)
+			int buf = 0;  // LDS buffer of tile `it` (it % NBUF)
 			// tile indices of iterations it, it+1, it+2 are carried in scalar registers; the list entry for
 			// it+3 is fetched at the top of an iteration and only consumed at its end
 			int kt = kt0, kt1 = __builtin_amdgcn_readfirstlane(live_at(1)), kt2 = __builtin_amdgcn_readfirstlane(live_at(2));

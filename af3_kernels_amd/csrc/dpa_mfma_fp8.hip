@@ -13,7 +13,7 @@
 // whose diagonal is 1/alpha (a power of two, exact in bf16), the key mask a third MFMA;
 // P^T = exp(logit - m) * 2^8 is quantised to e4m3 in registers (values in (0, 256], e4m3 tops out at
 // 448) and is the B operand of O^T += V8^T . P^T.  The row maximum m is the true running maximum
-// (no slack: P must stay below the e4m3 range), the row sum is taken over the unquantised P.
+// (no slack: P must stay below the e4m3 range), the row sum is taken over the quantised P, on the matrix pipe.
 // V arrives transposed, so V^T fragments are plain 4-byte LDS reads (no transposing loads exist for
 // 8-bit data paired with this accumulator layout).
 #include "common.hpp"
@@ -32,10 +32,6 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32v2;
 __device__ __forceinline__ float hswap_max(float x) {
 	auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
 	return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float hswap_sum(float x) {
-	auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-	return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 // DP: head_dim padded to 32 or 64 (bytes per K row in LDS, rows of the V^T tile).
@@ -241,8 +237,23 @@ __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2
 	const int mask_rd     = 2 * K_TILE + 2 * V_TILE + (half == 0 ? n * 4 : (n_ktiles * KT8 + n) * 4);
 	const int mask_stride = half == 0 ? KT8 * 4 : 0;
 
-	float  m_run = 0.f, mc = 0.f, l_run = 0.f;  // m_run in accumulator units; mc = m_run*c_exp - P_SHIFT
+	float  m_run = 0.f, mc = 0.f;  // m_run in accumulator units; mc = m_run*c_exp - P_SHIFT
 	bool   first = true;
+	// Row sums on the matrix pipe (as in dpa_mfma.hip): a 16x16x32 MFMA whose A operand is a 0/1 pattern adds the 16 quantised
+	// probabilities that a query's two lanes hold of a fragment; register 0 of the result is, in every lane, the running sum of
+	// that lane's own query row.  As a B operand of the 16x16x32 shape the P fragment's lane l is column l%16, contraction
+	// group l/16, and holds query l%32: groups 0,2 belong to queries 0..15, groups 1,3 to queries 16..31; output register 0
+	// of lane l is row 4*(l/16): rows 0 and 8 select the even groups, rows 4 and 12 the odd ones.  The normaliser is thus the
+	// sum of exactly the e4m3 weights that enter P.V (the result is a convex combination of V rows), and 16 vector adds per
+	// 32 x 32 block become two half-size matrix instructions.
+	f32x4 lacc = {0.f, 0.f, 0.f, 0.f};
+	long  ones_a;
+	{
+		const int  i16 = lane & 15, kg = lane >> 4;
+		const bool on  = ((i16 == 0 || i16 == 8) && (kg & 1) == 0) || ((i16 == 4 || i16 == 12) && (kg & 1) == 1);
+		const u32v2 w  = {on ? 0x38383838u : 0u, on ? 0x38383838u : 0u};  // e4m3 1.0
+		ones_a = __builtin_bit_cast(long, w);
+	}
 	f32x16 oacc[NDB];
 #pragma unroll
 	for(int db = 0; db < NDB; db++)
@@ -295,7 +306,8 @@ __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2
 			const float m_new = first ? mx : fmaxf(m_run, mx);
 			if(__ballot(first || m_new > m_run)) {
 				const float a = first ? 1.f : __builtin_amdgcn_exp2f((m_run - m_new) * c_exp);
-				l_run *= a;
+#pragma unroll
+				for(int i = 0; i < 4; i++) lacc[i] *= a;
 #pragma unroll
 				for(int db = 0; db < NDB; db++)
 #pragma unroll
@@ -304,19 +316,18 @@ __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2
 				mc    = m_new * c_exp - P_SHIFT;
 				first = false;
 			}
-			float psum = 0.f;
 			u32v2 pf[2];
 #pragma unroll
 			for(int i = 0; i < 16; i += 4) {
 				const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c_exp, -mc)), p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], c_exp, -mc));
 				const float p2 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 2], c_exp, -mc)), p3 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 3], c_exp, -mc));
-				psum += (p0 + p1) + (p2 + p3);
 				uint32_t w = 0;
 				w = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, w, false);
 				w = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, w, true);
 				pf[i >> 3][(i & 7) >> 2] = w;
 			}
-			l_run += psum;
+#pragma unroll
+			for(int cp = 0; cp < 2; cp++) lacc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(ones_a, __builtin_bit_cast(long, pf[cp]), lacc, 0, 0, 0);
 			// O^T += V8^T . P^T: contraction slot j of chunk cp is key 16cp + 8(j/4) + 4half + j%4
 #pragma unroll
 			for(int cp = 0; cp < 2; cp++)
@@ -331,8 +342,8 @@ __global__ void __launch_bounds__(NW8 * 64) __attribute__((amdgpu_waves_per_eu(2
 		__syncthreads();
 	}
 
-	// epilogue: out = O * dv / l   (l was summed over p * 2^8, the same factor O carries)
-	const float inv = dv / hswap_sum(l_run);
+	// epilogue: out = O * dv / l   (l was summed over p * 2^8, the same factor O carries; both half-waves are in it)
+	const float inv = dv / lacc[0];
 	if(row_ok) {
 		const int64_t ooff = b * p.out_stride[0] + h * p.out_stride[1] + qrow * p.out_stride[2];
 #pragma unroll

@@ -1010,7 +1010,9 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 					const int bufn = buf == NBUF - 1 ? 0 : buf + 1, bufnn = bufn == NBUF - 1 ? 0 : bufn + 1;
 					// The barrier hands the buffer of tile it-1 back to the loading wavefronts, so this wavefront's reads of that
 					// tile must have returned; the operands fetched at the end of the stage before (the last OPERAND_READS LDS
-					// reads issued, from the buffer of tile it+1) may stay in flight.  LDS reads return in issue order.
+					// reads issued, from the buffer of tile it+1) may stay in flight.  LDS reads return in issue order.  (The counter
+					// also counts scalar memory loads, which do not: this relies on the loop holding none -- every kernel argument
+					// is in registers before the loop, and the compiler has no reason to fetch one again while none is spilled.)
 					constexpr int OPERAND_READS = NC + 1 + (BRING ? 2 : 0);
 					asm volatile("s_waitcnt lgkmcnt(%0)\n\ts_barrier" ::"n"(OPERAND_READS) : "memory");
 					const int kt3_v = live_at(it + 3);  // (behind the barrier, which would wait for this read)

@@ -387,3 +387,27 @@ def test_static_scratch_entry_point_rejects_calls_beyond_its_limit_on_the_host()
     assert b"scratch" in lib.af3_status_string(-9)
     with pytest.raises(ValueError):
         _lib.check(-9, "x")
+
+
+def test_workspace_query_follows_the_batch_size_at_which_a_bias_rewrite_pays_off():
+    """af3_dpa_workspace_bytes (host only): a bf16 bias with 16-byte aligned rows is read in place -- no workspace -- while the
+    batch has fewer rows than about 224 + 2.4e8 / (H L^2); beyond that, or when the rows cannot be staged, the fp32 rewrite
+    (H * ceil(L/32)^2 blocks of 4 KB) is asked for."""
+    from af3_kernels_amd import _lib
+    lib = _lib.load()
+    need = lib.af3_dpa_workspace_bytes
+
+    def call(B, H, L, bias=0x1000, row_stride=None):
+        st = (ctypes.c_int64 * 3)(H * L * 32, L * 32, 32)
+        rs = L if row_stride is None else row_stride
+        return need(ctypes.byref(_params(B=B, H=H, L=L, bias=bias, bias_stride=(ctypes.c_int64 * 2)(L * rs, rs), q_stride=st, k_stride=st, v_stride=st, out_stride=st)))
+
+    rewrite = lambda H, L: H * ((L + 31) // 32) ** 2 * 4096
+    assert call(384, 4, 384) == 0                        # cfg2: 384 < 224 + 2.4e8 / (4 * 384^2) = 637
+    assert call(700, 4, 384) == rewrite(4, 384)
+    assert call(300, 4, 768) == 0                        # 300 < 327
+    assert call(768, 4, 768) == rewrite(4, 768)          # cfg4
+    assert call(64, 16, 1536) == 0 and call(256, 16, 1536) == rewrite(16, 1536)   # 230 for the diffusion bias
+    assert call(64, 4, 768, bias=0x1008) == rewrite(4, 768)          # rows only 8-byte aligned: not staged
+    assert call(64, 4, 396) == rewrite(4, 396)                       # L % 8 != 0: not staged
+    assert call(64, 4, 768, bias=None) == 0 and call(1, 16, 768) == 0

@@ -757,15 +757,18 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 			float alpha;
 			if(L2DOM) {
 				// s already has m_ref subtracted (by the mask MFMA)
-				// (a first sub-tile whose keys are all dropped says nothing about the row: the reference stays at 0, its
-				// probabilities are exactly 0, and the first live logits keep their own bits)
-				const bool  need  = (force && (all_dropped || mx > -0x1p99f)) || mx > REF_SLACK;  // (a row without any live key keeps the mask constant as its reference)
+				// A sub-tile whose keys are all dropped says nothing about the row: the reference stays at 0, its probabilities are
+				// exactly 0, and the first live logits keep their own bits.  Until a row has a non-zero sum (`fresh`) its first
+				// live logits fix the reference wherever they lie -- the largest then has probability exactly 1, so a row whose
+				// biases are all hugely negative cannot end with a zero sum -- and nothing is accumulated that would need rescaling.
+				const bool  fresh = force || lacc[0] == 0.f;
+				const bool  need  = (fresh && (all_dropped || mx > -0x1p99f)) || mx > REF_SLACK;  // (a row without any live key keeps the mask constant as its reference)
 				const float m_want = m_ref + mx;
 				const float m_hi   = bf16_bits_to_f32(f32_to_bf16_bits(need ? m_want : m_ref));
 				const float m_lo   = bf16_bits_to_f32(f32_to_bf16_bits((need ? m_want : m_ref) - m_hi));
 				const float m_new  = m_hi + m_lo;  // exactly what the mask MFMA will subtract (unchanged when !need)
 				const float delta  = m_new - m_ref;
-				alpha = force ? 1.f : __builtin_amdgcn_exp2f(-delta);  // nothing is accumulated yet when forced (first sub-tile)
+				alpha = fresh ? 1.f : __builtin_amdgcn_exp2f(-delta);
 #pragma unroll
 				for(int i = 0; i < 16; i++) s[i] -= delta;
 				if(pending) {
@@ -950,8 +953,10 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 			rowsum_mfma(pcur[1]);
 			if constexpr(KS2) fetch_operands(subn_c, k_next, mask_next_addr, ring_next);  // (this stage's have been consumed)
 			// The running sum stays below L * 2^REF_SLACK <= 2^25 while every probability respects the
-			// reference, so this also catches a single probability near or beyond the limit (inf, NaN).
-			if(__ballot(!(lacc[0] < PSUM_LIMIT))) {  // rare
+			// reference, so this also catches a single probability near or beyond the limit (inf, NaN).  A sum that is still
+			// zero (log2 variant: leading sub-tiles of dropped keys, or live logits so far below the initial reference that
+			// their probabilities flush to zero) takes the same path, which then fixes the reference at the first live logits.
+			if(__ballot(!(lacc[0] < PSUM_LIMIT) || (L2DOM && lacc[0] == 0.f))) {  // rare
 				lacc[0] = l_before;
 				rereference(sc, &sn, false);
 				exp_part(sc, pcur, ic<0>{}, ic<16>{});
@@ -1075,10 +1080,12 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 			float* const mred = reinterpret_cast<float*>(smem);        // [NW][32] reference maxima
 			float* const obuf = mred + NW * 32;                        // [NW / 2][16*NDB + 1][64]
 			static_assert((NW * 32 + (NW / 2) * (16 * NDB + 1) * 64) * 4 <= 2 * NBUF * TILE_BYTES, "the merge area fits in the K/V buffers");
-			if(half == 0) mred[wave * 32 + n] = m_ref;
+			// (a wavefront whose sum is zero has seen dropped keys only: its reference says nothing and must not enter the maximum)
+			const bool started = lacc[0] > 0.f;
+			if(half == 0) mred[wave * 32 + n] = started ? m_ref : -INFINITY;
 			__syncthreads();
 			const float mstar   = fmaxf(mred[(wave & ~1) * 32 + n], mred[(wave | 1) * 32 + n]);
-			const float scale_w = __builtin_amdgcn_exp2f((m_ref - mstar) * (L2DOM ? 1.f : LOG2E));
+			const float scale_w = started ? __builtin_amdgcn_exp2f((m_ref - mstar) * (L2DOM ? 1.f : LOG2E)) : 0.f;
 			lacc[0] *= scale_w;
 #pragma unroll
 			for(int db = 0; db < NDB; db++)
@@ -1106,12 +1113,15 @@ __global__ void __launch_bounds__((NW + (KSL ? 4 : 0)) * 64) __attribute__((amdg
 			__syncthreads();  // all K/V buffers are dead: reuse the front of LDS
 			float* const mred = reinterpret_cast<float*>(smem);        // [NW][32] reference maxima
 			float* const obuf = mred + NW * 32;                        // [NW][16*NDB + 1][64]
-			if(half == 0) mred[wave * 32 + n] = my_n > 0 ? m_ref : -INFINITY;
+			// (a wavefront without a tile, or whose sum is zero -- it has seen dropped keys only --, contributes nothing, and its
+			// reference must not enter the maximum)
+			const bool started = my_n > 0 && lacc[0] > 0.f;
+			if(half == 0) mred[wave * 32 + n] = started ? m_ref : -INFINITY;
 			__syncthreads();
 			float mstar = mred[n];
 #pragma unroll
 			for(int w = 1; w < NW; w++) mstar = fmaxf(mstar, mred[w * 32 + n]);
-			const float scale_w = my_n > 0 ? __builtin_amdgcn_exp2f((m_ref - mstar) * (L2DOM ? 1.f : LOG2E)) : 0.f;
+			const float scale_w = started ? __builtin_amdgcn_exp2f((m_ref - mstar) * (L2DOM ? 1.f : LOG2E)) : 0.f;
 			lacc[0] *= scale_w;
 #pragma unroll
 			for(int db = 0; db < NDB; db++)

@@ -108,6 +108,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	const int     n_t_all  = (int)((L + KT_R - 1) / KT_R);
 	uint16_t* const mask_tab = reinterpret_cast<uint16_t*>(smem + MASK_BASE);
 	__shared__ int  s_last[4];  // index of the last live key + 1 of each batch row (0: every key dropped)
+	__shared__ int  s_first[4]; // index of the first key tile of each batch row that holds a live key
 
 	// ---- workgroup -> (group of batch rows, head, query tile): all query tiles of one (group, head) get ids congruent
 	// mod 8, i.e. the same XCD (they share that XCD's L2 copy of K and V), and an XCD only sees heads xcd % H (for H | 8),
@@ -253,7 +254,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 		const int      r    = wave;
 		const int64_t  br   = b0 + r < b_end ? b0 + r : b_end - 1;
 		const uint8_t* keep = p.key_mask ? p.key_mask + br * p.key_mask_stride_b : nullptr;
-		int            last = 0;
+		int            last = 0, first = -1;   // (first: wave-uniform, from ballots)
 		const bool     vec  = !keep || (((reinterpret_cast<uintptr_t>(p.key_mask) | (uintptr_t)p.key_mask_stride_b | (uintptr_t)L) & 3) == 0);
 		if(vec) {
 			constexpr int MAXC = MAX_L_ROWS / 256 + 1;   // chunks of 256 keys (4 per lane) that cover the table
@@ -280,6 +281,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 					if(key0 < n_keys_tab) *reinterpret_cast<u32x2*>(mask_tab + ((key0 >> 5) * ROWS + r) * 32 + (key0 & 31)) = u32x2{e[0] | (e[1] << 16), e[2] | (e[3] << 16)};
 				}
 			};
+#pragma unroll
+			for(int c = MAXC - 1; c >= 0; c--) {   // a lane's four keys of chunk c lie in tile 8 c + lane / 8
+				const unsigned long long bal = __ballot(mraw[c] != 0u);   // (chunks at or beyond L hold zeros)
+				if(bal) first = 8 * c + (__builtin_ctzll(bal) >> 3);
+			}
 			write_chunks(false);
 #pragma unroll
 			for(int off = 32; off >= 1; off >>= 1) {
@@ -301,23 +307,31 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 				if(key < n_keys_tab) mask_tab[((key >> 5) * ROWS + r) * 32 + (key & 31)] = live ? (uint16_t)0 : (in ? MASK_DROPPED_BF16 : MASK_OUT_OF_RANGE_BF16);
 				const unsigned long long bal = __ballot(live);
 				if(bal) last = base + 64 - __builtin_clzll(bal);
+				if(bal && first < 0) first = (base + __builtin_ctzll(bal)) / KT_R;
 			}
 			if(last == 0)   // (as above)
 				for(int key = lane; key < n_keys_tab; key += 64) mask_tab[((key >> 5) * ROWS + r) * 32 + (key & 31)] = key < L ? (uint16_t)0 : MASK_OUT_OF_RANGE_BF16;
 		}
-		if(lane == 0) s_last[r] = last;
+		if(lane == 0) s_last[r] = last, s_first[r] = first;
 	}
 	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's pieces of the first tile and its bias fragment have landed
 	__syncthreads();                                    // the mask table and the first tile are complete
 	// keys behind the last live key of every row carry weight 0 and are not walked; a row without live keys needs them all
-	int  l_eff = 0;
+	// The softmax reference of a batch row is fixed by the first tile that holds a live key of that row (a tile of dropped
+	// keys says nothing about the row's logits): tiles up to the last such tile over the group's rows (normally tile 0 alone)
+	// run the variant of the tile code that can do so.
+	int  l_eff = 0, t_force_max = 0;
 	bool dropped[ROWS];
+	uint32_t first_tiles = 0;   // byte r: the first tile of batch row r that holds a live key (at most 128 tiles)
 #pragma unroll
 	for(int r = 0; r < ROWS; r++) {
 		const int last = __builtin_amdgcn_readfirstlane(s_last[r]);
 		dropped[r]     = last == 0;
 		const int need = dropped[r] ? (int)L : last;
 		l_eff          = need > l_eff ? need : l_eff;
+		const int ft   = dropped[r] ? 0 : __builtin_amdgcn_readfirstlane(s_first[r]);
+		first_tiles |= (uint32_t)ft << (8 * r);
+		t_force_max    = ft > t_force_max ? ft : t_force_max;
 	}
 	n_t = (l_eff + KT_R - 1) / KT_R;
 
@@ -395,9 +409,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 		for(int i = 3; i < 15; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
 		mx = half_swap_max(fmaxf(mx, s[15]));
 		// s already has m_ref subtracted (by the mask MFMA)
-		// (a first tile whose keys are all dropped says nothing about the row: the reference stays where it is, the tile's
-		// probabilities are exactly 0, and the first live logits are measured against a reference they can be subtracted
-		// from without losing their own bits)
+		// (forced: the row's first tile with a live key.  Every query then has a logit above the mask constants, the new
+		// reference is its maximum, and that key's probability is exactly 1: the row sum can no longer flush to zero however
+		// negative the row's biases are.  Tiles in front of it hold dropped keys only: their probabilities are exactly 0
+		// against the initial reference 0, and nothing has been accumulated when the reference moves.)
 		const bool  need   = (force && mx > -0x1p99f) || mx > REF_SLACK;
 		const float m_want = m_ref[R] + mx;
 		const float m_hi   = bf16_bits_to_f32(f32_to_bf16_bits(need ? m_want : m_ref[R]));
@@ -479,12 +494,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 	// k_addr2: LDS byte address of the K tile of the step after the next; m_addr: (per lane) of the next step's mask
 	// entries; v_addr: of this step's V tile; hook(i): run behind the i-th matrix instruction of the step (i = 0..4; 1 is the
 	// first K.Q^T instruction of the next step).
-	// FIRST: the very first tile, which fixes every row's softmax reference.  ANYDROP: some batch row of this group has no
+	// FIRST: a leading tile, in which a row that meets its first live key (`force`, wave-uniform) fixes its softmax reference.  ANYDROP: some batch row of this group has no
 	// live key (it then takes no bias: a wave-uniform branch the common instantiation does not carry).
-	auto step = [&](auto r_c, auto first_c, auto anydrop_c, int k_addr2, int m_addr, int v_addr, auto&& hook) {
+	auto step = [&](auto r_c, auto first_c, auto anydrop_c, bool force, int k_addr2, int m_addr, int v_addr, auto&& hook) {
 		constexpr int  R = decltype(r_c)::value, RN = (R + 1) % ROWS, RP = (R + ROWS - 1) % ROWS;
 		constexpr bool FIRST = decltype(first_c)::value != 0, ANYDROP = decltype(anydrop_c)::value != 0;
-		if constexpr(FIRST) rereference(r_c, sc, true);
+		if constexpr(FIRST) rereference(r_c, sc, force);
 		maskA[0] = *reinterpret_cast<const uint16_t*>(smem + m_addr);
 		u32x4  pcur[2];
 		f32x16 sn;
@@ -592,9 +607,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 				const int     k2 = (R2 >= ROWS ? bufn : buf) + (R2 % ROWS) * (2 * TILE_R);   // ... may belong to the next tile
 				const int     m1 = m0 + R1 * 64;                             // (row ROWS of tile t is row 0 of tile t + 1)
 				const int     vc = buf + R * (2 * TILE_R);
+				const bool    fr = decltype(first_c)::value != 0 && t == (int)((first_tiles >> (8 * (R < ROWS ? R : 0))) & 0xffu);
 				if constexpr(R == ROWS - 2) {
 					asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-					step(r_c, first_c, anydrop_c, k2, m1, vc, [&](auto s_c) {
+					step(r_c, first_c, anydrop_c, fr, k2, m1, vc, [&](auto s_c) {
 						constexpr int S = decltype(s_c)::value;
 						if constexpr(S == 1) {
 							load_tile(t + 2, bufnn);
@@ -604,12 +620,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 						}
 					});
 				} else if constexpr(R == ROWS - 1) {
-					step(r_c, first_c, anydrop_c, k2, m1, vc, [&](auto s_c) {
+					step(r_c, first_c, anydrop_c, fr, k2, m1, vc, [&](auto s_c) {
 						constexpr int S = decltype(s_c)::value;
 						if constexpr(S == 1) load_bias(t + 2);   // (behind this step's first K.Q^T instruction, which has waited for the slot's reads)
 					});
 				} else {
-					step(r_c, first_c, anydrop_c, k2, m1, vc, [](auto) {});
+					step(r_c, first_c, anydrop_c, fr, k2, m1, vc, [](auto) {});
 				}
 			}
 		};
@@ -636,9 +652,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 			kf[0] = read_kfrag(2 * TILE_R + k_rd[0]);
 			kf[1] = read_kfrag(2 * TILE_R + k_rd[1]);
 		}
-		tile(ic<1>{}, anydrop_c, 0, 0, BUF_R, 2 * BUF_R);
-		int buf = BUF_R;
-		for(int t = 1; t < n_t; t++) {
+		int buf = 0, t = 0;
+		for(; t <= t_force_max; t++) {   // (one trip unless some row's leading tiles hold dropped keys only)
+			const int bufn = buf == (NBUF_R - 1) * BUF_R ? 0 : buf + BUF_R, bufnn = bufn == (NBUF_R - 1) * BUF_R ? 0 : bufn + BUF_R;
+			tile(ic<1>{}, anydrop_c, t, buf, bufn, bufnn);
+			buf = bufn;
+		}
+		for(; t < n_t; t++) {
 			const int bufn = buf == (NBUF_R - 1) * BUF_R ? 0 : buf + BUF_R, bufnn = bufn == (NBUF_R - 1) * BUF_R ? 0 : bufn + BUF_R;
 			tile(ic<0>{}, anydrop_c, t, buf, bufn, bufnn);
 			buf = bufn;

@@ -1,6 +1,6 @@
 """Benchmark of the biased dot-product-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--case cfg4] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--case cfg4] [--no-cpu-baseline] [--only-headline]
     python bench.py --case grid_n768      (the fused grid self-attention caller; also grid_n384, grid_n1536, self_n1536, self5_n1536)
     python bench.py --case ln_bias_n768   (LayerNorm + pair-bias projection in front of it)
     python bench.py --case glu_n1536      (the gated linear unit of the transition blocks)
@@ -8,7 +8,8 @@
 A step is one call of dot_product_attention_cpp (the drop-in for the reference's
 af3_kernels.dot_product_attention_cpp) on synthetic inputs already resident in HBM.  The default
 workload is the headline case: triangle attention, N = 768, 4 heads x 32, batched over 768
-rows, bf16.  Prints ONE JSON line.
+rows, bf16.  The default run also times the other named configurations that fit the same call (cfg2, cfg3, cfg5: GPU
+legs only, `other_configs` of the same line) before the headline leg.  Prints ONE JSON line.
 """
 import argparse
 import json
@@ -341,6 +342,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--case", default="cfg4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only-headline", action="store_true", help="default case only: skip the legs of cfg2, cfg3 and cfg5 (e.g. under a profiler)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (every (batch, head, query-tile) task is "
@@ -366,87 +368,108 @@ def main():
         return bench_layernorm_pair_bias(args, int(args.case[len("ln_bias_n"):]))
     case = CASES[args.case]
     dev = torch.device("cuda:0")
-    q, k, v, mask, bias = make_inputs(case, device=dev)
-    fp8 = case.mma_dtype == "fp8"
-    fn = (lambda: af3.dot_product_attention_fp8(q, k, v, mask, bias)) if fp8 else (lambda: af3.dot_product_attention_cpp(q, k, v, mask, bias))
-    kernel = "fp8_mfma" if fp8 else af3.selected_kernel(q, k, v, mask, bias)
-
-    # The kernel is enqueued on torch's current stream, so events recorded on that stream bracket it.
+    # The kernels are enqueued on torch's current stream, so events recorded on that stream bracket them.
     stream = torch.cuda.current_stream(dev)
 
-    def measure():
-        """W untimed warm-up steps, then exactly K timed steps between synchronisations; per-launch HIP events."""
-        for _ in range(args.warmup):
+    def prepare(c):
+        q, k, v, mask, bias = make_inputs(c, device=dev)
+        fp8 = c.mma_dtype == "fp8"
+        fn = (lambda: af3.dot_product_attention_fp8(q, k, v, mask, bias)) if fp8 else (lambda: af3.dot_product_attention_cpp(q, k, v, mask, bias))
+        return fn, ("fp8_mfma" if fp8 else af3.selected_kernel(q, k, v, mask, bias)), (q, k, v, mask, bias)
+
+    def measure(fn, warmup, steps):
+        """`warmup` untimed steps, then exactly `steps` timed steps between synchronisations; per-launch HIP events."""
+        for _ in range(warmup):
             o = fn()
         torch.cuda.synchronize()
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
         t0 = time.perf_counter()
         for s, e in evs:
             s.record(stream)
             o = fn()
             e.record(stream)
         torch.cuda.synchronize()
-        wall = (time.perf_counter() - t0) * 1e3 / args.steps
+        wall = (time.perf_counter() - t0) * 1e3 / steps
         per = sorted(s.elapsed_time(e) for s, e in evs)
-        k_ms = sum(per) / len(per)          # average launch duration of the timed region
-        step_ms = max(wall, k_ms) if args.steps < 5 else (evs[0][0].elapsed_time(evs[-1][1]) / args.steps)
+        k_ms = sum(per) / len(per)          # average duration of one step's launches in the timed region
+        step_ms = max(wall, k_ms) if steps < 5 else (evs[0][0].elapsed_time(evs[-1][1]) / steps)
         assert torch.isfinite(o).all()
         return step_ms, k_ms, per
 
-    t_start = time.perf_counter()
-    ms_per_step, kernel_ms, per_launch = measure()
-    first_pass = None
-    # A run this short sits entirely inside the GPU's power-management transient: from idle the first few launches run
-    # at boost clock, the next ~25 are throttled hard (up to 30 % slower), and only after some tens of milliseconds does
-    # the clock settle where a model that calls this op layer after layer would see it.  The first pass (from idle,
-    # exactly as asked) is reported as `first_pass_from_idle`; the GPU is then kept busy with the same call for a
-    # fixed 0.4 s and the same W + K protocol is repeated: that second pass is the headline.  Long runs (the default
-    # 500 + 2000) settle within their own warm-up and are measured once.
-    settle = None
-    untimed_before = 0
-    if time.perf_counter() - t_start < 0.3:
-        first_pass = {"ms_per_step": round(ms_per_step, 4), "kernel_ms_avg": round(kernel_ms, 4)}
+    def roofline_of(c, kernel, kernel_ms, per_launch):
+        peak = PEAK_TFLOPS[c.mma_dtype]
+        if c.name in ("cfg3", "cfg5"):   # small head_dim, one bias stream for the whole call: priced against HBM
+            ach = c.bytes / (kernel_ms * 1e-3) / 1e9
+            r = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+                 "bias_stream_GBps": round(c.H * c.L * c.L * 2 / (kernel_ms * 1e-3) / 1e9, 1),
+                 "mfma_tflops": round(c.flops / (kernel_ms * 1e-3) / 1e12, 1), "mfma_frac": round(c.flops / (kernel_ms * 1e-3) / 1e12 / peak, 4)}
+        else:
+            k_tflops = c.flops / (kernel_ms * 1e-3) / 1e12
+            r = {"bound": "mfma", "achieved": round(k_tflops, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(k_tflops / peak, 4), "traffic": None}
+        r["traffic"] = measured_traffic_bytes(c.name)
+        r["kernel"] = kernel
+        r["kernel_ms_avg"] = round(kernel_ms, 4)
+        r["kernel_ms_median"] = round(per_launch[len(per_launch) // 2], 4)
+        r["algorithmic_flops_per_launch"] = c.flops
+        r["algorithmic_bytes_per_launch"] = c.bytes
+        return r
+
+    # ---- the other named configurations, GPU legs only, in front of the headline leg (default run only) ----
+    # Each leg: 20 untimed + 200 timed steps of the same drop-in call on that configuration's synthetic inputs (well under a
+    # second together).  They run first, in the order of their numbers, so that the headline leg below is what the timed
+    # region of this script ends with; the GPU therefore enters the headline leg busy, not idle.
+    others = {}
+    if args.case == "cfg4" and not args.only_headline:
+        for name in ("cfg2", "cfg3", "cfg5"):
+            c = CASES[name]
+            fn_c, kern_c, keep = prepare(c)
+            step_ms, k_ms, per = measure(fn_c, 20, 200)
+            rec = {"workload": f"{c.name}: B={c.B} H={c.H} L={c.L} D={c.D} io={c.io_dtype} mma={c.mma_dtype} mask={c.mask_kind}", "steps": 200, "warmup": 20,
+                   "ms_per_step": round(step_ms, 4), "tflops": round(c.flops / (step_ms * 1e-3) / 1e12, 2), "roofline": roofline_of(c, kern_c, k_ms, per)}
+            if name == "cfg5":   # the same shape through the bf16 path (the e4m3 path includes its quantisation launches)
+                q, k, v, mask, bias = keep
+                b_ms, bk_ms, _ = measure(lambda: af3.dot_product_attention_cpp(q, k, v, mask, bias), 20, 200)
+                rec["same_shape_bf16_path"] = {"ms_per_step": round(b_ms, 4), "kernel_ms_avg": round(bk_ms, 4), "kernel": af3.selected_kernel(q, k, v, mask, bias)}
+            others[name] = rec
+            del fn_c, keep
+        torch.cuda.empty_cache()
+
+    fn, kernel, _inputs = prepare(case)
+    # ---- the headline leg: exactly the W untimed and K timed steps asked for ----
+    ms_per_step, kernel_ms, per_launch = measure(fn, args.warmup, args.steps)
+    # A short run (the driver's 5 + 20 steps last 10 ms) sits inside the GPU's power-management transient: the clock is
+    # still moving when the timed steps start.  As a second, separately labelled figure the GPU is then kept busy with the
+    # same call for a fixed 0.4 s and the same W + K protocol is repeated (`settled_pass`): the rate a model sees that calls
+    # this op layer after layer.  Long runs (--warmup 500 --steps 2000) settle within their own warm-up.
+    settled = None
+    if args.warmup + args.steps < 400:
         t0, n_settle = time.perf_counter(), 0
         while time.perf_counter() - t0 < 0.4:
             for _ in range(20):
                 fn()
             torch.cuda.synchronize()
             n_settle += 20
-        settle = {"seconds": 0.4, "calls": n_settle}
-        untimed_before = args.warmup + args.steps + n_settle   # the whole first pass and the settling launches
-        ms_per_step, kernel_ms, per_launch = measure()
+        s_ms, sk_ms, s_per = measure(fn, args.warmup, args.steps)
+        settled = {"ms_per_step": round(s_ms, 4), "kernel_ms_avg": round(sk_ms, 4), "tflops": round(case.flops / (s_ms * 1e-3) / 1e12, 2),
+                   "roofline_frac": round(case.flops / (sk_ms * 1e-3) / 1e12 / PEAK_TFLOPS[case.mma_dtype], 4) if case.name not in ("cfg3", "cfg5") else None,
+                   "untimed_calls_before": args.warmup + args.steps + n_settle + args.warmup, "settle_seconds": 0.4}
 
     tflops = case.flops / (ms_per_step * 1e-3) / 1e12
-    k_tflops = case.flops / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[case.mma_dtype]
-    hbm_bound = case.name in ("cfg3", "cfg5")
-    if hbm_bound:
-        ach = case.bytes / (kernel_ms * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
-                    "bias_stream_GBps": round(case.H * case.L * case.L * 2 / (kernel_ms * 1e-3) / 1e9, 1)}
-    else:
-        roofline = {"bound": "mfma", "achieved": round(k_tflops, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(k_tflops / peak, 4), "traffic": None}
-    roofline["traffic"] = measured_traffic_bytes(case.name)
-    roofline["kernel"] = kernel
-    roofline["kernel_ms_avg"] = round(kernel_ms, 4)
-    roofline["kernel_ms_median"] = round(per_launch[len(per_launch) // 2], 4)
-    roofline["algorithmic_flops_per_launch"] = case.flops
-    roofline["algorithmic_bytes_per_launch"] = case.bytes
-
     line = {
         "metric": "biased-attention TFLOP/s + % MFMA peak, triangle attn N=768 bf16 (1 GPU)" if case.name == "cfg4" else f"biased-attention TFLOP/s ({case.name})",
-        # `warmup` is what actually ran untimed in front of the K timed steps: the W asked for, plus -- for a short run --
-        # the first pass and the settling launches described above
-        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup + untimed_before,
-        "warmup_requested": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": case.mma_dtype, "data": "synthetic",
         "config": {"workload": f"{case.name}: B={case.B} H={case.H} L={case.L} D={case.D} io={case.io_dtype} mask={case.mask_kind}",
                    "flops": case.flops, "pct_of_mfma_peak": round(100 * tflops / peak, 2)},
-        "roofline": roofline,
+        "roofline": roofline_of(case, kernel, kernel_ms, per_launch),
     }
-    if first_pass is not None:
-        line["first_pass_from_idle"] = first_pass
-        line["settle_between_passes"] = settle
+    if others:
+        line["legs_before_headline"] = list(others)
+        line["other_configs"] = others
+    if settled is not None:
+        line["settled_pass"] = settled
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(case)
     print(json.dumps(line))

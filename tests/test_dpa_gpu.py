@@ -639,6 +639,48 @@ def test_shared_bias_kernel_moves_its_reference(rows_kernel, oracle):
     assert np.abs(out - want).max() <= 0.25
 
 
+@pytest.mark.parametrize("B,L,bias_dtype", [(6, 320, torch.bfloat16), (6, 324, torch.bfloat16), (20, 324, torch.bfloat16), (20, 320, torch.float32)],
+                         ids=["bias_staged_through_lds", "bias_read_in_place", "bias_workspace", "bias_workspace_from_fp32"])
+def test_shared_bias_kernel_leading_dead_tiles_and_hugely_negative_bias_rows(rows_kernel, oracle, B, L, bias_dtype):
+    """A batch row whose leading key tiles hold no live key fixes its softmax reference at its first tile that does.  Query
+    rows whose biases are -3e4, -1e9 or -inf throughout (padded queries masked through the bias) then still get a finite
+    result -- the softmax over their live keys, uniform where nothing distinguishes them -- exactly as for batch rows whose
+    first tile is live, and as the one-row kernel gives."""
+    af3 = rows_kernel
+    H, D = 2, 32
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.bfloat16, seed=1234 + B, mask="random")
+    m[1, :64] = False        # two leading tiles without a live key
+    m[3, :32] = False        # one
+    m[2, :300] = False       # nearly everything: the reference is fixed in the row's last tile but one
+    m[:, 310] = True
+    bias = bias.to(bias_dtype)
+    bias[:, 5, :] = -3.0e4
+    bias[:, 6, :] = -1.0e9
+    bias[:, 7, :] = float("-inf")
+    bias[:, 40, :] = -3.0e4
+    bias[:, 40, 200] = -2.9e4     # one key stands out by far
+    try:
+        out = af3.dot_product_attention_cpp(*dev(q, k, v, m, bias)).float().cpu()
+        af3.set_rows_kernel("never")
+        other = af3.dot_product_attention_cpp(*dev(q, k, v, m, bias)).float().cpu()
+    finally:
+        af3.set_rows_kernel("always")
+    assert torch.isfinite(out).all() and torch.isfinite(other).all()
+    # The kernels clamp -1e9 and -inf in the bias to a large finite value, so such a query row is the softmax of q.k over its
+    # live keys, and dropped keys keep weight exactly 0.  The formula says the same once these rows hold a value that stays
+    # apart from its masked_fill(-1e9) (at -1e9 itself a dropped key would tie with the live ones; a row of -inf is NaN).
+    fbias = bias.float().clone()
+    fbias[:, 6, :] = -1.0e8
+    fbias[:, 7, :] = -1.0e8
+    want = torch.from_numpy(oracle.dpa_formula(f32np(q), f32np(k), f32np(v), m.numpy(), fbias.numpy()))
+    assert (out - want).abs().max().item() <= 2e-2
+    assert (out - other).abs().max().item() <= 2e-2
+    # the query row with one outstanding key returns that key's V row (where the key is live)
+    for b in range(B):
+        if m[b, 200]:
+            assert (out[b, :, 40, :] - v[b, :, 200, :].float()).abs().max().item() <= 2 ** -7 * v[b, :, 200, :].float().abs().max().item() + 1e-6
+
+
 # ---- element-wise kernels -------------------------------------------------------------------
 
 def test_convert_matches_torch_casts(af3):

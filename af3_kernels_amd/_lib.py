@@ -8,7 +8,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libaf3_dpa.so")
 
-AF3_F32, AF3_BF16, AF3_FP8_E4M3 = 0, 1, 2
+AF3_F32, AF3_BF16, AF3_FP8_E4M3, AF3_FP8_E5M2 = 0, 1, 2, 3
 ABI_VERSION = 4
 STATIC_SCRATCH_BYTES = 16 * 1024 * 1024   # AF3_STATIC_SCRATCH_BYTES
 

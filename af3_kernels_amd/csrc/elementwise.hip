@@ -80,6 +80,58 @@ __global__ void __launch_bounds__(EW_THREADS) cvt_e4m3_kernel(const uint8_t* __r
 	}
 }
 
+// ---- e5m2 (OCP float8 e5m2: fp16's exponent range with two mantissa bits; infinities and NaN like IEEE) ---------------
+// fp32 -> e5m2 bits, round to nearest even straight from fp32 (one rounding), overflow to infinity: what torch.float8_e5m2
+// does.  (The reference's AVX-512 helper _mm_convert_ps_bf8, src/csrc/xsmm_functors.h:214-217, rounds to fp16 first and then
+// drops the low mantissa byte, i.e. rounds twice, the second time towards zero.)
+__device__ __forceinline__ uint32_t f32_to_e5m2_bits(float f) {
+	uint32_t       u    = __float_as_uint(f);
+	const uint32_t sign = (u >> 24) & 0x80u;
+	u &= 0x7fffffffu;
+	uint32_t r;
+	if(u >= (143u << 23)) r = u > 0x7f800000u ? 0x7fu : 0x7cu;          // |x| >= 2^16, infinity, NaN
+	else if(u < (113u << 23)) r = __float_as_uint(__uint_as_float(u) + __uint_as_float(134u << 23)) - (134u << 23);   // below 2^-14: the adder rounds to the subnormal grid 2^-16
+	else r = (u + ((uint32_t)(15 - 127) << 23) + 0xfffffu + ((u >> 21) & 1u)) >> 21;
+	return r | sign;
+}
+
+template <bool SRC_BF16>
+__global__ void __launch_bounds__(EW_THREADS) cvt_to_e5m2_kernel(const void* __restrict__ src, uint8_t* __restrict__ dst, int64_t n) {
+	const int64_t stride = (int64_t)gridDim.x * EW_THREADS;
+	const int64_t nvec   = n >> 2;
+	const bool    vec    = ((reinterpret_cast<uintptr_t>(src) & (SRC_BF16 ? 7 : 15)) | (reinterpret_cast<uintptr_t>(dst) & 3)) == 0;
+	int64_t       done   = 0;
+	if(vec) {
+		for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < nvec; i += stride) {
+			float f[4];
+			if(SRC_BF16) {
+				const u32x2 w = static_cast<const u32x2*>(src)[i];
+				f[0] = bf16_bits_to_f32(w[0] & 0xffffu), f[1] = bf16_bits_to_f32(w[0] >> 16), f[2] = bf16_bits_to_f32(w[1] & 0xffffu), f[3] = bf16_bits_to_f32(w[1] >> 16);
+			} else {
+				const float4 w = static_cast<const float4*>(src)[i];
+				f[0] = w.x, f[1] = w.y, f[2] = w.z, f[3] = w.w;
+			}
+			reinterpret_cast<uint32_t*>(dst)[i] = f32_to_e5m2_bits(f[0]) | (f32_to_e5m2_bits(f[1]) << 8) | (f32_to_e5m2_bits(f[2]) << 16) | (f32_to_e5m2_bits(f[3]) << 24);
+		}
+		done = nvec << 2;
+	}
+	for(int64_t i = done + (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += stride)
+		dst[i] = (uint8_t)f32_to_e5m2_bits(SRC_BF16 ? bf16_bits_to_f32(static_cast<const uint16_t*>(src)[i]) : static_cast<const float*>(src)[i]);
+}
+
+// e5m2 -> f32 / bf16: the byte is the upper half of the fp16 pattern of the same value (src/csrc/xsmm_functors.h:211-213);
+// exact in both targets (two mantissa bits)
+template <bool TO_BF16>
+__global__ void __launch_bounds__(EW_THREADS) cvt_e5m2_kernel(const uint8_t* __restrict__ src, void* __restrict__ dst, int64_t n) {
+	const int64_t stride = (int64_t)gridDim.x * EW_THREADS;
+	for(int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += stride) {
+		const _Float16 h = __builtin_bit_cast(_Float16, (uint16_t)((uint16_t)src[i] << 8));
+		const float    f = (float)h;
+		if(TO_BF16) static_cast<uint16_t*>(dst)[i] = (uint16_t)f32_to_bf16_bits(f);
+		else static_cast<float*>(dst)[i] = f;
+	}
+}
+
 // ---- per-tensor amax -------------------------------------------------------------------------
 // 16-byte loads, wave then workgroup reduction, one atomic per workgroup (a few hundred atomics on
 // the one result word instead of one per wavefront).
@@ -355,6 +407,14 @@ extern "C" int af3_convert(const void* src, int32_t sd, void* dst, int32_t dd, i
 		hipLaunchKernelGGL(cvt_e4m3_kernel<false>, dim3(ew_blocks((n + 3) / 4)), dim3(EW_THREADS), 0, s, static_cast<const uint8_t*>(src), dst, n);
 	else if(sd == AF3_FP8_E4M3 && dd == AF3_BF16)
 		hipLaunchKernelGGL(cvt_e4m3_kernel<true>, dim3(ew_blocks((n + 3) / 4)), dim3(EW_THREADS), 0, s, static_cast<const uint8_t*>(src), dst, n);
+	else if(sd == AF3_F32 && dd == AF3_FP8_E5M2)
+		hipLaunchKernelGGL(cvt_to_e5m2_kernel<false>, dim3(ew_blocks((n + 3) / 4)), dim3(EW_THREADS), 0, s, src, static_cast<uint8_t*>(dst), n);
+	else if(sd == AF3_BF16 && dd == AF3_FP8_E5M2)
+		hipLaunchKernelGGL(cvt_to_e5m2_kernel<true>, dim3(ew_blocks((n + 3) / 4)), dim3(EW_THREADS), 0, s, src, static_cast<uint8_t*>(dst), n);
+	else if(sd == AF3_FP8_E5M2 && dd == AF3_F32)
+		hipLaunchKernelGGL(cvt_e5m2_kernel<false>, dim3(ew_blocks(n)), dim3(EW_THREADS), 0, s, static_cast<const uint8_t*>(src), dst, n);
+	else if(sd == AF3_FP8_E5M2 && dd == AF3_BF16)
+		hipLaunchKernelGGL(cvt_e5m2_kernel<true>, dim3(ew_blocks(n)), dim3(EW_THREADS), 0, s, static_cast<const uint8_t*>(src), dst, n);
 	else
 		return AF3_ERR_BAD_DTYPE;
 	return launch_status();

@@ -20,6 +20,7 @@ Weights arrive in the layout the reference's callers produce with vnni_repack_te
 and are unpacked once per weight set into the fused matrix (cached per live weight tensor and version).
 """
 import ctypes
+import threading
 import weakref
 from typing import Optional
 
@@ -34,6 +35,7 @@ _FUSED_MIN_GROUPS = 128
 _W_CACHE = {}
 _W_CACHE_MAX = 64
 _ATTEND_TEMPLATES = {}   # (B, N, head, K, dtype code) -> bytes of an af3_dpa_params block with the shape-dependent fields set
+_CACHE_LOCK = threading.RLock()   # guards the two caches' updates (lookups of immutable values need none)
 
 
 def _unpack_panels(w: torch.Tensor, head: int) -> torch.Tensor:
@@ -64,12 +66,13 @@ def _cached(sources, extra, make):
         refs, seen, value = hit
         if all(r() is t for r, t in zip(refs, sources)) and seen == state:
             return value
-    for k in [k for k, (refs, _, _) in list(_W_CACHE.items()) if any(r() is None for r in refs)]:
-        _W_CACHE.pop(k, None)                # derived matrices of weights that no longer exist
-    if len(_W_CACHE) >= _W_CACHE_MAX:
-        _W_CACHE.clear()
-    value = make()
-    _W_CACHE[key] = (tuple(weakref.ref(t) for t in sources), state, value)
+    value = make()                               # (outside the lock: it may launch kernels; two threads that miss together both build it)
+    with _CACHE_LOCK:
+        for k in [k for k, (refs, _, _) in list(_W_CACHE.items()) if any(r() is None for r in refs)]:
+            _W_CACHE.pop(k, None)                # derived matrices of weights that no longer exist
+        if len(_W_CACHE) >= _W_CACHE_MAX:
+            _W_CACHE.clear()
+        _W_CACHE[key] = (tuple(weakref.ref(t) for t in sources), state, value)
     return value
 
 
@@ -78,7 +81,8 @@ def clear_weight_cache() -> None:
     projection, the gated linear unit's weight^T).  Needed only after weights were overwritten in a way that
     does not bump the tensor's version counter, e.g. `module.weight.data.copy_(new)`; ordinary in-place
     updates (`copy_`, `load_state_dict`, optimiser steps) are noticed without it."""
-    _W_CACHE.clear()
+    with _CACHE_LOCK:
+        _W_CACHE.clear()
 
 
 def _fused_weight(ws, head: int, dtype: torch.dtype) -> torch.Tensor:
@@ -155,9 +159,11 @@ def _attend(y: torch.Tensor, B: int, N: int, head: int, mask, bias) -> torch.Ten
         t.io_dtype = t.out_dtype = t.mma_dtype = t.bias_dtype = code
         t.softmax_scale = float(K) ** -0.5
         t.q_descale = t.k_descale = t.v_descale = 1.0
-        if len(_ATTEND_TEMPLATES) >= 256:
-            _ATTEND_TEMPLATES.clear()
-        template = _ATTEND_TEMPLATES[shape_key] = bytes(t)
+        template = bytes(t)
+        with _CACHE_LOCK:
+            if len(_ATTEND_TEMPLATES) >= 256:
+                _ATTEND_TEMPLATES.clear()
+            _ATTEND_TEMPLATES[shape_key] = template
     p = _lib.DpaParams.from_buffer_copy(template)
     p.k, p.v, p.q, p.gate = base, base + K * esz, base + 2 * K * esz, base + 3 * K * esz   # per token and head: (k | v | q | gate)
     p.out = out.data_ptr()

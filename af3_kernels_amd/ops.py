@@ -5,17 +5,20 @@ PyTorch is used for device memory and streams only; every computation below happ
 HIP library.  CPU tensors are rejected: there is no CPU or eager fallback.
 """
 import ctypes
+import threading
 import math
 from typing import Optional
 
 import torch
 
 from . import _lib
-from ._lib import AF3_BF16, AF3_F32, AF3_FP8_E4M3, DpaParams
+from ._lib import AF3_BF16, AF3_F32, AF3_FP8_E4M3, AF3_FP8_E5M2, DpaParams
 
 _DTYPE_CODE = {torch.float32: AF3_F32, torch.bfloat16: AF3_BF16}
 if hasattr(torch, "float8_e4m3fn"):
     _DTYPE_CODE[torch.float8_e4m3fn] = AF3_FP8_E4M3
+if hasattr(torch, "float8_e5m2"):
+    _DTYPE_CODE[torch.float8_e5m2] = AF3_FP8_E5M2
 KERNEL_NAMES = {0: "fp32_fma", 1: "bf16_mfma", 2: "fp8_mfma", 3: "fp32_mfma"}
 
 
@@ -114,6 +117,7 @@ def print_debug_thread_imbalance():
 # attention
 # ------------------------------------------------------------------------------------------
 _PARAM_TEMPLATES = {}   # layout of a call (shapes, strides, dtypes, flags) -> bytes of an af3_dpa_params block with everything but the addresses
+_PARAM_TEMPLATES_LOCK = threading.Lock()   # taken on a miss only: values are immutable bytes, a hit needs no lock
 
 
 def _fill_params(q, k, v, keep, bias, out, mma_dtype, force_generic, descales=None, softmax_scale=None, v_transposed=False, gate=None) -> DpaParams:
@@ -147,9 +151,11 @@ def _fill_params(q, k, v, keep, bias, out, mma_dtype, force_generic, descales=No
         t.reserved = _rows_kernel_hint
         if gate is not None:
             t.gate_stride = (ctypes.c_int64 * 3)(*gate.stride()[:3])
-        if len(_PARAM_TEMPLATES) >= 256:
-            _PARAM_TEMPLATES.clear()
-        template = _PARAM_TEMPLATES[key] = bytes(t)
+        template = bytes(t)
+        with _PARAM_TEMPLATES_LOCK:
+            if len(_PARAM_TEMPLATES) >= 256:
+                _PARAM_TEMPLATES.clear()
+            _PARAM_TEMPLATES[key] = template
     p = DpaParams.from_buffer_copy(template)
     p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     if bias is not None:
@@ -183,9 +189,9 @@ _rows_kernel_hint = 0
 
 
 def set_rows_kernel(mode: str) -> str:
-    """Kernel choice for batched bf16 calls whose shape suits the four-batch-rows-per-wavefront kernel (head_dim <= 32,
-    at least four batch rows): "auto" (default: taken when the launch is large enough to fill the GPU), "always" or
-    "never" (testing aids).  Returns the previous mode."""
+    """Kernel choice for batched bf16 calls that the shared-bias kernel (two to four batch rows per wavefront) can take
+    (head_dim <= 32, at least two batch rows, L <= 4096): "auto" (default: taken when the launch suits it), "always" or
+    "never" (testing aids).  Process-wide, like the reference's module-level switches.  Returns the previous mode."""
     global _rows_kernel_hint
     names = ("auto", "always", "never")
     prev, _rows_kernel_hint = names[_rows_kernel_hint], names.index(mode)
@@ -193,10 +199,11 @@ def set_rows_kernel(mode: str) -> str:
 
 
 def set_exact_bias(flag: bool) -> bool:
-    """With True, batched bf16 calls read the bias in place and add it exactly instead of going
-    through the kernel's fp16 log2-domain bias workspace (whose rounding error in a logit is at most
-    2^-11 * |bias| * log2 e: irrelevant for pair biases of ordinary size, 2 % of a softmax weight
-    at |bias| = 40).  Slower for B >= 2.  Returns the previous setting."""
+    """With True, batched bf16 calls pass no bias workspace: the bias is read in place and added exactly.  That only
+    matters for calls the one-row kernel serves (head_dim 48/64, small launches), whose workspace holds
+    fp16(bias * log2 e) -- a rounding error of at most 2^-11 * |bias| * log2 e per logit: irrelevant for pair biases of
+    ordinary size, 2 % of a softmax weight at |bias| = 40; the shared-bias kernel's workspace is fp32 and exact.
+    Slower for B >= 2.  Returns the previous setting."""
     global _exact_bias
     prev, _exact_bias = _exact_bias, bool(flag)
     return prev
@@ -339,7 +346,8 @@ def selected_kernel(q, k, v, mask, bias, force_generic=False) -> str:
 # ------------------------------------------------------------------------------------------
 def convert(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     """Element-wise cast on the device (tpp::ConvertTPP, src/csrc/xsmm_functors.h:838-885):
-    f32<->bf16 (round to nearest even) and e4m3 -> f32 / bf16."""
+    f32<->bf16 (round to nearest even), e4m3 -> f32 / bf16, and e5m2 <-> f32 / bf16 (the reference's bf8 helpers,
+    src/csrc/xsmm_functors.h:211-217; to e5m2: round to nearest even, overflow to infinity, like torch.float8_e5m2)."""
     _require_device(x)
     x = x.contiguous()
     out = torch.empty(x.shape, dtype=dtype, device=x.device)

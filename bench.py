@@ -27,21 +27,53 @@ PEAK_HBM_GBS = 8000.0
 # runs (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch) scaled by what the same counters read for a device copy of known
 # size.  Each such run is summarised in a file under profiles/ that ends with two machine-readable lines,
 #     traffic_bytes_per_launch: <number>
-#     kernel_sources_sha256: <digest of the kernel sources the run was made with>
-# and the figure is only reported while the sources still have that digest: after any kernel change it is null until
-# the counters are collected again.
+#     kernel_code_sha256: <digest of the kernel sources' code the run was made with>
+# and the figure is only reported while the sources still have that digest -- taken over the code alone, comments and
+# whitespace stripped, so that an edit of the commentary does not invalidate a measurement and nothing ever needs
+# re-stamping by hand: after any change of the kernels' code it is null until the counters are collected again.
 TRAFFIC_PROFILES = {"cfg4": "dpa_rows_bf16_cfg4_hbm_traffic.txt", "cfg2": "dpa_rows_bf16_cfg2_hbm_traffic.txt", "cfg3": "dpa_mfma_bf16_cfg3_hbm_traffic.txt",
                     "cfg5": "dpa_mfma_fp8_cfg5_hbm_traffic.txt", "grid_n768": "grid_attention_one_kernel_grid_n768_hbm_traffic.txt"}
 KERNEL_SOURCES = ("common.hpp", "mfma_helpers.hpp", "dpa_mfma.hip", "dpa_mfma_rows.hip", "dpa_mfma_fp8.hip", "elementwise.hip")
 
 
+def _code_only(text):
+    """C++ source without comments and without whitespace (string and character literals kept as they are), so that
+    the digest below changes with the code and not with its commentary or layout."""
+    out, i, n = [], 0, len(text)
+    while i < n:
+        c = text[i]
+        if c == "/" and i + 1 < n and text[i + 1] == "/":
+            while i < n and text[i] != "\n":
+                i += 1
+        elif c == "/" and i + 1 < n and text[i + 1] == "*":
+            i = text.index("*/", i + 2) + 2
+        elif c in "\"'":
+            j = i + 1
+            while text[j] != c:
+                j += 2 if text[j] == "\\" else 1
+            out.append(text[i:j + 1])
+            i = j + 1
+        elif c.isspace():
+            i += 1
+        else:
+            out.append(c)
+            i += 1
+    return "".join(out)
+
+
+_DIGEST = []
+
+
 def kernel_sources_digest():
     import hashlib
+    if _DIGEST:
+        return _DIGEST[0]
     h = hashlib.sha256()
     for name in KERNEL_SOURCES:
-        with open(os.path.join(ROOT, "af3_kernels_amd", "csrc", name), "rb") as f:
-            h.update(f.read())
-    return h.hexdigest()
+        with open(os.path.join(ROOT, "af3_kernels_amd", "csrc", name)) as f:
+            h.update(_code_only(f.read()).encode())
+    _DIGEST.append(h.hexdigest())
+    return _DIGEST[0]
 
 
 def measured_traffic_bytes(name):
@@ -53,9 +85,9 @@ def measured_traffic_bytes(name):
     fields = {}
     for line in open(path):
         key, sep, val = line.partition(":")
-        if sep and key.strip() in ("traffic_bytes_per_launch", "kernel_sources_sha256"):
+        if sep and key.strip() in ("traffic_bytes_per_launch", "kernel_code_sha256"):
             fields[key.strip()] = val.strip()
-    if fields.get("kernel_sources_sha256") != kernel_sources_digest():
+    if fields.get("kernel_code_sha256") != kernel_sources_digest():
         return None
     try:
         return float(fields["traffic_bytes_per_launch"])
@@ -377,24 +409,33 @@ def main():
         fn = (lambda: af3.dot_product_attention_fp8(q, k, v, mask, bias)) if fp8 else (lambda: af3.dot_product_attention_cpp(q, k, v, mask, bias))
         return fn, ("fp8_mfma" if fp8 else af3.selected_kernel(q, k, v, mask, bias)), (q, k, v, mask, bias)
 
-    def measure(fn, warmup, steps):
-        """`warmup` untimed steps, then exactly `steps` timed steps between synchronisations; per-launch HIP events."""
+    def run_leg(fn, warmup, steps):
+        """`warmup` untimed steps, then exactly `steps` timed steps between synchronisations; per-launch HIP events.  Returns
+        the raw events: reading them out (and everything else on the host) waits until every leg has run, because a host
+        pause of a few milliseconds between two legs is enough for the GPU's clock to dip at the start of the next one."""
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
         for _ in range(warmup):
             o = fn()
         torch.cuda.synchronize()
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
         t0 = time.perf_counter()
         for s, e in evs:
             s.record(stream)
             o = fn()
             e.record(stream)
         torch.cuda.synchronize()
-        wall = (time.perf_counter() - t0) * 1e3 / steps
+        return evs, (time.perf_counter() - t0) * 1e3 / steps, o
+
+    def read_leg(leg):
+        evs, wall, o = leg
+        steps = len(evs)
         per = sorted(s.elapsed_time(e) for s, e in evs)
         k_ms = sum(per) / len(per)          # average duration of one step's launches in the timed region
         step_ms = max(wall, k_ms) if steps < 5 else (evs[0][0].elapsed_time(evs[-1][1]) / steps)
         assert torch.isfinite(o).all()
         return step_ms, k_ms, per
+
+    def measure(fn, warmup, steps):
+        return read_leg(run_leg(fn, warmup, steps))
 
     def roofline_of(c, kernel, kernel_ms, per_launch):
         peak = PEAK_TFLOPS[c.mma_dtype]
@@ -415,28 +456,40 @@ def main():
         return r
 
     # ---- the other named configurations, GPU legs only, in front of the headline leg (default run only) ----
-    # Each leg: 20 untimed + 200 timed steps of the same drop-in call on that configuration's synthetic inputs (well under a
-    # second together).  They run first, in the order of their numbers, so that the headline leg below is what the timed
-    # region of this script ends with; the GPU therefore enters the headline leg busy, not idle.
+    # Each leg: 50 untimed + 500 timed steps of the same drop-in call on that configuration's synthetic inputs (about 0.2 s of
+    # GPU time together).  All inputs, the headline's included, are generated and copied to HBM first, so that the legs run
+    # back to back, in the order of their work per call (cfg3, cfg5, cfg2), and the headline leg -- the largest -- is what the
+    # GPU part of this script ends with.  The GPU therefore enters the headline leg busy, not idle: after any pause of 50 ms
+    # or more this GPU's power management answers the first hundred launches of a heavy kernel with a dip of the clock (per
+    # launch, cfg4 from idle: 420 us, then up to 560 us around the eighth launch, 440 us at the fortieth, 410 us from about
+    # the hundredth on), and the 5 + 20 steps the driver asks for would lie inside that dip.
     others = {}
+    prepared = {}
     if args.case == "cfg4" and not args.only_headline:
-        for name in ("cfg2", "cfg3", "cfg5"):
-            c = CASES[name]
-            fn_c, kern_c, keep = prepare(c)
-            step_ms, k_ms, per = measure(fn_c, 20, 200)
-            rec = {"workload": f"{c.name}: B={c.B} H={c.H} L={c.L} D={c.D} io={c.io_dtype} mma={c.mma_dtype} mask={c.mask_kind}", "steps": 200, "warmup": 20,
-                   "ms_per_step": round(step_ms, 4), "tflops": round(c.flops / (step_ms * 1e-3) / 1e12, 2), "roofline": roofline_of(c, kern_c, k_ms, per)}
-            if name == "cfg5":   # the same shape through the bf16 path (the e4m3 path includes its quantisation launches)
-                q, k, v, mask, bias = keep
-                b_ms, bk_ms, _ = measure(lambda: af3.dot_product_attention_cpp(q, k, v, mask, bias), 20, 200)
-                rec["same_shape_bf16_path"] = {"ms_per_step": round(b_ms, 4), "kernel_ms_avg": round(bk_ms, 4), "kernel": af3.selected_kernel(q, k, v, mask, bias)}
-            others[name] = rec
-            del fn_c, keep
-        torch.cuda.empty_cache()
-
+        for name in ("cfg3", "cfg5", "cfg2"):
+            prepared[name] = prepare(CASES[name])
     fn, kernel, _inputs = prepare(case)
+    torch.cuda.synchronize()
+    legs = {}
+    for name, (fn_c, kern_c, keep) in prepared.items():
+        legs[name] = run_leg(fn_c, 50, 500)
+        if name == "cfg5":   # the same shape through the bf16 path (the e4m3 path includes its quantisation launches)
+            q5, k5, v5, mask5, bias5 = keep
+            legs["cfg5_bf16"] = run_leg(lambda: af3.dot_product_attention_cpp(q5, k5, v5, mask5, bias5), 50, 500)
+
     # ---- the headline leg: exactly the W untimed and K timed steps asked for ----
-    ms_per_step, kernel_ms, per_launch = measure(fn, args.warmup, args.steps)
+    headline = run_leg(fn, args.warmup, args.steps)
+    ms_per_step, kernel_ms, per_launch = read_leg(headline)
+    for name, (fn_c, kern_c, keep) in prepared.items():
+        c = CASES[name]
+        step_ms, k_ms, per = read_leg(legs[name])
+        rec = {"workload": f"{c.name}: B={c.B} H={c.H} L={c.L} D={c.D} io={c.io_dtype} mma={c.mma_dtype} mask={c.mask_kind}", "steps": 500, "warmup": 50,
+               "ms_per_step": round(step_ms, 4), "tflops": round(c.flops / (step_ms * 1e-3) / 1e12, 2), "roofline": roofline_of(c, kern_c, k_ms, per)}
+        if name == "cfg5":
+            q5, k5, v5, mask5, bias5 = keep
+            b_ms, bk_ms, _ = read_leg(legs["cfg5_bf16"])
+            rec["same_shape_bf16_path"] = {"ms_per_step": round(b_ms, 4), "kernel_ms_avg": round(bk_ms, 4), "kernel": af3.selected_kernel(q5, k5, v5, mask5, bias5)}
+        others[name] = rec
     # A short run (the driver's 5 + 20 steps last 10 ms) sits inside the GPU's power-management transient: the clock is
     # still moving when the timed steps start.  As a second, separately labelled figure the GPU is then kept busy with the
     # same call for a fixed 0.4 s and the same W + K protocol is repeated (`settled_pass`): the rate a model sees that calls
@@ -453,6 +506,38 @@ def main():
         settled = {"ms_per_step": round(s_ms, 4), "kernel_ms_avg": round(sk_ms, 4), "tflops": round(case.flops / (s_ms * 1e-3) / 1e12, 2),
                    "roofline_frac": round(case.flops / (sk_ms * 1e-3) / 1e12 / PEAK_TFLOPS[case.mma_dtype], 4) if case.name not in ("cfg3", "cfg5") else None,
                    "untimed_calls_before": args.warmup + args.steps + n_settle + args.warmup, "settle_seconds": 0.4}
+
+    # The small configurations' calls are shorter than the host's launch path (cfg3: a 10-us kernel behind 18 us of Python and
+    # launch), so their event-bracketed figures above include the dispatch gaps around a lone kernel.  Second figure for them:
+    # ten calls recorded into a HIP graph and the graph replayed, which keeps the GPU fed back to back.
+    def graph_ms_per_call(fn_c, calls=10, replays=40):
+        side = torch.cuda.Stream(dev)
+        side.wait_stream(stream)
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                fn_c()
+        stream.wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(calls):
+                fn_c()
+        for _ in range(5):
+            g.replay()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        for _ in range(replays):
+            g.replay()
+        b.record(stream)
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / (calls * replays)
+
+    for name, (fn_c, kern_c, keep) in prepared.items():
+        others[name]["graph_replay_ms_per_call"] = round(graph_ms_per_call(fn_c), 4)
+        if name == "cfg5":
+            q5, k5, v5, mask5, bias5 = keep
+            others[name]["same_shape_bf16_path"]["graph_replay_ms_per_call"] = round(graph_ms_per_call(lambda: af3.dot_product_attention_cpp(q5, k5, v5, mask5, bias5)), 4)
 
     tflops = case.flops / (ms_per_step * 1e-3) / 1e12
     peak = PEAK_TFLOPS[case.mma_dtype]

@@ -38,7 +38,8 @@ typedef enum af3_status {
 typedef enum af3_dtype {
 	AF3_F32      = 0,
 	AF3_BF16     = 1,
-	AF3_FP8_E4M3 = 2 /* OCP e4m3fn: bias 7, max 448, no infinity */
+	AF3_FP8_E4M3 = 2, /* OCP e4m3fn: bias 7, max 448, no infinity */
+	AF3_FP8_E5M2 = 3  /* OCP e5m2: bias 15, max 57344, infinities and NaN (af3_convert only) */
 } af3_dtype;
 
 #define AF3_DPA_MAX_HEAD_DIM 128
@@ -97,20 +98,32 @@ typedef struct af3_dpa_params {
 	float          k_descale;
 	float          v_descale;
 	int32_t        force_generic; /* non-zero: always take the fp32-FMA kernel (testing aid) */
-	int32_t        reserved;      /* kernel hint for batched bf16 calls that suit the four-batch-rows-per-wavefront kernel
-	                                 (head_dim <= 32, B >= 4): 0 = chosen by launch size, 1 = always, 2 = never (testing aids) */
+	int32_t        reserved;      /* kernel hint for batched bf16 calls that the shared-bias kernel (two to four batch rows per
+	                                 wavefront) can take (head_dim <= 32, B >= 2, L <= 4096): 0 = chosen by launch size, 1 = always,
+	                                 2 = never (testing aids) */
 	/* Optional: 3 device floats {q_descale, k_descale, v_descale} as written by
 	 * af3_quantize_fp8_e4m3; when non-NULL they override the three host values above, so a
 	 * quantise -> attend sequence needs no device-to-host copy. */
 	const float*   device_descales;
 	/* Optional scratch in device memory, at least af3_dpa_workspace_bytes() long and 256-byte
-	 * aligned.  With it the bf16 kernel first rewrites the bias once (scaled by log2 e and laid
-	 * out in matrix-operand order, shared by all B batch rows) and then runs its fastest variant;
-	 * without it (NULL) the bias is read in place.  Contents are overwritten by every call.
-	 * Precision: the rewritten bias is fp16(bias * log2 e), i.e. each logit carries a rounding
-	 * error of at most 2^-11 * |bias| * 1.4427 (0.4 % of a softmax weight at |bias| = 8, 2 % at
-	 * |bias| = 40; values beyond +-45400 saturate).  Callers whose biases are that large and who
-	 * need them exact pass workspace = NULL: the in-place variant adds the bf16 bias exactly. */
+	 * aligned.  With it a bf16 call of two or more batch rows may first rewrite the bias once
+	 * (scaled by log2 e and laid out in matrix-operand order, shared by all B batch rows) and
+	 * then run its fastest variant; without it (NULL) the bias is read in place.  Contents are
+	 * overwritten by every call.  What the rewritten bias holds depends on the kernel the call
+	 * takes (af3_dpa_workspace_bytes() returns the size for that kernel):
+	 *  - the shared-bias kernel (head_dim <= 32, batch rows that share the bias; the headline
+	 *    path): fp32(bias * log2 e) in accumulator order, 4 bytes per logit, exact for bf16 and
+	 *    fp32 biases alike; entries below -2^17 (log2 units), -inf and NaN become -2^17.
+	 *  - the one-row kernel (head_dim 48/64, small launches): fp16(bias * log2 e), 2 bytes per
+	 *    logit: each logit carries a rounding error of at most 2^-11 * |bias| * 1.4427 (0.4 % of
+	 *    a softmax weight at |bias| = 8, 2 % at |bias| = 40; values beyond +-45400 saturate).
+	 *    Callers whose biases are that large and who need them exact pass workspace = NULL.
+	 * In place, a bf16 bias is added exactly; the shared-bias kernel clamps entries below -2^16
+	 * (and -inf) to -2^16 first, the one-row kernel those below -2^126.  A clamped entry has
+	 * weight exactly 0 beside any ordinary logit; a query row made of nothing but clamped entries
+	 * comes out as the softmax of q.k alone over its live keys.  (Add-then-softmax in the
+	 * reference differs only where a row mixes entries on both sides of the clamp that are all
+	 * hugely negative, e.g. -1e9 beside -70000: there the reference lets the larger one win.) */
 	void*          workspace;
 	int64_t        workspace_bytes;
 	/* Optional (fp8 only): residual tensors q_lo = e4m3(q*s - q8), k_lo = e4m3(k*s - k8) at the same
@@ -155,7 +168,10 @@ int64_t af3_dpa_workspace_bytes(const af3_dpa_params* params);
  * AF3_STATIC_SCRATCH_BYTES that is part of the library's code object, one copy per GPU for the life of the process.
  * The call allocates and frees nothing.  A call that needs more scratch than that returns AF3_ERR_SCRATCH_LIMIT and
  * enqueues nothing (H * ceil(L/32)^2 * 4 KiB must fit: e.g. 4 heads up to L = 1024, 16 heads up to L = 512); a call
- * that needs none (one batch row, no bias, float32 or fp8 arithmetic) is af3_dpa_forward.  Every call on one GPU shares
+ * that needs none (one batch row, no bias, float32 or fp8 arithmetic) is af3_dpa_forward.  The first call on a device
+ * looks up the array's address and the device's properties and sets kernel attributes (host-side work that loads the
+ * code object): make one call, of any size, on each device OUTSIDE stream capture before the first captured one.  The
+ * array costs every GPU the process runs this library on 16 MiB of device memory, used or not.  Every call on one GPU shares
  * that GPU's array and overwrites all of it that it reads, so nothing needs clearing between calls, but calls that
  * overlap in time on one GPU (two streams, two threads) race on it: serialise them, or give af3_dpa_forward separate
  * workspaces instead.
@@ -172,7 +188,11 @@ int af3_dpa_select_kernel(const af3_dpa_params* params);
  * Element-wise dtype conversion, n contiguous elements, round-to-nearest-even.
  * Replaces: tpp::ConvertTPP (src/csrc/xsmm_functors.h:838-885) and the AVX-512 helpers
  * _mm512_convert_bf_ps / _mm256_convert_ps_bf (src/csrc/xsmm_functors.h:139-145).
- * Supported pairs: f32->bf16, bf16->f32, fp8_e4m3->f32, fp8_e4m3->bf16.
+ * Supported pairs: f32->bf16, bf16->f32, fp8_e4m3->f32, fp8_e4m3->bf16, and the e5m2 pair of the reference's
+ * _mm512_convert_bf8_ps / _mm_convert_ps_bf8 (src/csrc/xsmm_functors.h:211-217): fp8_e5m2->f32, fp8_e5m2->bf16 (exact),
+ * f32->fp8_e5m2 and bf16->fp8_e5m2, rounded to nearest even in one step with overflow to infinity (torch.float8_e5m2's
+ * rule; the reference's helper rounds to fp16 first and then truncates the low byte, which differs in the last bit for
+ * about three values in eight).
  */
 int af3_convert(const void* src, int32_t src_dtype, void* dst, int32_t dst_dtype, int64_t n, void* hip_stream);
 

@@ -120,6 +120,92 @@ float af3o_e4m3_bits_to_f32(uint8_t b) {
 	return s ? -v : v;
 }
 
+/*
+ * e5m2 ("bf8"): fp16's exponent range with two mantissa bits, infinities and NaN like IEEE.
+ * af3o_e5m2_bits_to_f32: _mm512_convert_bf8_ps, xsmm_functors.h:211-213 -- the byte is the upper half of the fp16
+ * pattern of the same value.
+ * af3o_f32_to_e5m2_bits_reference: _mm_convert_ps_bf8, xsmm_functors.h:214-217 -- round to fp16 (nearest even), then
+ * arithmetic shift right by 8, i.e. the low mantissa byte is dropped: two roundings, the second towards zero in magnitude
+ * (the shift acts on the sign-magnitude pattern, so the sign bit is kept and the magnitude truncated).
+ * af3o_f32_to_e5m2_bits: one rounding to nearest even from fp32, overflow to infinity -- the rule of the shipped
+ * converter; pinned against torch.float8_e5m2.
+ */
+static uint16_t f32_to_f16_bits_rne(float f) {
+	uint32_t u;
+	memcpy(&u, &f, 4);
+	uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+	uint32_t a    = u & 0x7fffffffu;
+	if(a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);
+	if(a >= 0x47800000u) return (uint16_t)(sign | 0x7c00u); /* |x| >= 65536 (values that round up to it are caught below) */
+	float af;
+	memcpy(&af, &a, 4);
+	if(af < 6.103515625e-05f) { /* below 2^-14: quantum 2^-24 */
+		float q = nearbyintf(af * 16777216.0f);
+		return (uint16_t)(sign | (uint16_t)q); /* q == 1024 is the first normal */
+	}
+	int   e;
+	float m = frexpf(af, &e);
+	int   E = e - 1;
+	float q = nearbyintf((2.0f * m - 1.0f) * 1024.0f);
+	if(q >= 1024.0f) {
+		q = 0.0f;
+		E += 1;
+	}
+	if(E > 15) return (uint16_t)(sign | 0x7c00u);
+	return (uint16_t)(sign | (uint16_t)((E + 15) << 10) | (uint16_t)q);
+}
+uint8_t af3o_f32_to_e5m2_bits_reference(float f) {
+	return (uint8_t)(f32_to_f16_bits_rne(f) >> 8);
+}
+uint8_t af3o_f32_to_e5m2_bits(float f) {
+	uint32_t u;
+	memcpy(&u, &f, 4);
+	uint8_t  sign = (uint8_t)((u >> 24) & 0x80u);
+	uint32_t a    = u & 0x7fffffffu;
+	if(a > 0x7f800000u) return (uint8_t)(sign | 0x7fu);
+	float af;
+	memcpy(&af, &a, 4);
+	if(af >= 65536.0f) return (uint8_t)(sign | 0x7cu);
+	if(af < 6.103515625e-05f) { /* below 2^-14: quantum 2^-16 */
+		float q = nearbyintf(af * 65536.0f);
+		return (uint8_t)(sign | (uint8_t)q);
+	}
+	int   e;
+	float m = frexpf(af, &e);
+	int   E = e - 1;
+	float q = nearbyintf((2.0f * m - 1.0f) * 4.0f);
+	if(q >= 4.0f) {
+		q = 0.0f;
+		E += 1;
+	}
+	if(E > 15) return (uint8_t)(sign | 0x7cu);
+	return (uint8_t)(sign | (uint8_t)((E + 15) << 2) | (uint8_t)q);
+}
+float af3o_e5m2_bits_to_f32(uint8_t b) {
+	int   s = b & 0x80;
+	int   E = (b >> 2) & 0x1f;
+	int   m = b & 3;
+	float v;
+	if(E == 0x1f) {
+		v = m ? NAN : INFINITY;
+	} else if(E == 0) {
+		v = (float)m * 1.52587890625e-05f; /* m * 2^-16 */
+	} else {
+		v = ldexpf(1.0f + (float)m / 4.0f, E - 15);
+	}
+	return s ? -v : v;
+}
+void af3o_convert_f32_to_e5m2(const float* in, uint8_t* out, int64_t n, int reference_rule) {
+	for(int64_t i = 0; i < n; i++) {
+		out[i] = reference_rule ? af3o_f32_to_e5m2_bits_reference(in[i]) : af3o_f32_to_e5m2_bits(in[i]);
+	}
+}
+void af3o_convert_e5m2_to_f32(const uint8_t* in, float* out, int64_t n) {
+	for(int64_t i = 0; i < n; i++) {
+		out[i] = af3o_e5m2_bits_to_f32(in[i]);
+	}
+}
+
 /* ConvertTPP::ref, xsmm_functors.h:867-873: out[i] = (Tout)in[i]. Array forms for the tests. */
 void af3o_convert_f32_to_bf16(const float* in, uint16_t* out, int64_t n) {
 	for(int64_t i = 0; i < n; i++) {

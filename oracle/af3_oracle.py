@@ -46,6 +46,8 @@ def lib():
         L.af3o_quantize_e4m3_pow2.argtypes = [fp, u8, i64, ctypes.c_float]
         L.af3o_quantize_e4m3_pow2.restype = ctypes.c_float
         L.af3o_dequantize_e4m3.argtypes = [u8, fp, i64, ctypes.c_float]
+        L.af3o_convert_f32_to_e5m2.argtypes = [fp, u8, i64, ctypes.c_int]
+        L.af3o_convert_e5m2_to_f32.argtypes = [u8, fp, i64]
         L.af3o_f32_to_e4m3_bits.argtypes = [ctypes.c_float]
         L.af3o_f32_to_e4m3_bits.restype = ctypes.c_uint8
         L.af3o_e4m3_bits_to_f32.argtypes = [ctypes.c_uint8]
@@ -183,6 +185,22 @@ def bf16_bits_to_f32(h):
 
 def round_bf16(x):
     return bf16_bits_to_f32(f32_to_bf16_bits(x))
+
+
+def f32_to_e5m2_bits(x, reference_rule=False):
+    """fp32 -> e5m2 bits: one rounding to nearest even with overflow to infinity (the shipped converter's rule), or with
+    reference_rule the two-step rule of the reference's _mm_convert_ps_bf8 (fp16 nearest-even, then the low byte dropped)."""
+    x, xp = _f(x)
+    out = np.empty(x.shape, np.uint8)
+    lib().af3o_convert_f32_to_e5m2(xp, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), x.size, int(bool(reference_rule)))
+    return out
+
+
+def e5m2_bits_to_f32(b):
+    b = np.ascontiguousarray(b, np.uint8)
+    out = np.empty(b.shape, np.float32)
+    lib().af3o_convert_e5m2_to_f32(b.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), b.size)
+    return out
 
 
 def quantize_e4m3(x):

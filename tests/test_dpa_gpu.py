@@ -698,6 +698,30 @@ def test_convert_matches_torch_casts(af3):
     assert torch.equal(af3.convert(codes.cuda(), torch.bfloat16).cpu()[~nan], want.to(torch.bfloat16)[~nan])
 
 
+def test_convert_e5m2_matches_torch_casts_bit_for_bit(af3):
+    """The e5m2 pair of the cast functors (src/csrc/xsmm_functors.h:211-217): every code decodes like torch.float8_e5m2, and
+    fp32 / bf16 values -- any bit pattern, ties between representable values and their neighbours, subnormals, the overflow
+    threshold, infinities -- encode to exactly torch's bits (one rounding to nearest even, overflow to infinity)."""
+    codes = torch.arange(256, dtype=torch.uint8)
+    want = codes.view(torch.float8_e5m2).float()
+    nan = torch.isnan(want)
+    got = af3.convert(codes.view(torch.float8_e5m2).cuda(), torch.float32).cpu()
+    assert torch.equal(torch.isnan(got), nan) and torch.equal(got[~nan], want[~nan])
+    got16 = af3.convert(codes.view(torch.float8_e5m2).cuda(), torch.bfloat16).cpu()
+    assert torch.equal(got16[~nan].float(), want[~nan])
+    g = torch.Generator().manual_seed(5)
+    bits = torch.randint(-2 ** 31, 2 ** 31 - 1, (300001,), generator=g, dtype=torch.int64).to(torch.int32).view(torch.float32)
+    finite = want[torch.isfinite(want)].sort().values
+    mid = (finite[:-1] + finite[1:]) / 2
+    x = torch.cat([bits, torch.randn(100003, generator=g) * 3, mid, torch.nextafter(mid, torch.tensor(float("inf"))), torch.nextafter(mid, torch.tensor(float("-inf"))),
+                   torch.tensor([0.0, -0.0, 2.0 ** -17, 2.0 ** -16, 1.5 * 2.0 ** -16, 57344.0, 61439.99, 61440.0, 65535.0, 65536.0, float("inf"), float("-inf")])])
+    x = x[~torch.isnan(x)]
+    for src in (x, x.to(torch.bfloat16)):
+        got = af3.convert(src.cuda(), torch.float8_e5m2).cpu().view(torch.uint8)
+        assert torch.equal(got, src.to(torch.float8_e5m2).view(torch.uint8))
+    assert (af3.convert(torch.tensor([float("nan")]).cuda(), torch.float8_e5m2).cpu().view(torch.uint8) & 0x7f).item() > 0x7c
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_quantize_fp8_per_tensor_scale(af3, dtype):
     g = torch.Generator().manual_seed(4)

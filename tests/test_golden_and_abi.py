@@ -411,3 +411,44 @@ def test_workspace_query_follows_the_batch_size_at_which_a_bias_rewrite_pays_off
     assert call(64, 4, 768, bias=0x1008) == rewrite(4, 768)          # rows only 8-byte aligned: not staged
     assert call(64, 4, 396) == rewrite(4, 396)                       # L % 8 != 0: not staged
     assert call(64, 4, 768, bias=None) == 0 and call(1, 16, 768) == 0
+
+
+def test_argument_blocks_and_weight_cache_can_be_built_from_several_threads():
+    """The Python side promises that calls may come from several threads: the per-layout templates of the argument block and
+    the derived-weight cache are shared, filled on a miss and cleared when full.  Eight threads build blocks for more
+    layouts than the template cache holds (so it is cleared under their feet) and look up derived weights of tensors
+    that come and go; every block must describe exactly the tensors it was built for."""
+    import threading
+    from af3_kernels_amd import fused, ops, _lib
+    errors = []
+
+    def worker(seed):
+        try:
+            g = torch.Generator().manual_seed(seed)
+            for i in range(300):
+                B, H, L, D = 1 + (seed + i) % 5, 1 + i % 7, 8 * (1 + (i * 7 + seed) % 40), 8 * (1 + i % 4)
+                q = torch.empty(B, H, L, D, dtype=torch.bfloat16)
+                k, v, out = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+                bias = torch.empty(H, L, L, dtype=torch.bfloat16)
+                keep = torch.ones(B, L, dtype=torch.uint8)
+                p = ops._fill_params(q, k, v, keep, bias, out, _lib.AF3_BF16, False)
+                assert (p.B, p.H, p.L, p.D) == (B, H, L, D)
+                assert tuple(p.q_stride) == tuple(q.stride()[:3]) and tuple(p.bias_stride) == (L * L, L)
+                assert p.q == q.data_ptr() and p.k == k.data_ptr() and p.v == v.data_ptr() and p.out == out.data_ptr()
+                assert p.bias == bias.data_ptr() and p.key_mask == keep.data_ptr() and p.key_mask_stride_b == (0 if B == 1 else L)
+                assert abs(p.softmax_scale - D ** -0.5) < 1e-7
+                w = torch.randn(4 + i % 3, 5, generator=g)
+                got = fused._cached((w,), ("t", seed % 2), lambda: w.t().contiguous())
+                assert torch.equal(got, w.t())
+                if i % 50 == 49:
+                    fused.clear_weight_cache()
+        except Exception as e:   # noqa: BLE001 -- reported by the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(s,)) for s in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors[:3]
+    assert len(ops._PARAM_TEMPLATES) <= 256 and len(fused._W_CACHE) <= fused._W_CACHE_MAX

@@ -190,6 +190,35 @@ def test_e4m3_matches_torch_for_every_code_and_random_values(oracle):
     assert lib.af3o_f32_to_e4m3_bits(1e6) == 0x7E and lib.af3o_f32_to_e4m3_bits(-1e6) == 0xFE  # saturating
 
 
+def test_e5m2_matches_torch_for_every_code_and_both_rounding_rules(oracle):
+    """Decoding: every code against torch.float8_e5m2.  Encoding, one-step rule (the shipped converter's): random values over
+    the whole range, ties, subnormals, the overflow threshold and non-finite inputs against torch's cast.  Encoding, the
+    reference's two-step rule (src/csrc/xsmm_functors.h:214-217): torch's fp16 cast followed by dropping the low byte."""
+    codes = np.arange(256, dtype=np.uint8)
+    want = torch.from_numpy(codes).view(torch.float8_e5m2).float().numpy()
+    got = oracle.e5m2_bits_to_f32(codes)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(got[~np.isnan(got)], want[~np.isnan(want)])
+    rng = np.random.default_rng(52)
+    bits = rng.integers(0, 2 ** 32, 200000, dtype=np.uint64).astype(np.uint32)           # any fp32 pattern
+    grid = (codes.astype(np.uint16) << 8).view(np.float16).astype(np.float32)            # the representable values ...
+    finite = grid[np.isfinite(grid)]
+    ties = np.concatenate([(finite[:-1] + finite[1:]) / 2, np.nextafter(finite, np.float32(np.inf)), np.nextafter(finite, np.float32(-np.inf))])   # ... midpoints and neighbours
+    x = np.concatenate([bits.view(np.float32), rng.standard_normal(50000).astype(np.float32) * 3, ties.astype(np.float32),
+                        np.array([0.0, -0.0, 2 ** -17, 2 ** -16, 1.5 * 2 ** -16, 57344, 61439.99, 61440, 65535, 65536, np.inf, -np.inf, np.nan], np.float32)])
+    want = torch.from_numpy(x).to(torch.float8_e5m2).view(torch.uint8).numpy()
+    got = oracle.f32_to_e5m2_bits(x)
+    nan = np.isnan(x)
+    assert np.array_equal(got[~nan], want[~nan])
+    assert ((got[nan] & 0x7f) > 0x7c).all()                                               # NaN stays NaN (payload free)
+    two_step = (torch.from_numpy(x).to(torch.float16).view(torch.int16).numpy().view(np.uint16) >> 8).astype(np.uint8)
+    ref = oracle.f32_to_e5m2_bits(x, reference_rule=True)
+    assert np.array_equal(ref[~nan], two_step[~nan])
+    # the two rules differ only by the last bit, and only where the dropped byte rounds up
+    d = got[~nan].astype(np.int16) - ref[~nan].astype(np.int16)
+    assert set(np.unique(d)) <= {0, 1}
+
+
 def test_quantize_e4m3_uses_per_tensor_amax_scale(oracle):
     rng = np.random.default_rng(13)
     x = rng.standard_normal(4096).astype(np.float32) * 3

@@ -58,6 +58,7 @@ SYMBOLS = {
     "af3_grid_attention_supported": (ctypes.c_int, [ctypes.POINTER(GridAttentionParams)]),
     "af3_layernorm_pair_bias": (ctypes.c_int, [vp, ctypes.POINTER(i64), vp, vp, f32, vp, vp, vp, ctypes.POINTER(i64), i64, i64, i64, i64, i32, vp]),
     "af3_gated_linear_unit": (ctypes.c_int, [vp, vp, vp, i64, i64, i64, i32, vp]),
+    "af3_silu_mul": (ctypes.c_int, [vp, vp, i64, i64, i32, vp]),
     "af3_linear": (ctypes.c_int, [vp, vp, vp, i64, i64, i64, i32, vp]),
     "af3_convert": (ctypes.c_int, [vp, i32, vp, i32, i64, vp]),
     "af3_amax": (ctypes.c_int, [vp, i32, i64, vp, vp]),

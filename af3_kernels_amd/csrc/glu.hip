@@ -195,6 +195,40 @@ int launch_rows_times_weights(const void* x, const void* weight_t, void* out, in
 
 }  // namespace
 
+namespace {
+
+// out[m][n] = silu(y[m][n]) * y[m][N + n]: the gate of a gated linear unit whose [M, 2N] product came from a library GEMM
+// (the one-kernel form above takes the reference's own shapes; this closes every other shape without an elementwise
+// pass of a second framework).  Arithmetic as in src/csrc/gated_linear_unit.cpp:56-61: silu in fp32 on the stored value.
+template <bool F32>
+__global__ void __launch_bounds__(256) silu_mul_kernel(const void* __restrict__ y, void* __restrict__ out, int64_t M, int64_t N) {
+	const int64_t total = M * N, stride = (int64_t)gridDim.x * 256;
+	for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+		const int64_t m = i / N, n = i - m * N;
+		float         a, b;
+		if(F32) a = static_cast<const float*>(y)[m * 2 * N + n], b = static_cast<const float*>(y)[m * 2 * N + N + n];
+		else a = bf16_bits_to_f32(static_cast<const uint16_t*>(y)[m * 2 * N + n]), b = bf16_bits_to_f32(static_cast<const uint16_t*>(y)[m * 2 * N + N + n]);
+		float g = a / (1.f + __expf(-a));
+		if(!F32) g = bf16_bits_to_f32(f32_to_bf16_bits(g));   // (the reference rounds silu's result to the storage type before the product)
+		const float o = g * b;
+		if(F32) static_cast<float*>(out)[i] = o;
+		else static_cast<uint16_t*>(out)[i] = (uint16_t)f32_to_bf16_bits(o);
+	}
+}
+
+}  // namespace
+
+extern "C" int af3_silu_mul(const void* y, void* out, int64_t M, int64_t N, int32_t dtype, void* stream) {
+	if(!y || !out) return AF3_ERR_NULL_POINTER;
+	if(M <= 0 || N <= 0 || M > ((int64_t)1 << 40) || N > ((int64_t)1 << 30)) return AF3_ERR_BAD_SHAPE;
+	if(dtype != AF3_BF16 && dtype != AF3_F32) return AF3_ERR_BAD_DTYPE;
+	const int64_t  blocks = (M * N + 255) / 256;
+	const unsigned g      = (unsigned)(blocks > 256 * 32 ? 256 * 32 : blocks);
+	if(dtype == AF3_F32) hipLaunchKernelGGL(silu_mul_kernel<true>, dim3(g), dim3(256), 0, static_cast<hipStream_t>(stream), y, out, M, N);
+	else hipLaunchKernelGGL(silu_mul_kernel<false>, dim3(g), dim3(256), 0, static_cast<hipStream_t>(stream), y, out, M, N);
+	return launch_status();
+}
+
 extern "C" int af3_gated_linear_unit(const void* x, const void* weight_t, void* out, int64_t M, int64_t K, int64_t N, int32_t dtype, void* stream) {
 	return launch_rows_times_weights(x, weight_t, out, M, K, N, dtype, true, stream);
 }

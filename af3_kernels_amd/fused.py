@@ -304,16 +304,23 @@ def self_attention_cpp(
 
 def layernorm_pair_bias(pair: torch.Tensor, ln_weight: torch.Tensor, ln_bias: torch.Tensor, eps: float, proj_weight: torch.Tensor):
     """act_norm + pair_bias_projection + permute(2, 0, 1) of the reference module (src/af3_kernels/Attention.py:51-52) in
-    one pass over the pair tensor: returns (normed [N1, N2, C], bias [head, N1, N2]).  One HIP kernel for bfloat16 pairs
-    with 128 channels and 4 heads; the same torch ops as the reference otherwise."""
+    one pass over the pair tensor: returns (normed [N1, N2, C], bias [head, N1, N2]).  One HIP kernel: a specialised one
+    for bfloat16 pairs with 128 channels and 4 heads (the pair tensor's own shape), one wavefront per token for any other
+    channel and head count (C <= 2048) in bfloat16 or float32.  Parameters in another dtype are cast to the pair's."""
     ops._require_device(pair, ln_weight, ln_bias, proj_weight)
+    if pair.dim() != 3 or proj_weight.dim() != 2 or proj_weight.shape[1] != pair.shape[-1] or ln_weight.numel() != pair.shape[-1] or ln_bias.numel() != pair.shape[-1]:
+        raise ValueError(f"pair must be [N1, N2, C] with ln_weight, ln_bias [C] and proj_weight [head, C], got {tuple(pair.shape)}, {tuple(ln_weight.shape)}, "
+                         f"{tuple(ln_bias.shape)}, {tuple(proj_weight.shape)}")
+    if pair.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError(f"unsupported dtype {pair.dtype}: float32 or bfloat16")
     head, C = proj_weight.shape
-    ln_weight, ln_bias, proj_weight = ln_weight.contiguous(), ln_bias.contiguous(), proj_weight.contiguous()
-    if not (pair.dtype == torch.bfloat16 and pair.dim() == 3 and C == 128 and head == 4 and pair.shape[-1] == C and pair.numel() > 0
-            and ln_weight.dtype == ln_bias.dtype == proj_weight.dtype == torch.bfloat16 and pair.stride(2) == 1 and pair.stride(0) % 8 == 0
-            and pair.stride(1) % 8 == 0 and all(t.data_ptr() % 16 == 0 for t in (pair, ln_weight, ln_bias, proj_weight))):
-        normed = torch.nn.functional.layer_norm(pair, (C,), ln_weight, ln_bias, eps)
-        return normed, torch.nn.functional.linear(normed, proj_weight).permute(2, 0, 1)
+    if C > 2048 or head > 64 or (2 + head) * C * 4 > 160 * 1024 - 1024:
+        raise ValueError(f"layernorm_pair_bias takes at most 2048 channels and (2 + head) * C * 4 bytes of LDS, got C={C}, head={head}")
+    ln_weight, ln_bias, proj_weight = [t.to(pair.dtype).contiguous() for t in (ln_weight, ln_bias, proj_weight)]
+    if pair.stride(2) != 1:
+        pair = pair.contiguous()
+    if pair.numel() == 0:
+        return torch.empty_like(pair), torch.empty(head, *pair.shape[:2], dtype=pair.dtype, device=pair.device)
     n_i, n_j = pair.shape[:2]
     normed = torch.empty(n_i, n_j, C, dtype=pair.dtype, device=pair.device)
     bias = torch.empty(head, n_i, n_j, dtype=pair.dtype, device=pair.device)
@@ -399,17 +406,25 @@ def gated_linear_unit_cpp(x: torch.Tensor, weight: torch.Tensor, vnni_repacked: 
     """silu(x @ W[:, :N]) * (x @ W[:, N:]) -- drop-in for the reference's gated_linear_unit_cpp (src/af3_kernels/__init__.py:
     21-28; src/csrc/gated_linear_unit.cpp:20-80).  x [..., K], weight [K, 2N] (plain or VNNI-repacked with N_BLK); returns
     [..., N] in x's dtype.  bfloat16 with K = 64 or 128 and N % 32 == 0 is one HIP kernel (the [.., 2N] product is never
-    stored); other shapes run the formula's torch ops on the device.  M_BLK and N_BLK are CPU blocking sizes (N_BLK also
-    names the panel width of a repacked weight) and change nothing else."""
+    stored); other shapes (bfloat16 or float32) are a library GEMM for x @ W followed by the silu-and-multiply kernel
+    (af3_silu_mul).  M_BLK and N_BLK are CPU blocking sizes (N_BLK also names the panel width of a repacked weight) and
+    change nothing else."""
     ops._require_device(x, weight)
     if weight.dim() != 2 or weight.shape[0] != x.shape[-1] or weight.shape[1] % 2 != 0:
         raise ValueError(f"weight must be [K, 2N] with K = x.shape[-1] = {x.shape[-1]}, got {tuple(weight.shape)}")
     K, N = weight.shape[0], weight.shape[1] // 2
     lead = x.shape[:-1]
-    if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and K in (64, 128) and N % 32 == 0 and x.numel() > 0):
-        y = torch.matmul(x, _plain_weight(weight, vnni_repacked, N_BLK).to(x.dtype))
-        a, b = torch.chunk(y, 2, dim=-1)
-        return torch.nn.functional.silu(a) * b
+    if x.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError(f"unsupported dtype {x.dtype}: float32 or bfloat16")
+    if x.numel() == 0:
+        return torch.empty(*lead, N, dtype=x.dtype, device=x.device)
+    if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and K in (64, 128) and N % 32 == 0):
+        w = _cached((weight,), (bool(vnni_repacked), N_BLK, x.dtype, "glu_plain"), lambda: _plain_weight(weight, vnni_repacked, N_BLK).to(x.dtype).contiguous())
+        y = torch.matmul(x.reshape(-1, K), w)                       # [M, 2N]: the library GEMM (hipBLASLt)
+        out = torch.empty(y.shape[0], N, dtype=x.dtype, device=x.device)
+        with ops._on_device(x.device):
+            _lib.check(_lib.load().af3_silu_mul(y.data_ptr(), out.data_ptr(), y.shape[0], N, ops._DTYPE_CODE[x.dtype], ops._stream_ptr(x.device)), "af3_silu_mul")
+        return out.view(*lead, N)
     wt = _cached((weight,), (bool(vnni_repacked), N_BLK, "glu"), lambda: _plain_weight(weight, vnni_repacked, N_BLK).t().contiguous())
     x2 = x.reshape(-1, K)
     if not x2.is_contiguous() or x2.data_ptr() % 16:

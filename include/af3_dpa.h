@@ -285,7 +285,10 @@ int     af3_grid_attention_supported(const af3_grid_attention_params* params);
  * the reference has no native code for this step.
  * pair [n_i, n_j, C] with element strides pair_stride[2] (innermost stride 1, multiples of 8), ln_weight / ln_bias [C],
  * proj_weight [head, C] (nn.Linear weight, contiguous), normed [n_i, n_j, C] contiguous, bias_stride = {head, row i}.
- * Supported: dtype AF3_BF16, C == 128, head == 4, 16-byte aligned pointers; AF3_ERR_BAD_ARGUMENT otherwise.
+ * Supported: dtype AF3_BF16 or AF3_F32 (all tensors of that type), C <= 2048, head <= 64 with (2 + head) * C * 4 bytes
+ * fitting in LDS, pointers aligned to their element size.  bf16 with C == 128, head == 4, 16-byte aligned pointers and
+ * pair strides that are multiples of 8 takes a specialised kernel (four tokens per wave-wide load); everything else one
+ * wavefront per token.  AF3_ERR_BAD_ARGUMENT for shapes beyond these.
  */
 int af3_layernorm_pair_bias(const void* pair, const int64_t* pair_stride, const void* ln_weight, const void* ln_bias, float eps, const void* proj_weight,
 							void* normed, void* bias, const int64_t* bias_stride, int64_t n_i, int64_t n_j, int64_t C, int64_t head, int32_t dtype, void* hip_stream);
@@ -300,6 +303,14 @@ int af3_layernorm_pair_bias(const void* pair, const int64_t* pair_stride, const 
  * Supported: dtype AF3_BF16, K == 64 or 128, N % 32 == 0, 16-byte aligned x and weight_t; AF3_ERR_BAD_ARGUMENT otherwise.
  */
 int af3_gated_linear_unit(const void* x, const void* weight_t, void* out, int64_t M, int64_t K, int64_t N, int32_t dtype, void* hip_stream);
+
+/*
+ * The gate of a gated linear unit on an already computed product: out[m][n] = silu(y[m][n]) * y[m][N + n] for y [M, 2N]
+ * and out [M, N], both contiguous, AF3_BF16 or AF3_F32 (bf16: silu's result is rounded to bf16 before the product, as in
+ * src/csrc/gated_linear_unit.cpp:56-61).  For shapes af3_gated_linear_unit does not take: the caller computes y = x . W
+ * with a library GEMM and applies this.
+ */
+int af3_silu_mul(const void* y, void* out, int64_t M, int64_t N, int32_t dtype, void* hip_stream);
 
 /*
  * Bias-free linear layer for narrow contractions: out[M, N] = x[M, K] . weight^T with weight in nn.Linear layout

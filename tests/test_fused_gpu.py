@@ -378,17 +378,52 @@ def test_layernorm_pair_bias_matches_formula(af3, oracle, n_i, n_j, transposed):
     assert float((bias.float() - ref_b.float()).abs().max()) <= 3e-2 * max(1.0, float(ref_b.float().abs().max()))
 
 
-def test_layernorm_pair_bias_falls_back_to_torch_ops_for_other_shapes(af3, oracle):
-    """Shapes the kernel does not take (64 channels, float32) run the reference's own torch ops on the device."""
-    for C, H, dtype in ((64, 2, torch.bfloat16), (128, 4, torch.float32)):
-        g = torch.Generator().manual_seed(C)
-        x = torch.randn(6, 9, C, generator=g).to(dtype)
-        gamma, beta = torch.ones(C, dtype=dtype), torch.zeros(C, dtype=dtype)
-        wb = (torch.randn(H, C, generator=g) / C ** 0.5).to(dtype)
-        normed, bias = af3.layernorm_pair_bias(x.cuda(), gamma.cuda(), beta.cuda(), 1e-5, wb.cuda())
-        want_n, want_b = oracle.layernorm_pair_bias(f32np(x), f32np(gamma), f32np(beta), f32np(wb), 1e-5)
-        tol = 1e-4 if dtype == torch.float32 else 4e-2
-        assert np.abs(f32np(normed) - want_n).max() <= tol and np.abs(f32np(bias) - want_b).max() <= tol
+@pytest.mark.parametrize("n_i,n_j,C,H,dtype,strided", [
+    (6, 9, 64, 2, torch.bfloat16, False), (5, 37, 256, 8, torch.bfloat16, False), (3, 70, 384, 16, torch.bfloat16, True), (4, 11, 128, 4, torch.float32, False),
+    (2, 65, 96, 3, torch.float32, True), (1, 1, 8, 1, torch.bfloat16, False), (3, 5, 100, 5, torch.bfloat16, False), (2, 3, 768, 16, torch.float32, False),
+    (7, 13, 128, 8, torch.bfloat16, False), (3, 66, 128, 4, torch.bfloat16, "odd_stride"),
+], ids=lambda v: str(v).replace("torch.", ""))
+def test_layernorm_pair_bias_any_channel_and_head_count(af3, oracle, n_i, n_j, C, H, dtype, strided):
+    """Channel and head counts other than the pair tensor's own (128, 4), float32, and bf16 rows the specialised kernel's
+    16-byte loads cannot take: the one-wavefront-per-token kernel against the oracle's fp64 formula, same bars as above
+    (float32: 2e-5 relative on the normalised rows, 1e-4 on the bias)."""
+    g = torch.Generator().manual_seed(C * 10 + H)
+    wide = torch.randn(n_i, n_j, C + (4 if strided == "odd_stride" else 8), generator=g) * 1.5 + 0.3
+    x = wide[..., 2 if strided == "odd_stride" else 0:][..., :C].to(dtype)
+    gamma = (1.0 + 0.2 * torch.randn(C, generator=g)).to(dtype)
+    beta = (0.1 * torch.randn(C, generator=g)).to(dtype)
+    wb = (torch.randn(H, C, generator=g) / C ** 0.5).to(dtype)
+    if strided:
+        dwide = torch.empty(n_i, n_j, wide.shape[-1], dtype=dtype, device="cuda")
+        dx = dwide[..., 2 if strided == "odd_stride" else 0:][..., :C]
+        dx.copy_(x)
+        assert not dx.is_contiguous()
+    else:
+        dx = x.cuda()
+    print(f"layernorm_pair_bias any {n_i}x{n_j}x{C} heads={H} {dtype} strided={strided}", flush=True)
+    normed, bias = af3.layernorm_pair_bias(dx, gamma.cuda(), beta.cuda(), 1e-5, wb.cuda())
+    torch.cuda.synchronize()
+    assert normed.shape == x.shape and bias.shape == (H, n_i, n_j) and normed.dtype == bias.dtype == dtype
+    want_n, want_b = oracle.layernorm_pair_bias(f32np(x), f32np(gamma), f32np(beta), f32np(wb), 1e-5)
+    got_n = f32np(normed)
+    assert np.isfinite(got_n).all() and np.isfinite(f32np(bias)).all()
+    if dtype == torch.float32:
+        assert (np.abs(got_n - want_n) <= np.maximum(np.abs(want_n), 1.0) * 2e-5).all()
+        assert np.abs(f32np(bias) - want_b).max() <= 1e-4 * max(1.0, np.abs(want_b).max())
+    else:
+        assert (np.abs(got_n - want_n) <= np.maximum(np.abs(want_n), 1e-2) * 2.0 ** -8 + 1e-6).all()
+        want_b = np.einsum("ijc,hc->hij", got_n.astype(np.float64), f32np(wb).astype(np.float64))      # the projection of the rows as stored
+        assert np.abs(f32np(bias) - want_b).max() <= 2e-2 * max(1.0, np.abs(want_b).max())
+
+
+def test_layernorm_pair_bias_rejects_what_it_cannot_take(af3):
+    x = torch.randn(3, 4, 16, device="cuda")
+    with pytest.raises(ValueError):
+        af3.layernorm_pair_bias(x.half(), torch.ones(16, device="cuda").half(), torch.zeros(16, device="cuda").half(), 1e-5, torch.ones(2, 16, device="cuda").half())
+    with pytest.raises(ValueError):
+        af3.layernorm_pair_bias(x, torch.ones(8, device="cuda"), torch.zeros(16, device="cuda"), 1e-5, torch.ones(2, 16, device="cuda"))
+    with pytest.raises(ValueError):
+        af3.layernorm_pair_bias(torch.randn(2, 2, 4096, device="cuda"), torch.ones(4096, device="cuda"), torch.zeros(4096, device="cuda"), 1e-5, torch.ones(2, 4096, device="cuda"))
 
 
 @pytest.mark.parametrize("lead,K,N,repacked", [((37, 37), 128, 256, False), ((200,), 128, 512, True), ((3, 50), 64, 512, False), ((65,), 128, 1024, True),
@@ -414,14 +449,20 @@ def test_gated_linear_unit_matches_formula(af3, oracle, lead, K, N, repacked):
 
 
 def test_gated_linear_unit_other_shapes_and_linear_module(af3, oracle):
-    """Shapes outside the kernel's (float32, K = 48) run the formula's torch ops on the device; the Linear module is x @ W^T."""
+    """Shapes outside the one-kernel form's (float32; K = 48, 384, 768; N not a multiple of 32; a repacked weight at K = 384)
+    are a library GEMM plus the silu-and-multiply kernel; the Linear module is x @ W^T."""
     g = torch.Generator().manual_seed(9)
-    for K, N, dtype, tol in ((48, 40, torch.bfloat16, 3e-2), (128, 64, torch.float32, 1e-4)):
+    for K, N, dtype, tol, repacked in ((48, 40, torch.bfloat16, 3e-2, False), (128, 64, torch.float32, 1e-4, False), (384, 1536, torch.bfloat16, 3e-2, True),
+                                       (768, 100, torch.bfloat16, 3e-2, False), (64, 7, torch.float32, 1e-4, False)):
         x = torch.randn(7, 11, K, generator=g).to(dtype)
         w = (torch.randn(K, 2 * N, generator=g) / K ** 0.5).to(dtype)
-        out = af3.gated_linear_unit_cpp(x.cuda(), w.cuda())
+        dw = af3.vnni_repack_tensor(w.cuda(), 2, 128) if repacked else w.cuda()
+        out = af3.gated_linear_unit_cpp(x.cuda(), dw, repacked, 128, 128)
+        assert out.shape == (7, 11, N) and out.dtype == dtype
         want = oracle.gated_linear_unit(f32np(x), f32np(w))
         assert np.abs(f32np(out) - want).max() <= tol * max(1.0, float(np.abs(want).max()))
+    with pytest.raises(ValueError):
+        af3.gated_linear_unit_cpp(torch.randn(4, 64, device="cuda").half(), torch.randn(64, 64, device="cuda").half())
     for n_out in (128, 64):                                                # narrow layers run af3_linear, bit-identical to the library GEMM here
         g2 = torch.Generator().manual_seed(n_out)
         lin = af3.Linear(128, n_out, False, dtype=torch.bfloat16).cuda()

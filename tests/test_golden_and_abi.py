@@ -286,7 +286,7 @@ def test_weight_unpacking_inverts_the_panel_layout(oracle):
 
 
 def test_row_op_entry_points_validate_on_the_host():
-    """af3_gated_linear_unit, af3_linear and af3_layernorm_pair_bias refuse malformed calls with a status code, before any launch."""
+    """af3_gated_linear_unit, af3_linear, af3_silu_mul and af3_layernorm_pair_bias refuse malformed calls with a status code, before any launch."""
     from af3_kernels_amd import _lib
     lib = _lib.load()
     P, BF, F32 = 0x1000, _lib.AF3_BF16, _lib.AF3_F32
@@ -301,12 +301,16 @@ def test_row_op_entry_points_validate_on_the_host():
     ps, bs = (ctypes.c_int64 * 2)(9 * 128, 128), (ctypes.c_int64 * 2)(6 * 9, 9)
     assert ln(None, ps, P, P, 1e-5, P, P, P, bs, 6, 9, 128, 4, BF, None) == -1
     assert ln(P, ps, P, P, 1e-5, P, P, P, bs, 0, 9, 128, 4, BF, None) == -3
-    assert ln(P, ps, P, P, 1e-5, P, P, P, bs, 6, 9, 128, 4, F32, None) == -2
-    assert ln(P, ps, P, P, 1e-5, P, P, P, bs, 6, 9, 64, 4, BF, None) == -7      # 128 channels, 4 heads
-    assert ln(P, ps, P, P, 1e-5, P, P, P, bs, 6, 9, 128, 8, BF, None) == -7
+    assert ln(P, ps, P, P, 1e-5, P, P, P, bs, 6, 9, 128, 4, _lib.AF3_FP8_E4M3, None) == -2   # bfloat16 or float32
+    assert ln(P, ps, P, P, 1e-5, P, P, P, bs, 6, 9, 0, 4, BF, None) == -3
+    assert ln(P, (ctypes.c_int64 * 2)(9 * 4096, 4096), P, P, 1e-5, P, P, P, bs, 6, 9, 4096, 4, BF, None) == -7   # at most 2048 channels
+    assert ln(P, (ctypes.c_int64 * 2)(9 * 1024, 1024), P, P, 1e-5, P, P, P, bs, 6, 9, 1024, 64, BF, None) == -7  # gamma, beta and the weights must fit in LDS
+    assert ln(P + 1, ps, P, P, 1e-5, P, P, P, bs, 6, 9, 128, 4, BF, None) == -7                                     # not aligned to the element size
     assert ln(P, (ctypes.c_int64 * 2)(9 * 128, 64), P, P, 1e-5, P, P, P, bs, 6, 9, 128, 4, BF, None) == -4   # tokens overlap
     assert ln(P, ps, P, P, 1e-5, P, P, P, (ctypes.c_int64 * 2)(6 * 9, 4), 6, 9, 128, 4, BF, None) == -4        # bias rows overlap
     assert ln(P, ps, P, P, -1.0, P, P, P, bs, 6, 9, 128, 4, BF, None) == -7
+    sm = lib.af3_silu_mul
+    assert sm(None, P, 4, 8, BF, None) == -1 and sm(P, P, 0, 8, BF, None) == -3 and sm(P, P, 4, 8, _lib.AF3_FP8_E4M3, None) == -2
 
 
 def test_derived_weight_cache_follows_tensor_identity_and_version():

@@ -58,3 +58,22 @@ def test_static_scratch_entry_point_matches_the_workspace_entry_point_on_two_cal
     got, _ = _call(lib.af3_dpa_forward_static_scratch, q, k, v, mask, bias, None)
     torch.cuda.synchronize()
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # Under stream capture the entry point must only enqueue kernels: its host-side set-up (address of the scratch array, device
+    # properties, kernel attributes) happened in the eager calls above, which is the documented order -- one call outside
+    # capture first.  Replays are checked against the eager result with eager work and synchronisations in between.
+    q, k, v, mask, bias = _inputs(3, 4, 204, 32, 6)
+    tmp = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    p = ops._fill_params(q, k, v, ops._lift_mask(mask, 204), bias, tmp, _lib.AF3_BF16, False)
+    ws = torch.empty(lib.af3_dpa_workspace_bytes(ctypes.byref(p)), dtype=torch.uint8, device=q.device)
+    want, _ = _call(lib.af3_dpa_forward, q, k, v, mask, bias, ws)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got, _ = _call(lib.af3_dpa_forward_static_scratch, q, k, v, mask, bias, None)
+    for i in range(3):
+        got.fill_(float("nan"))
+        other, _ = _call(lib.af3_dpa_forward_static_scratch, *_inputs(18, 4, 412, 32, 5), None)    # eager work that overwrites the scratch array
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"replay {i}"

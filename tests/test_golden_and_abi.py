@@ -456,3 +456,23 @@ def test_argument_blocks_and_weight_cache_can_be_built_from_several_threads():
         t.join()
     assert not errors, errors[:3]
     assert len(ops._PARAM_TEMPLATES) <= 256 and len(fused._W_CACHE) <= fused._W_CACHE_MAX
+
+
+def test_traffic_digest_follows_the_code_and_not_its_commentary():
+    """bench.py reports roofline.traffic from a committed counter summary only while the kernel sources' code has the digest the
+    counters were collected with.  The digest ignores comments and whitespace (no hand re-stamping after an edit of the
+    commentary), changes with any other edit, keeps string literals intact -- and every committed summary matches the
+    sources as they are, so that a kernel change without fresh counters shows up here and not as a silent null."""
+    import sys
+    sys.path.insert(0, ROOT)
+    import bench
+    a = 'int x = 1; // one\n/* block\n comment */ asm volatile("s_nop 0 // kept\\n\\t" ::: "memory");  char c = \'"\';\n'
+    b = 'int x=1;asm volatile("s_nop 0 // kept\\n\\t":::"memory");\n\n   char c=\'"\'; // trailing words\n'
+    assert bench._code_only(a) == bench._code_only(b)
+    assert bench._code_only(a) != bench._code_only(a.replace("x = 1", "x = 2"))
+    assert bench._code_only(a) != bench._code_only(a.replace("// kept", "// changed"))     # inside a string literal: code
+    digest = bench.kernel_sources_digest()
+    for name, fname in bench.TRAFFIC_PROFILES.items():
+        text = open(os.path.join(ROOT, "profiles", fname)).read()
+        assert "kernel_code_sha256: " + digest in text, f"profiles/{fname} was collected with other kernel code: re-collect the counters"
+        assert bench.measured_traffic_bytes(name) > 0

@@ -181,7 +181,7 @@ __global__ void __launch_bounds__(F32_NW * 64) dpa_mfma_f32_kernel(af3_dpa_param
 		f32x16       s;
 		const float* krow = k_lds + buf * TILE_FLOATS + n * RS + half * NK;
 #pragma unroll
-		for(int i = 0; i < 16; i++) s[i] = bcur[i];  // the accumulator starts from the bias
+		for(int i = 0; i < 16; i++) s[i] = 0.f;
 #pragma unroll
 		for(int t4 = 0; t4 < NK / 4; t4++) {
 			const float4 w = *reinterpret_cast<const float4*>(krow + 4 * t4);
@@ -190,6 +190,10 @@ __global__ void __launch_bounds__(F32_NW * 64) dpa_mfma_f32_kernel(af3_dpa_param
 			s = __builtin_amdgcn_mfma_f32_32x32x2f32(w.z, qreg[4 * t4 + 2], s, 0, 0, 0);
 			s = __builtin_amdgcn_mfma_f32_32x32x2f32(w.w, qreg[4 * t4 + 3], s, 0, 0, 0);
 		}
+		// The bias joins the finished products in one rounding, as an addition of two fp32 tensors would: products accumulated on
+		// top of a bias of magnitude 10^3..10^4 (a row offset, a soft mask value) would be rounded at that magnitude D/2 times.
+#pragma unroll
+		for(int i = 0; i < 16; i++) s[i] += bcur[i];
 		// key states of this lane's 16 keys: dropped -> -1e9 (as masked_fill does), past L -> -inf
 		float mx = -INFINITY;
 #pragma unroll

@@ -352,6 +352,18 @@ def test_fp32_mfma_strided_inputs_and_large_logits(af3, oracle):
     assert np.abs(f32np(out) - want).max() <= 1e-4
 
 
+def test_fp32_mfma_bias_rows_with_a_large_offset(af3, oracle):
+    """Query rows whose biases all carry an offset of -1000 (a soft mask value): the softmax of such a row is that of the
+    row without the offset, up to the rounding of one fp32 addition per logit (half an ulp of 1000: 3e-5).  Products
+    accumulated on top of the bias would be rounded at that magnitude once per matrix instruction (3e-4 measured)."""
+    B, H, L, D = 3, 2, 200, 32
+    q, k, v, m, bias = rand_inputs(B, H, L, D, torch.float32, seed=43, mask="random")
+    g = torch.Generator().manual_seed(44)
+    bias = bias * 2
+    bias[:, torch.rand(L, generator=g) < 0.3, :] -= 1000.0
+    run_case(af3, oracle, q, k, v, m, bias, tol=1e-4, expect_kernel="fp32_mfma")
+
+
 def test_fp32_bias_and_other_dtypes_are_cast_like_the_reference(af3, oracle):
     q, k, v, m, bias = rand_inputs(2, 4, 64, 32, torch.bfloat16, seed=12, mask="tail")
     out = af3.dot_product_attention_cpp(q.cuda(), k.float().cuda(), v.float().cuda(), m.float().cuda(), bias.float().cuda())

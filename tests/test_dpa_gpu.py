@@ -309,6 +309,98 @@ def test_bf16_seeded_shape_sweep(af3, oracle, B, H, L, D, mask, rank, seed):
     run_case(af3, oracle, q, k, v, m, bias, expect_kernel="bf16_mfma")
 
 
+def _pattern_case(rng, idx):
+    """One seeded case of the sweep below: shape, storage type, memory layout of q/k/v, bias pattern, mask form and
+    pattern, kernel hint.  CPU tensors (views keep their strides when moved to the GPU)."""
+    dtype = torch.bfloat16 if rng.random() < 0.75 else torch.float32
+    D = rng.choice([8, 16, 24, 32, 32, 48, 64, 20, 40])
+    L = rng.choice([1, 2, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 200, 255, 257, rng.randint(1, 300)])
+    B = rng.choice([1, 1, 2, 3, 4, 5, 7, 9, 13, 17])
+    H = rng.choice([1, 2, 4, 8])
+    while B * H * L * L > 1_500_000 and B > 1:
+        B //= 2
+    layout = rng.choice(["bhld", "blhd", "packed"])
+    g = torch.Generator().manual_seed(5000 + idx)
+
+    def qkv():
+        if layout == "bhld":
+            return torch.randn(B, H, L, D, generator=g).to(dtype)
+        if layout == "blhd":                                      # [B, L, H, D] storage seen as [B, H, L, D]
+            return torch.randn(B, L, H, D, generator=g).to(dtype).permute(0, 2, 1, 3)
+        return torch.randn(B, L, H, 3 * D, generator=g).to(dtype).permute(0, 2, 1, 3)[..., D:2 * D]   # a slice of a packed q|k|v projection
+
+    q, k, v = qkv(), qkv(), qkv()
+    bias_kind = rng.choice(["plain", "plain", "padded", "wide", "dropped_pairs", "shifted"])
+    M = L + rng.choice([1, 3, 8, 29]) if bias_kind == "padded" else L
+    bias = torch.randn(H, M, M, generator=g) * (5.0 if bias_kind == "wide" else 1.5)
+    if bias_kind == "dropped_pairs":                              # a mask folded into the bias, at three usual magnitudes
+        bias[torch.rand(bias.shape, generator=g) < 0.15] = -rng.choice([1e4, 3e4, 1e8])
+    if bias_kind == "shifted":
+        bias += 5.0
+    bias = bias.to(dtype)
+    mask_kind = rng.choice(["all", "bernoulli", "bernoulli", "tail", "leading_dropped", "rows_without_keys", "one_key", "1d"])
+    mask = torch.ones(B, L, dtype=torch.bool)
+    if mask_kind == "bernoulli":
+        mask = torch.rand(B, L, generator=g) < rng.choice([0.05, 0.5, 0.9])
+    elif mask_kind == "tail":
+        for b in range(B):
+            mask[b, rng.randint(0, L):] = False
+    elif mask_kind == "leading_dropped":
+        mask = torch.rand(B, L, generator=g) < 0.7
+        for b in range(B):
+            mask[b, :rng.randint(0, L)] = False
+    elif mask_kind == "rows_without_keys":
+        mask = torch.rand(B, L, generator=g) < 0.8
+        for b in range(B):
+            if rng.random() < 0.4:
+                mask[b] = False
+    elif mask_kind == "one_key":
+        mask = torch.zeros(B, L, dtype=torch.bool)
+        for b in range(B):
+            mask[b, rng.randint(0, L - 1)] = True
+    elif mask_kind == "1d":
+        mask = torch.rand(L, generator=g) < 0.8
+    mask_form = rng.choice(["bool", "typed", "b11l"])
+    rows = rng.choice(["auto", "auto", "always", "never"])
+    desc = f"pattern case {idx}: {dtype} B={B} H={H} L={L} D={D} layout={layout} bias={bias_kind} mask={mask_kind}/{mask_form} rows={rows}"
+    return desc, q, k, v, mask, mask_form, bias, rows
+
+
+@pytest.mark.parametrize("chunk", range(5))
+def test_seeded_sweep_of_layouts_masks_and_bias_patterns(af3, oracle, chunk):
+    """What the shape sweeps above hold fixed: q/k/v as strided views of [B, L, H, D] and packed-projection storage, the
+    mask as bool / typed / [B,1,1,L] / 1-D with leading dropped tiles, rows without keys and single live keys, biases
+    that are pre-padded, wide (sigma 5), shifted, or carry a folded-in mask of -1e4 / -3e4 / -1e8 at scattered pairs;
+    every kernel hint.  Each case against the fp64 formula of the oracle at the storage type's tolerance."""
+    import random
+    rng = random.Random(9000 + chunk)
+    for i in range(30):
+        idx = 100 * chunk + i
+        desc, q, k, v, mask, mask_form, bias, rows = _pattern_case(rng, idx)
+        print(desc, flush=True)
+        dm = mask.cuda()
+        if mask_form == "typed":
+            dm = dm.to(q.dtype)
+        elif mask_form == "b11l" and mask.dim() == 2:
+            dm = dm[:, None, None, :]
+        prev = af3.set_rows_kernel(rows)
+        try:
+            out = af3.dot_product_attention_cpp(q.cuda(), k.cuda(), v.cuda(), dm, bias.cuda())
+            torch.cuda.synchronize()
+        finally:
+            af3.set_rows_kernel(prev)
+        L = q.shape[2]
+        want = oracle.dpa_formula(f32np(q), f32np(k), f32np(v), mask.numpy(), f32np(bias[:, :L, :L]))
+        got = f32np(out)
+        assert np.isfinite(got).all(), desc
+        # Query rows all of whose live keys sit on folded-in mask values are only required to be finite: their logits are
+        # -1e4 .. -1e8 plus the products, which no fp32 addition resolves to the tolerance (nor does the reference's).
+        live = (mask if mask.dim() == 2 else mask[None, :]).numpy()[:, None, None, :]
+        usable = (live & (f32np(bias[:, :L, :L]) > -1e3)[None]).any(-1) | ~live.any(-1)       # [B, H, L]
+        err = float(np.abs(got - want)[np.broadcast_to(usable, got.shape[:3])].max()) if usable.any() else 0.0
+        assert err <= TOL[q.dtype], f"{desc}: max abs err {err}"
+
+
 @pytest.mark.parametrize("B,H,L,D,mask,kernel", [
     (1, 2, 700, 40, "random", "fp32_mfma"),     # head_dim 40: padded to 64 columns
     (2, 3, 37, 20, "tail", "fp32_mfma"),        # odd length, head_dim 20
